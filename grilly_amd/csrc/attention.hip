@@ -1,0 +1,427 @@
+// Flash-Attention-2 forward for gfx950, layout (B,S,H,D), optional key-padding mask,
+// causal exclusion and fused interleaved RoPE.
+//
+// A workgroup (4 waves) owns 128 queries of one (batch, head); each wave owns 32 of them and
+// keeps, per lane, ONE query: the kernel computes the transposed products
+//     S^T = K . Q^T   (keys x queries)      and      O^T = V^T . P^T   (head-dim x queries)
+// on 32x32 MFMA tiles, so every accumulator register of a lane belongs to that lane's query.
+// The online-softmax state (running max m, running sum l) and the rescale factor are then
+// per-lane scalars; the only cross-lane step is one exchange with lane^32 for the row max.
+//
+//   HBM --128-bit loads--> VGPR --(RoPE on K) --> LDS: K tile [key][d], XOR-swizzled chunks
+//                                              --> LDS: V tile, fp32 [key][d]; bf16 transposed
+//                                                  to [d][key] in 4-key groups so that the MFMA
+//                                                  operand is two 8-byte reads
+//   K/V tiles are double buffered; the next tile's loads are in flight during the MFMAs.
+//   S, P and O never leave registers; P is rounded to bf16 only as MFMA operand (bf16 path).
+//
+// Semantics (constants of shaders/flash-attention2.glsl:95,152,214):
+//   score = <q,k>*scale + (mask[b,k]-1)*1e9 ; running max starts at -1e10 ;
+//   out = acc / max(sum, 1e-10) ; causal keys (k > q) and keys >= S are excluded outright.
+#include "common.hpp"
+#include <type_traits>
+
+int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling);
+
+struct FaArgs {
+    const void* Q; const void* K; const void* V;
+    const float* mask;        // (B,S) or null
+    void* O;
+    const float2* rope;       // (S, D/2) {cos, sin} or null
+    int B, S, H;
+    float scale;
+    int causal;
+    int64_t q_stride, k_stride, v_stride, o_stride;   // elements between consecutive positions
+};
+
+template <int N, typename F> __device__ __forceinline__ void sfor(F&& f) {
+    if constexpr (N > 0) {
+        sfor<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+template <typename T> struct Slab;
+template <> struct Slab<uint16_t> {
+    static __device__ __forceinline__ void run(const u32x4& a, const u32x4& b, f32x16& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+    }
+};
+template <> struct Slab<float> {
+    static __device__ __forceinline__ void run(const u32x4& a, const u32x4& b, f32x16& acc) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a[e]), __builtin_bit_cast(float, b[e]), acc, 0, 0, 0);
+    }
+};
+
+// rotate the pairs held in one 16-byte chunk; cs[i] = {cos, sin} of pair i
+template <typename T> __device__ __forceinline__ u32x4 rope_chunk(u32x4 v, const float2* cs);
+template <> __device__ __forceinline__ u32x4 rope_chunk<float>(u32x4 v, const float2* cs) {
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        float x0 = __builtin_bit_cast(float, v[2 * i]), x1 = __builtin_bit_cast(float, v[2 * i + 1]);
+        o[2 * i] = __builtin_bit_cast(uint32_t, x0 * cs[i].x - x1 * cs[i].y);
+        o[2 * i + 1] = __builtin_bit_cast(uint32_t, x0 * cs[i].y + x1 * cs[i].x);
+    }
+    return o;
+}
+template <> __device__ __forceinline__ u32x4 rope_chunk<uint16_t>(u32x4 v, const float2* cs) {
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float x0 = bf16lo(v[i]), x1 = bf16hi(v[i]);
+        o[i] = pack_bf16x2(x0 * cs[i].x - x1 * cs[i].y, x0 * cs[i].y + x1 * cs[i].x);
+    }
+    return o;
+}
+
+template <typename OutT> __device__ __forceinline__ void fa_store4(OutT* p, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void fa_store4<float>(float* p, float a, float b, float c, float d) {
+    f32x4 v = {a, b, c, d};
+    *(f32x4*)p = v;
+}
+template <> __device__ __forceinline__ void fa_store4<uint16_t>(uint16_t* p, float a, float b, float c, float d) {
+    u32x2 v = {pack_bf16x2(a, b), pack_bf16x2(c, d)};
+    *(u32x2*)p = v;
+}
+
+template <typename T, int D, bool ROPE>
+__global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
+    constexpr bool BF = sizeof(T) == 2;
+    constexpr int ES = (int)sizeof(T), RB = D * ES, NCH = RB / 16, NS = RB / 32, EPC = 16 / ES;
+    constexpr int KT = (BF && D <= 64) ? 128 : 64;      // keys per tile
+    constexpr int NKB = KT / 32, DT = D / 32;
+    constexpr int CK = KT * NCH / 256;                  // K chunks per thread
+    constexpr int NU = BF ? (KT / 4) * (D / 8) : 0;     // bf16 V transposition units (4 keys x 8 dims)
+    constexpr int CV = BF ? 4 : CK;
+    constexpr int TILE = KT * RB;
+    constexpr int PPC = EPC / 2;                        // RoPE pairs per chunk
+    static_assert(KT * NCH % 256 == 0 && NU <= 256, "tile does not divide over 256 threads");
+    __shared__ __attribute__((aligned(16))) char ldsK[2][TILE];
+    __shared__ __attribute__((aligned(16))) char ldsV[2][TILE];
+    __shared__ __attribute__((aligned(16))) float ldsBias[2][KT];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 31, lg = lane >> 5;
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int qb = p.causal ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;   // heavy blocks first
+    const int q0 = qb * 128;
+    const int S = p.S;
+    const int qi = q0 + wave * 32 + li;
+    const int qc = qi < S ? qi : S - 1;
+    const T* Qg = (const T*)p.Q + (int64_t)b * S * p.q_stride + h * D;
+    const T* Kg = (const T*)p.K + (int64_t)b * S * p.k_stride + h * D;
+    const T* Vg = (const T*)p.V + (int64_t)b * S * p.v_stride + h * D;
+
+    // ---- this lane's query, as MFMA "B" operand: slab s holds dims (2s+lg)*EPC .. +EPC-1
+    u32x4 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int c = 2 * s + lg;
+        u32x4 v = *(const u32x4*)(Qg + (int64_t)qc * p.q_stride + c * EPC);
+        if (ROPE) {
+            float2 cs[PPC];
+#pragma unroll
+            for (int i = 0; i < PPC; ++i) cs[i] = p.rope[(int64_t)qc * (D / 2) + c * PPC + i];
+            v = rope_chunk<T>(v, cs);
+        }
+        qf[s] = v;
+    }
+
+    int nkt = (S + KT - 1) / KT;
+    if (p.causal) {
+        int last = (q0 + 127 < S - 1 ? q0 + 127 : S - 1) / KT + 1;
+        nkt = nkt < last ? nkt : last;
+    }
+
+    // ---- staging registers and their loaders
+    u32x4 kreg[CK], vreg[CV];
+    float2 kcs[ROPE ? CK : 1][PPC];
+    float breg = 0.f;
+    auto load_tile = [&](int kt) {
+        const int k0 = kt * KT;
+#pragma unroll
+        for (int i = 0; i < CK; ++i) {
+            const int q = tid + i * 256, key = q / NCH, c = q % NCH;
+            const int kk = k0 + key, kc = kk < S ? kk : S - 1;
+            kreg[i] = *(const u32x4*)(Kg + (int64_t)kc * p.k_stride + c * EPC);
+            if (ROPE) {
+#pragma unroll
+                for (int j = 0; j < PPC; ++j) kcs[i][j] = p.rope[(int64_t)kc * (D / 2) + c * PPC + j];
+            }
+        }
+        if (BF) {
+            if (tid < NU) {
+                const int dc = tid % (D / 8), kg = tid / (D / 8);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int kk = k0 + 4 * kg + j, kc = kk < S ? kk : S - 1;
+                    vreg[j] = *(const u32x4*)(Vg + (int64_t)kc * p.v_stride + dc * 8);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < CV; ++i) {
+                const int q = tid + i * 256, key = q / NCH, c = q % NCH;
+                const int kk = k0 + key, kc = kk < S ? kk : S - 1;
+                vreg[i] = *(const u32x4*)(Vg + (int64_t)kc * p.v_stride + c * EPC);
+            }
+        }
+        if (tid < KT) {
+            const int kk = k0 + tid;
+            breg = 0.f;
+            if (p.mask && kk < S) breg = (p.mask[(int64_t)b * S + kk] - 1.0f) * 1e9f;
+            if (kk >= S) breg = -__builtin_inff();
+        }
+    };
+    auto stash_tile = [&](int kt) {
+        const int st = kt & 1, k0 = kt * KT;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        char* Kb = ldsK[st];
+        char* Vb = ldsV[st];
+#pragma unroll
+        for (int i = 0; i < CK; ++i) {
+            const int q = tid + i * 256, key = q / NCH, c = q % NCH;
+            u32x4 v = kreg[i];
+            if (ROPE) v = rope_chunk<T>(v, kcs[i]);
+            if (k0 + key >= S) v = zero;
+            const int slot = NCH >= 8 ? (c ^ (key & 7)) : (c ^ ((key >> 1) & 3));
+            *(u32x4*)(Kb + key * RB + slot * 16) = v;
+        }
+        if (BF) {
+            if (tid < NU) {
+                const int dc = tid % (D / 8), kg = tid / (D / 8);
+                u32x4 r[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) r[j] = (k0 + 4 * kg + j >= S) ? zero : vreg[j];
+#pragma unroll
+                for (int dd = 0; dd < 8; ++dd) {
+                    const int w = dd >> 1;
+                    uint32_t e0, e1, e2, e3;
+                    if (dd & 1) { e0 = r[0][w] >> 16; e1 = r[1][w] & 0xffff0000u; e2 = r[2][w] >> 16; e3 = r[3][w] & 0xffff0000u; }
+                    else { e0 = r[0][w] & 0xffffu; e1 = r[1][w] << 16; e2 = r[2][w] & 0xffffu; e3 = r[3][w] << 16; }
+                    const int d = dc * 8 + dd;
+                    const int slot = (kg + d + (d >> 4)) & (KT / 4 - 1);
+                    u32x2 o = {e0 | e1, e2 | e3};
+                    *(u32x2*)(Vb + d * (KT * 2) + slot * 8) = o;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < CV; ++i) {
+                const int q = tid + i * 256, key = q / NCH, c = q % NCH;
+                *(u32x4*)(Vb + key * RB + c * 16) = (k0 + key >= S) ? zero : vreg[i];
+            }
+        }
+        if (tid < KT) ldsBias[st][tid] = breg;
+    };
+
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[t][r] = 0.f;
+    float m_run = -1e10f, l_run = 0.f;
+
+    load_tile(0);
+    stash_tile(0);
+    __syncthreads();
+    for (int kt = 0; kt < nkt; ++kt) {
+        const bool more = kt + 1 < nkt;
+        if (more) load_tile(kt + 1);
+        const int st = kt & 1, k0 = kt * KT;
+        const char* Kb = ldsK[st];
+        const char* Vb = ldsV[st];
+
+        // ---- S^T = K . Q^T for the tile's NKB blocks of 32 keys
+        f32x16 sacc[NKB];
+        sfor<NKB>([&](auto it) {
+            constexpr int t = decltype(it)::value;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[t][r] = 0.f;
+            const int key = 32 * t + li;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const int c = 2 * s + lg;
+                const int slot = NCH >= 8 ? (c ^ (key & 7)) : (c ^ ((key >> 1) & 3));
+                u32x4 kf = *(const u32x4*)(Kb + key * RB + slot * 16);
+                Slab<T>::run(kf, qf[s], sacc[t]);
+            }
+        });
+
+        // ---- scores, running max
+        const bool diag = p.causal && (k0 + KT - 1 > q0 + wave * 32);
+        float mx = -__builtin_inff();
+        sfor<NKB>([&](auto it) {
+            constexpr int t = decltype(it)::value;
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int kl = 32 * t + 8 * qd + 4 * lg;          // first of 4 consecutive keys
+                f32x4 bias = *(const f32x4*)(&ldsBias[st][kl]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float s = sacc[t][4 * qd + e] * p.scale + bias[e];
+                    if (diag && (k0 + kl + e > qi)) s = -__builtin_inff();
+                    sacc[t][4 * qd + e] = s;
+                    mx = fmaxf(mx, s);
+                }
+            }
+        });
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = __expf(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.f;
+        sfor<NKB>([&](auto it) {
+            constexpr int t = decltype(it)::value;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float pv = __expf(sacc[t][r] - m_new);
+                sacc[t][r] = pv;
+                psum += pv;
+            }
+        });
+        l_run = l_run * alpha + psum;
+        sfor<DT>([&](auto idt) {
+            constexpr int dt = decltype(idt)::value;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        });
+
+        // ---- O^T += V^T . P^T
+        if (BF) {
+            sfor<NKB>([&](auto it) {
+                constexpr int t = decltype(it)::value;
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh) {
+                    u32x4 pf;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) pf[e] = pack_bf16x2(sacc[t][8 * hh + 2 * e], sacc[t][8 * hh + 2 * e + 1]);
+                    const int kgA = 8 * t + 4 * hh + lg;
+                    sfor<DT>([&](auto idt) {
+                        constexpr int dt = decltype(idt)::value;
+                        const int d = 32 * dt + li, f = d + (d >> 4);
+                        u32x2 va = *(const u32x2*)(Vb + d * (KT * 2) + ((kgA + f) & (KT / 4 - 1)) * 8);
+                        u32x2 vb = *(const u32x2*)(Vb + d * (KT * 2) + ((kgA + 2 + f) & (KT / 4 - 1)) * 8);
+                        u32x4 vf = {va[0], va[1], vb[0], vb[1]};
+                        Slab<uint16_t>::run(vf, pf, oacc[dt]);
+                    });
+                }
+            });
+        } else {
+            sfor<NKB>([&](auto it) {
+                constexpr int t = decltype(it)::value;
+                sfor<16>([&](auto ir) {
+                    constexpr int r = decltype(ir)::value;
+                    const int kl = 32 * t + 8 * (r / 4) + 4 * lg + (r % 4);
+                    sfor<DT>([&](auto idt) {
+                        constexpr int dt = decltype(idt)::value;
+                        float vv = *(const float*)(Vb + kl * RB + (32 * dt + li) * 4);
+                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, sacc[t][r], oacc[dt], 0, 0, 0);
+                    });
+                });
+            });
+        }
+
+        if (more) stash_tile(kt + 1);
+        __syncthreads();
+    }
+
+    // ---- normalise and store: lane holds, for its query, dims 32dt + 8qd + 4lg + {0..3}
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / fmaxf(l_tot, 1e-10f);
+    if (qi < S) {
+        T* Og = (T*)p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
+        sfor<DT>([&](auto idt) {
+            constexpr int dt = decltype(idt)::value;
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int d = 32 * dt + 8 * qd + 4 * lg;
+                fa_store4<T>(Og + d, oacc[dt][4 * qd] * inv, oacc[dt][4 * qd + 1] * inv, oacc[dt][4 * qd + 2] * inv, oacc[dt][4 * qd + 3] * inv);
+            }
+        });
+    }
+}
+
+template <typename T, int D>
+static int launch_fa(grl_ctx* c, FaArgs& a, bool rope) {
+    dim3 grid((unsigned)((a.S + 127) / 128), (unsigned)a.H, (unsigned)a.B), block(256);
+    if (rope) hipLaunchKernelGGL((fa2_fwd_kernel<T, D, true>), grid, block, 0, c->stream, a);
+    else hipLaunchKernelGGL((fa2_fwd_kernel<T, D, false>), grid, block, 0, c->stream, a);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                      const void* Q, const void* K, const void* V, const float* mask, void* O,
+                      int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                      float scale, int causal, int rope, float rope_base, float rope_scaling, void* workspace) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "%s: null context", who);
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "%s: bad dtype %d", who, dtype);
+    GRL_REQUIRE(rope >= GRL_ROPE_NONE && rope <= GRL_ROPE_HALF, GRL_ERR_ARG, "%s: bad rope style %d", who, rope);
+    GRL_REQUIRE(B >= 0 && S >= 0 && H >= 0, GRL_ERR_SHAPE, "%s: negative dimension", who);
+    GRL_REQUIRE(D == 32 || D == 64 || D == 128, GRL_ERR_SHAPE, "%s: head_dim must be 32, 64 or 128 (got %lld)", who, (long long)D);
+    GRL_REQUIRE(B < 65536 && H < 65536 && S < (1LL << 24), GRL_ERR_SHAPE, "%s: B,H must be < 65536 and S < 2^24", who);
+    if (B == 0 || S == 0 || H == 0) return GRL_OK;
+    GRL_REQUIRE(Q && K && V && O, GRL_ERR_ARG, "%s: null argument", who);
+    const int64_t es = (int64_t)grl_dtype_size(dtype), hd = H * D;
+    GRL_REQUIRE(q_stride >= hd && k_stride >= hd && v_stride >= hd && o_stride >= hd, GRL_ERR_SHAPE,
+                "%s: position stride smaller than num_heads*head_dim", who);
+    GRL_REQUIRE(((((uintptr_t)Q) | ((uintptr_t)K) | ((uintptr_t)V) | ((uintptr_t)O)) & 15u) == 0 &&
+                ((q_stride | k_stride | v_stride | o_stride) * es) % 16 == 0, GRL_ERR_ARG,
+                "%s: Q,K,V,O and their position strides must be 16-byte aligned", who);
+    if (rope != GRL_ROPE_NONE) GRL_REQUIRE(rope_base > 0.f && rope_scaling != 0.f, GRL_ERR_ARG, "%s: bad rope base/scaling", who);
+
+    FaArgs a{};
+    a.Q = Q; a.K = K; a.V = V; a.mask = mask; a.O = O;
+    a.B = (int)B; a.S = (int)S; a.H = (int)H; a.scale = scale; a.causal = causal ? 1 : 0;
+    a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.o_stride = o_stride;
+
+    void* own = nullptr;
+    int rc = GRL_OK;
+    if (rope == GRL_ROPE_HALF) {
+        // (d, d+D/2) pairs straddle MFMA chunks: rotate Q and K once into a workspace with the
+        // standalone kernel, then run the plain kernel on the rotated copies.
+        GRL_REQUIRE(q_stride == hd && k_stride == hd, GRL_ERR_SHAPE, "%s: rotate-half RoPE needs contiguous Q and K", who);
+        const size_t n = (size_t)B * S * H * D, bytes = n * grl_dtype_size(dtype);
+        char* ws = (char*)workspace;
+        if (!ws) { own = grl_malloc(c, 2 * bytes); if (!own) return GRL_ERR_OOM; ws = (char*)own; }
+        rc = grl_rope(c, dtype, B, S, H, D, Q, nullptr, ws, GRL_ROPE_HALF, rope_base, rope_scaling);
+        if (!rc) rc = grl_rope(c, dtype, B, S, H, D, K, nullptr, ws + bytes, GRL_ROPE_HALF, rope_base, rope_scaling);
+        a.Q = ws; a.K = ws + bytes;
+    } else if (rope == GRL_ROPE_INTERLEAVED) {
+        const size_t bytes = (size_t)S * (D / 2) * sizeof(float2);
+        own = grl_malloc(c, bytes);
+        if (!own) return GRL_ERR_OOM;
+        rc = grl_build_rope_table(c, (float*)own, (int)S, (int)D, rope_base, rope_scaling);
+        a.rope = (const float2*)own;
+    }
+    const bool fused = rope == GRL_ROPE_INTERLEAVED;
+    if (!rc) {
+        if (dtype == GRL_F32) {
+            rc = D == 32 ? launch_fa<float, 32>(c, a, fused) : D == 64 ? launch_fa<float, 64>(c, a, fused) : launch_fa<float, 128>(c, a, fused);
+        } else {
+            rc = D == 32 ? launch_fa<uint16_t, 32>(c, a, fused) : D == 64 ? launch_fa<uint16_t, 64>(c, a, fused) : launch_fa<uint16_t, 128>(c, a, fused);
+        }
+    }
+    if (own) grl_free(c, own);   // stream order keeps it alive until the kernel has finished
+    return rc;
+}
+
+extern "C" int grl_fa2_fwd(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                           const void* Q, const void* K, const void* V, const float* mask, void* O,
+                           float scale, int causal, int rope, float rope_base, float rope_scaling, void* workspace) {
+    const int64_t hd = H * D;
+    return fa2_common(c, "grl_fa2_fwd", dtype, B, S, H, D, Q, K, V, mask, O, hd, hd, hd, hd, scale, causal, rope,
+                      rope_base, rope_scaling, workspace);
+}
+
+extern "C" int grl_fa2_fwd_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                                   const void* Q, const void* K, const void* V, const float* mask, void* O,
+                                   int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                                   float scale, int causal, int rope, float rope_base, float rope_scaling) {
+    return fa2_common(c, "grl_fa2_fwd_strided", dtype, B, S, H, D, Q, K, V, mask, O, q_stride, k_stride, v_stride,
+                      o_stride, scale, causal, rope, rope_base, rope_scaling, nullptr);
+}

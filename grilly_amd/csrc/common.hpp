@@ -1,0 +1,115 @@
+// Shared host/device helpers for libgrilly_hip (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <cstdio>
+#include <cstdarg>
+#include <map>
+#include <mutex>
+#include <vector>
+#include "../../include/grilly_hip.h"
+
+// ---------------------------------------------------------------- context
+struct grl_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipDeviceProp_t prop{};
+    std::mutex mu;
+    // caching pool: bucket size -> free blocks; live pointer -> bucket size
+    std::map<size_t, std::vector<void*>> free_blocks;
+    std::map<void*, size_t> live;
+    grl_pool_stats stats{};
+};
+
+void grl_set_error(const char* fmt, ...);
+
+#define GRL_CHECK_HIP(expr)                                                              \
+    do {                                                                                 \
+        hipError_t _e = (expr);                                                          \
+        if (_e != hipSuccess) {                                                          \
+            grl_set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+            return GRL_ERR_HIP;                                                          \
+        }                                                                                \
+    } while (0)
+
+#define GRL_REQUIRE(cond, code, ...)                                                     \
+    do {                                                                                 \
+        if (!(cond)) {                                                                   \
+            grl_set_error(__VA_ARGS__);                                                  \
+            return (code);                                                               \
+        }                                                                                \
+    } while (0)
+
+// Checks the launch itself (bad configuration, missing code object); kernel faults
+// surface at the next synchronisation.
+#define GRL_CHECK_LAUNCH()  GRL_CHECK_HIP(hipGetLastError())
+
+static inline bool grl_valid_dtype(int d) { return d == GRL_F32 || d == GRL_BF16; }
+static inline size_t grl_dtype_size(int d) { return d == GRL_BF16 ? 2 : 4; }
+
+// pool-backed temporary that is returned to the pool when it goes out of scope;
+// safe because every kernel of a context runs in order on the one stream.
+struct grl_temp {
+    grl_ctx* ctx; void* p;
+    grl_temp(grl_ctx* c, size_t bytes) : ctx(c), p(grl_malloc(c, bytes)) {}
+    ~grl_temp() { if (p) grl_free(ctx, p); }
+    grl_temp(const grl_temp&) = delete;
+    grl_temp& operator=(const grl_temp&) = delete;
+};
+
+// ---------------------------------------------------------------- device helpers
+#if defined(__HIPCC__)
+typedef __bf16 bf16_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+// fp32 -> bf16 bits, round to nearest even; NaN stays NaN.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+    return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+// two floats -> packed pair of bf16 (lo in bits 0..15)
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+__device__ __forceinline__ float bf16lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+template <typename T> struct elem;
+template <> struct elem<float> {
+    static __device__ __forceinline__ float ld(const float* p) { return *p; }
+    static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template <> struct elem<uint16_t> {   // bf16 storage
+    static __device__ __forceinline__ float ld(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+    static __device__ __forceinline__ void st(uint16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+};
+
+// ---- activation closed forms of the reference shaders
+// shaders/fused-linear-gelu.glsl:45-63 and shaders/activation-gelu.glsl:33-50
+__device__ __forceinline__ float gelu_ref(float x) {
+    float c = fminf(fmaxf(x, -50.0f), 50.0f);
+    float inner = 0.7978845608028654f * (c + 0.044715f * (c * c * c));
+    float r = 0.5f * x * (1.0f + tanhf(inner));
+    if (fabsf(x) > 50.0f) r = x > 0.0f ? x : 0.0f;
+    return r;
+}
+// shaders/fused-linear-silu.glsl:43-48
+__device__ __forceinline__ float silu_clamped(float x) {
+    float c = fminf(fmaxf(x, -88.0f), 88.0f);
+    return x * (1.0f / (1.0f + __expf(-c)));
+}
+// shaders/fused-swiglu.glsl:44-46
+__device__ __forceinline__ float silu_plain(float x) { return x / (1.0f + __expf(-x)); }
+#endif

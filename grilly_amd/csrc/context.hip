@@ -1,0 +1,204 @@
+// Context, caching device-buffer pool, copies and the event stopwatch.
+#include "common.hpp"
+#include <cstring>
+
+static thread_local char g_err[512] = "";
+
+void grl_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char* grl_last_error(void) { return g_err; }
+
+extern "C" grl_ctx* grl_create(int device) {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        grl_set_error("no HIP device visible (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+        return nullptr;
+    }
+    if (device < 0 || device >= n) {
+        grl_set_error("device %d out of range (0..%d)", device, n - 1);
+        return nullptr;
+    }
+    grl_ctx* c = new grl_ctx();
+    c->device = device;
+    if ((e = hipSetDevice(device)) != hipSuccess ||
+        (e = hipGetDeviceProperties(&c->prop, device)) != hipSuccess ||
+        (e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking)) != hipSuccess ||
+        (e = hipEventCreate(&c->ev0)) != hipSuccess ||
+        (e = hipEventCreate(&c->ev1)) != hipSuccess) {
+        grl_set_error("context creation failed: %s", hipGetErrorString(e));
+        delete c;
+        return nullptr;
+    }
+    if (strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
+        grl_set_error("device %d is %s; this library carries gfx950 code only", device, c->prop.gcnArchName);
+        hipStreamDestroy(c->stream);
+        delete c;
+        return nullptr;
+    }
+    return c;
+}
+
+extern "C" void grl_destroy(grl_ctx* c) {
+    if (!c) return;
+    hipSetDevice(c->device);
+    hipStreamSynchronize(c->stream);
+    for (auto& kv : c->free_blocks)
+        for (void* p : kv.second) hipFree(p);
+    for (auto& kv : c->live) hipFree(kv.first);
+    hipEventDestroy(c->ev0);
+    hipEventDestroy(c->ev1);
+    hipStreamDestroy(c->stream);
+    delete c;
+}
+
+extern "C" void* grl_stream(grl_ctx* c) { return c ? (void*)c->stream : nullptr; }
+
+extern "C" int grl_device_info(grl_ctx* c, grl_devinfo* out) {
+    GRL_REQUIRE(c && out, GRL_ERR_ARG, "grl_device_info: null argument");
+    memset(out, 0, sizeof(*out));
+    strncpy(out->name, c->prop.name, sizeof(out->name) - 1);
+    strncpy(out->arch, c->prop.gcnArchName, sizeof(out->arch) - 1);
+    out->compute_units = c->prop.multiProcessorCount;
+    out->clock_khz = c->prop.clockRate;
+    out->lds_bytes_per_block = (int32_t)c->prop.sharedMemPerBlock;
+    out->wavefront = c->prop.warpSize;
+    out->hbm_bytes = (int64_t)c->prop.totalGlobalMem;
+    return GRL_OK;
+}
+
+// ---------------------------------------------------------------- pool
+// Buckets are powers of two from 256 B; blocks above 1 GiB round to a multiple of
+// 256 MiB instead so a 3 GiB activation does not pin 4 GiB.
+static size_t bucket_of(size_t bytes) {
+    if (bytes <= 256) return 256;
+    const size_t big = (size_t)1 << 30, step = (size_t)256 << 20;
+    if (bytes > big) return (bytes + step - 1) / step * step;
+    size_t b = 256;
+    while (b < bytes) b <<= 1;
+    return b;
+}
+
+extern "C" void* grl_malloc(grl_ctx* c, size_t bytes) {
+    if (!c) { grl_set_error("grl_malloc: null context"); return nullptr; }
+    if (bytes == 0) bytes = 1;
+    size_t b = bucket_of(bytes);
+    std::lock_guard<std::mutex> lk(c->mu);
+    void* p = nullptr;
+    auto it = c->free_blocks.find(b);
+    if (it != c->free_blocks.end() && !it->second.empty()) {
+        p = it->second.back();
+        it->second.pop_back();
+        c->stats.hits++;
+        c->stats.bytes_cached -= (int64_t)b;
+    } else {
+        hipSetDevice(c->device);
+        hipError_t e = hipMalloc(&p, b);
+        if (e != hipSuccess) {
+            // drop the cache and retry once before reporting out-of-memory
+            (void)hipGetLastError();
+            hipStreamSynchronize(c->stream);
+            for (auto& kv : c->free_blocks) {
+                for (void* q : kv.second) hipFree(q);
+                kv.second.clear();
+            }
+            c->stats.bytes_cached = 0;
+            e = hipMalloc(&p, b);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                grl_set_error("grl_malloc: hipMalloc(%zu) failed: %s", b, hipGetErrorString(e));
+                return nullptr;
+            }
+        }
+        c->stats.misses++;
+        c->stats.allocations++;
+    }
+    c->live[p] = b;
+    c->stats.bytes_in_use += (int64_t)b;
+    if (c->stats.bytes_in_use > c->stats.bytes_peak) c->stats.bytes_peak = c->stats.bytes_in_use;
+    return p;
+}
+
+extern "C" int grl_free(grl_ctx* c, void* p) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_free: null context");
+    if (!p) return GRL_OK;
+    std::lock_guard<std::mutex> lk(c->mu);
+    auto it = c->live.find(p);
+    GRL_REQUIRE(it != c->live.end(), GRL_ERR_ARG, "grl_free: pointer %p was not allocated by this context", p);
+    size_t b = it->second;
+    c->live.erase(it);
+    c->free_blocks[b].push_back(p);
+    c->stats.bytes_in_use -= (int64_t)b;
+    c->stats.bytes_cached += (int64_t)b;
+    return GRL_OK;
+}
+
+extern "C" int grl_pool_get_stats(grl_ctx* c, grl_pool_stats* out) {
+    GRL_REQUIRE(c && out, GRL_ERR_ARG, "grl_pool_get_stats: null argument");
+    std::lock_guard<std::mutex> lk(c->mu);
+    *out = c->stats;
+    return GRL_OK;
+}
+
+extern "C" int grl_pool_trim(grl_ctx* c) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_pool_trim: null context");
+    GRL_CHECK_HIP(hipStreamSynchronize(c->stream));
+    std::lock_guard<std::mutex> lk(c->mu);
+    for (auto& kv : c->free_blocks) {
+        for (void* q : kv.second) hipFree(q);
+        kv.second.clear();
+    }
+    c->stats.bytes_cached = 0;
+    return GRL_OK;
+}
+
+// ---------------------------------------------------------------- copies
+extern "C" int grl_h2d(grl_ctx* c, void* dst, const void* src, size_t bytes) {
+    GRL_REQUIRE(c && (bytes == 0 || (dst && src)), GRL_ERR_ARG, "grl_h2d: null argument");
+    if (!bytes) return GRL_OK;
+    GRL_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, c->stream));
+    GRL_CHECK_HIP(hipStreamSynchronize(c->stream));
+    return GRL_OK;
+}
+extern "C" int grl_d2h(grl_ctx* c, void* dst, const void* src, size_t bytes) {
+    GRL_REQUIRE(c && (bytes == 0 || (dst && src)), GRL_ERR_ARG, "grl_d2h: null argument");
+    if (!bytes) return GRL_OK;
+    GRL_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c->stream));
+    GRL_CHECK_HIP(hipStreamSynchronize(c->stream));
+    return GRL_OK;
+}
+extern "C" int grl_d2d(grl_ctx* c, void* dst, const void* src, size_t bytes) {
+    GRL_REQUIRE(c && (bytes == 0 || (dst && src)), GRL_ERR_ARG, "grl_d2d: null argument");
+    if (!bytes) return GRL_OK;
+    GRL_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, c->stream));
+    return GRL_OK;
+}
+extern "C" int grl_memset(grl_ctx* c, void* dst, int byte, size_t bytes) {
+    GRL_REQUIRE(c && (bytes == 0 || dst), GRL_ERR_ARG, "grl_memset: null argument");
+    if (!bytes) return GRL_OK;
+    GRL_CHECK_HIP(hipMemsetAsync(dst, byte, bytes, c->stream));
+    return GRL_OK;
+}
+extern "C" int grl_sync(grl_ctx* c) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_sync: null context");
+    GRL_CHECK_HIP(hipStreamSynchronize(c->stream));
+    return GRL_OK;
+}
+
+extern "C" int grl_timer_start(grl_ctx* c) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_timer_start: null context");
+    GRL_CHECK_HIP(hipEventRecord(c->ev0, c->stream));
+    return GRL_OK;
+}
+extern "C" int grl_timer_stop(grl_ctx* c, float* ms) {
+    GRL_REQUIRE(c && ms, GRL_ERR_ARG, "grl_timer_stop: null argument");
+    GRL_CHECK_HIP(hipEventRecord(c->ev1, c->stream));
+    GRL_CHECK_HIP(hipEventSynchronize(c->ev1));
+    GRL_CHECK_HIP(hipEventElapsedTime(ms, c->ev0, c->ev1));
+    return GRL_OK;
+}

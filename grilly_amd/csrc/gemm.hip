@@ -1,0 +1,436 @@
+// MFMA GEMM family for gfx950:  C[m,n] = epi( sum_k A[m,k]*W[n,k] + bias[n] )
+//
+// Both operands are K-contiguous, which is the layout MFMA wants: every lane feeds the
+// matrix core 16 contiguous bytes of one row (8 bf16 for v_mfma_f32_32x32x16_bf16, or
+// 4 fp32 that drive four v_mfma_f32_32x32x2_f32).  A workgroup owns a BM x BN tile of C
+// and walks K in slabs of 128 bytes per row (64 bf16 / 32 fp32):
+//
+//   HBM --128-bit loads--> VGPR --ds_write_b128--> LDS (2 stages, XOR-swizzled 16-B chunks)
+//       --ds_read_b128--> MFMA operands --> fp32 accumulators (registers, never spilled to LDS)
+//       --> bias / GELU / SiLU / SwiGLU epilogue in registers --> 8/16-byte stores
+//
+// The loads for slab t+1 are issued before the MFMAs of slab t and parked in registers, so
+// HBM/L2 latency hides behind the matrix work; one barrier per slab.
+//
+// MFMA operand roles are swapped (the weight rows are the "A" operand, the activation rows
+// the "B" operand) so that each lane ends up with 4 consecutive output columns of one
+// output row: stores are 8 B (bf16) / 16 B (fp32) wide and bias is a 4-vector per lane.
+//
+// LDS bank behaviour: a tile row is 128 B = 8 chunks of 16 B; chunk c of row r lives at
+// slot c ^ (r & 7).  Eight consecutive lanes (eight consecutive rows, same logical chunk)
+// therefore hit eight different slots = all 32 banks once, for the reads as for the writes.
+#include "common.hpp"
+#include <type_traits>
+
+int grl_transpose2d(grl_ctx* c, int dtype, int64_t R, int64_t C, const void* in, void* out);
+
+struct GemmArgs {
+    const void* A;       // (M,K)
+    const void* W;       // (N,K)
+    const void* W2;      // (N,K) second weight (SwiGLU "up"), else null
+    const float* bias;   // (N) or null
+    const float* bias2;  // (N) or null
+    void* C;             // (M,N)
+    float* cache1;       // fp32 (M,N) pre-activation of W  (SwiGLU gate) or null
+    float* cache2;       // fp32 (M,N) pre-activation of W2 (SwiGLU up) or null
+    int M, N, K;
+    int tiles_m, tiles_n;
+};
+
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
+
+template <int EPI> __device__ __forceinline__ float epi_apply(float v) {
+    if (EPI == EPI_GELU) {
+        // same closed form as gelu_ref, with tanh(u) = 1 - 2/(exp(2u)+1): one v_exp instead of
+        // the library tanhf; absolute error ~1e-7, and the +-50 rule is kept.
+        float c = fminf(fmaxf(v, -50.0f), 50.0f);
+        float inner = 0.7978845608028654f * (c + 0.044715f * (c * c * c));
+        float t = 1.0f - 2.0f / (__expf(2.0f * inner) + 1.0f);
+        float r = 0.5f * v * (1.0f + t);
+        if (fabsf(v) > 50.0f) r = v > 0.0f ? v : 0.0f;
+        return r;
+    }
+    if (EPI == EPI_SILU) return silu_clamped(v);
+    return v;
+}
+
+// ---- one 128-byte-per-row K slab on the matrix cores --------------------------------------
+template <typename T> struct MfmaSlab;
+template <> struct MfmaSlab<uint16_t> {   // bf16: 16 B = 8 values, k = 8*(lane/32)+e
+    static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), acc, 0, 0, 0);
+    }
+};
+template <> struct MfmaSlab<float> {      // fp32: 16 B = 4 values, each feeds one 32x32x2 MFMA
+    static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, w[e]), __builtin_bit_cast(float, x[e]), acc, 0, 0, 0);
+    }
+};
+
+// compile-time loop: f(std::integral_constant<int, 0..N-1>)
+template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+template <typename OutT> __device__ __forceinline__ void store4(OutT* p, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
+    f32x4 v = {a, b, c, d};
+    *(f32x4*)p = v;
+}
+template <> __device__ __forceinline__ void store4<uint16_t>(uint16_t* p, float a, float b, float c, float d) {
+    u32x2 v = {pack_bf16x2(a, b), pack_bf16x2(c, d)};
+    *(u32x2*)p = v;
+}
+
+// BN counts LDS rows of the weight tile; with DUAL it is 2x the output-column count of the
+// tile (first half gate rows, second half up rows).
+template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL>
+__global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int EPC = 16 / (int)sizeof(T);     // elements per 16-byte chunk
+    constexpr int BK = 8 * EPC;                  // elements per 128-byte slab row
+    constexpr int WM = BM / WGM, WN = BN / WGN;  // per-wave tile (WN in LDS rows)
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int BNO = DUAL ? BN / 2 : BN;      // output columns per tile
+    constexpr int WNO = DUAL ? WN / 2 : WN;      // output columns per wave
+    constexpr int TNO = DUAL ? TN / 2 : TN;
+    constexpr int CA = BM * 8 / NT, CB = BN * 8 / NT;
+    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile rows must divide over the threads");
+    static_assert(!DUAL || (BN / 2) % (NT / 8) == 0, "a staging pass must not straddle the two weights");
+    static_assert(WM % 32 == 0 && WN % 32 == 0 && (!DUAL || TN % 2 == 0), "wave tile is made of 32x32 MFMA tiles");
+    constexpr int STAGE = (BM + BN) * 128;
+    __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int li = lane & 31, lg = lane >> 5;
+
+    // ---- workgroup -> tile: give each XCD (workgroups are dealt round-robin over the 8 XCDs)
+    // a contiguous run of tiles, and walk tiles in bands of 8 tile-rows so that the 32 CUs of
+    // an XCD share a small set of A and W row panels in their L2.
+    int tile_m, tile_n;
+    {
+        const int nb = gridDim.x, pid = blockIdx.x;
+        const int per = nb >> 3, rem = nb & 7, xcd = pid & 7, loc = pid >> 3;
+        const int npid = xcd * per + (xcd < rem ? xcd : rem) + loc;
+        constexpr int GROUP = 8;
+        const int width = GROUP * p.tiles_n;
+        const int first_m = (npid / width) * GROUP;
+        const int gsize = p.tiles_m - first_m < GROUP ? p.tiles_m - first_m : GROUP;
+        tile_m = first_m + (npid % width) % gsize;
+        tile_n = (npid % width) / gsize;
+    }
+    const int m0 = tile_m * BM, n0 = tile_n * BNO;
+
+    // ---- global -> register staging through buffer loads: the resource starts at the tile's
+    // first row and ends with the tensor, so rows past the edge read as zero in hardware; the
+    // slab offset travels in a scalar register.  Thread t owns chunk (t & 7) of row (t >> 3)
+    // of every 32-row pass; K chunks past the end are zeroed when the slab is written to LDS.
+    constexpr int RPP = NT / 8;                   // rows per pass
+    const int row_t = tid >> 3, c_t = tid & 7;
+    const int64_t rowbytes = (int64_t)p.K * (int64_t)sizeof(T);
+    auto make_rsrc = [&](const void* base, int first_row, int rows_total) {
+        int64_t left = (int64_t)(rows_total - first_row) * rowbytes;
+        if (left < 0) left = 0;
+        uint32_t nrec = left > 0xffffffffLL ? 0xffffffffu : (uint32_t)left;
+        return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base + (int64_t)first_row * rowbytes), 0, (int)nrec, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(p.A, m0, p.M);
+    const __amdgpu_buffer_rsrc_t rsW = make_rsrc(p.W, n0, p.N);
+    const __amdgpu_buffer_rsrc_t rsW2 = make_rsrc(DUAL ? p.W2 : p.W, n0, p.N);
+    const int voff = row_t * (int)rowbytes + c_t * 16;
+    const int pass_stride = RPP * (int)rowbytes;
+    const int soff_t = row_t * 128 + ((c_t ^ (row_t & 7)) << 4);
+
+    u32x4 ra[CA], rb[CB];
+    auto load_slab = [&](int kt) {
+        const int sbyte = kt * 128;
+#pragma unroll
+        for (int i = 0; i < CA; ++i)
+            ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsA, voff + i * pass_stride, sbyte, 0));
+#pragma unroll
+        for (int i = 0; i < CB; ++i) {
+            const bool second = DUAL && (i * RPP >= BNO);
+            const int vo = voff + (second ? i - BNO / RPP : i) * pass_stride;
+            rb[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(second ? rsW2 : rsW, vo, sbyte, 0));
+        }
+    };
+    // the K-tail select sits here, after the MFMAs of the previous slab, so that nothing
+    // between the load and this point waits on the data
+    auto stash_slab = [&](int kt) {
+        char* s = lds + (kt & 1) * STAGE + soff_t;
+        const bool live = kt * BK + c_t * EPC < p.K;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < CA; ++i) *(u32x4*)(s + i * RPP * 128) = live ? ra[i] : zero;
+#pragma unroll
+        for (int i = 0; i < CB; ++i) *(u32x4*)(s + BM * 128 + i * RPP * 128) = live ? rb[i] : zero;
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+    // LDS row of this lane inside each 32-row operand tile
+    int rowX[TM], rowW[TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a) rowX[a] = wm * WM + a * 32 + li;
+#pragma unroll
+    for (int b = 0; b < TN; ++b) {
+        int base = DUAL ? ((b >= TNO ? BNO : 0) + wn * WNO + (b % TNO) * 32) : (wn * WN + b * 32);
+        rowW[b] = base + li;
+    }
+
+    const int KT = (p.K + BK - 1) / BK;
+    load_slab(0);
+    stash_slab(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const bool more = kt + 1 < KT;
+        if (more) load_slab(kt + 1);
+        const char* s = lds + (kt & 1) * STAGE;
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            const int ch = 2 * sl + lg;
+            u32x4 xf[TM], wf[TN];
+#pragma unroll
+            for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ (rowX[a] & 7)) << 4));
+#pragma unroll
+            for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ (rowW[b] & 7)) << 4));
+            static_for<TM>([&](auto ia) {
+                static_for<TN>([&](auto ib) {
+                    MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
+                });
+            });
+        }
+        if (more) stash_slab(kt + 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane (li, lg) holds, for output row m = .. + li, the columns
+    // n = .. + 8*q + 4*lg + {0..3} in accumulator registers 4q..4q+3.  Every index into the
+    // accumulators is a compile-time constant so they stay in registers.
+    OutT* C = (OutT*)p.C;
+    const bool vec_ok = (p.N & 3) == 0;
+    static_for<TM>([&](auto ia) {
+        constexpr int a = decltype(ia)::value;
+        const int m = m0 + wm * WM + a * 32 + li;
+        static_for<TNO>([&](auto ib) {
+            constexpr int b = decltype(ib)::value;
+            static_for<4>([&](auto iq) {
+                constexpr int q = decltype(iq)::value;
+                const int n = n0 + wn * WNO + b * 32 + 8 * q + 4 * lg;
+                if (m < p.M && n < p.N) {
+                    float v[4], u[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = acc[a][b][4 * q + e];
+                        u[e] = DUAL ? acc[a][DUAL ? b + TNO : b][4 * q + e] : 0.f;
+                    }
+                    const int64_t o = (int64_t)m * p.N + n;
+                    if (vec_ok) {
+                        if (p.bias) {
+                            f32x4 bv = *(const f32x4*)(p.bias + n);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] += bv[e];
+                        }
+                        if (DUAL) {
+                            if (p.bias2) {
+                                f32x4 bv = *(const f32x4*)(p.bias2 + n);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) u[e] += bv[e];
+                            }
+                            if (p.cache1) store4<float>(p.cache1 + o, v[0], v[1], v[2], v[3]);
+                            if (p.cache2) store4<float>(p.cache2 + o, u[0], u[1], u[2], u[3]);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(u[e]);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
+                        }
+                        store4<OutT>(C + o, v[0], v[1], v[2], v[3]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (n + e < p.N) {
+                                float x = v[e] + (p.bias ? p.bias[n + e] : 0.f);
+                                if (DUAL) {
+                                    float y = u[e] + (p.bias2 ? p.bias2[n + e] : 0.f);
+                                    if (p.cache1) p.cache1[o + e] = x;
+                                    if (p.cache2) p.cache2[o + e] = y;
+                                    x = x * silu_plain(y);
+                                } else {
+                                    x = epi_apply<EPI>(x);
+                                }
+                                elem<OutT>::st(C + o + e, x);
+                            }
+                        }
+                    }
+                }
+            });
+        });
+    });
+}
+
+// ---- any shape / any alignment: one thread per output, ascending-k fp32 sum (the summation
+// order of shaders/fnn-linear.glsl:45-49).  Used only when rows are not 16-byte aligned.
+template <typename T, typename OutT, int EPI, bool DUAL>
+__global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmArgs p) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)p.M * p.N) return;
+    const int m = (int)(idx / p.N), n = (int)(idx % p.N);
+    const T* a = (const T*)p.A + (int64_t)m * p.K;
+    const T* w = (const T*)p.W + (int64_t)n * p.K;
+    float s = 0.f;
+    for (int k = 0; k < p.K; ++k) s += elem<T>::ld(a + k) * elem<T>::ld(w + k);
+    if (p.bias) s += p.bias[n];
+    if (DUAL) {
+        const T* w2 = (const T*)p.W2 + (int64_t)n * p.K;
+        float u = 0.f;
+        for (int k = 0; k < p.K; ++k) u += elem<T>::ld(a + k) * elem<T>::ld(w2 + k);
+        if (p.bias2) u += p.bias2[n];
+        if (p.cache1) p.cache1[idx] = s;
+        if (p.cache2) p.cache2[idx] = u;
+        s = s * silu_plain(u);
+    } else {
+        s = epi_apply<EPI>(s);
+    }
+    elem<OutT>::st((OutT*)p.C + idx, s);
+}
+
+// ------------------------------------------------------------------ host dispatch
+template <typename T, typename OutT, int EPI, bool DUAL>
+static int launch_gemm(grl_ctx* c, GemmArgs& a) {
+    const int64_t epc = 16 / (int64_t)sizeof(T);
+    const bool aligned = (a.K % epc == 0) && ((((uintptr_t)a.A) | ((uintptr_t)a.W) | ((uintptr_t)a.W2)) & 15u) == 0 &&
+                         ((((uintptr_t)a.C) | ((uintptr_t)a.bias) | ((uintptr_t)a.bias2) | ((uintptr_t)a.cache1) | ((uintptr_t)a.cache2)) & 15u) == 0;
+    if (!aligned) {
+        int64_t total = (int64_t)a.M * a.N;
+        GRL_REQUIRE((total + 255) / 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: unaligned problem too large for the scalar kernel");
+        hipLaunchKernelGGL((gemm_nt_scalar_kernel<T, OutT, EPI, DUAL>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, a);
+        GRL_CHECK_LAUNCH();
+        return GRL_OK;
+    }
+    // big tile when it fills the 256 CUs at least ~once, else the small tile for more workgroups
+    const int64_t big_m = (a.M + 255) / 256, big_n = (a.N + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
+    if (big_m * big_n >= 192) {
+        a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
+        hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 256, 256, 2, 2, EPI, DUAL>), dim3((unsigned)(big_m * big_n)), dim3(256), 0, c->stream, a);
+    } else {
+        const int64_t sm = (a.M + 127) / 128, sn = (a.N + (DUAL ? 63 : 127)) / (DUAL ? 64 : 128);
+        GRL_REQUIRE(sm * sn < (1LL << 31), GRL_ERR_SHAPE, "gemm: too many tiles");
+        a.tiles_m = (int)sm; a.tiles_n = (int)sn;
+        hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)(sm * sn)), dim3(256), 0, c->stream, a);
+    }
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+template <typename T, typename OutT>
+static int dispatch_epi(grl_ctx* c, GemmArgs& a, int epi) {
+    switch (epi) {
+        case EPI_NONE: return launch_gemm<T, OutT, EPI_NONE, false>(c, a);
+        case EPI_GELU: return launch_gemm<T, OutT, EPI_GELU, false>(c, a);
+        case EPI_SILU: return launch_gemm<T, OutT, EPI_SILU, false>(c, a);
+        case EPI_SWIGLU: return launch_gemm<T, OutT, EPI_SWIGLU, true>(c, a);
+    }
+    grl_set_error("gemm: bad epilogue %d", epi);
+    return GRL_ERR_ARG;
+}
+
+static int dispatch_types(grl_ctx* c, GemmArgs& a, int in_dtype, int out_dtype, int epi) {
+    if (in_dtype == GRL_F32 && out_dtype == GRL_F32) return dispatch_epi<float, float>(c, a, epi);
+    if (in_dtype == GRL_BF16 && out_dtype == GRL_BF16) return dispatch_epi<uint16_t, uint16_t>(c, a, epi);
+    if (in_dtype == GRL_BF16 && out_dtype == GRL_F32) return dispatch_epi<uint16_t, float>(c, a, epi);
+    if (in_dtype == GRL_F32 && out_dtype == GRL_BF16) return dispatch_epi<float, uint16_t>(c, a, epi);
+    grl_set_error("gemm: bad dtype in=%d out=%d", in_dtype, out_dtype);
+    return GRL_ERR_ARG;
+}
+
+static int check_dims(const char* who, int64_t M, int64_t N, int64_t K) {
+    GRL_REQUIRE(M >= 0 && N >= 0 && K >= 0, GRL_ERR_SHAPE, "%s: negative dimension", who);
+    GRL_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31), GRL_ERR_SHAPE, "%s: dimension exceeds 2^31-1", who);
+    return GRL_OK;
+}
+
+// K == 0: the sum is empty, C = epi(bias)
+template <typename OutT>
+__global__ __launch_bounds__(256) void bias_fill_kernel(OutT* C, const float* bias, int64_t total, int N, int epi) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float v = bias ? bias[i % N] : 0.f;
+    v = epi == EPI_GELU ? epi_apply<EPI_GELU>(v) : epi == EPI_SILU ? epi_apply<EPI_SILU>(v) : v;
+    elem<OutT>::st(C + i, v);
+}
+
+extern "C" int grl_gemm_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                           const void* A, const void* W, const float* bias, void* C, int epilogue) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_gemm_nt: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_gemm_nt: bad dtype");
+    GRL_REQUIRE(epilogue >= GRL_EPI_NONE && epilogue <= GRL_EPI_SILU, GRL_ERR_ARG, "grl_gemm_nt: bad epilogue %d", epilogue);
+    int rc = check_dims("grl_gemm_nt", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    GRL_REQUIRE(C && (K == 0 || (A && W)), GRL_ERR_ARG, "grl_gemm_nt: null argument");
+    if (K == 0) {
+        int64_t total = M * N;
+        GRL_REQUIRE((total + 255) / 256 < (1LL << 31), GRL_ERR_SHAPE, "grl_gemm_nt: output too large");
+        if (out_dtype == GRL_F32) hipLaunchKernelGGL(bias_fill_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, (float*)C, bias, total, (int)N, epilogue);
+        else hipLaunchKernelGGL(bias_fill_kernel<uint16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, (uint16_t*)C, bias, total, (int)N, epilogue);
+        GRL_CHECK_LAUNCH();
+        return GRL_OK;
+    }
+    GemmArgs a{};
+    a.A = A; a.W = W; a.bias = bias; a.C = C;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    return dispatch_types(c, a, in_dtype, out_dtype, epilogue);
+}
+
+extern "C" int grl_swiglu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                             const void* x, const void* W_gate, const void* W_up, const float* b_gate,
+                             const float* b_up, void* out, float* gate_cache, float* up_cache) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_swiglu_nt: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_swiglu_nt: bad dtype");
+    int rc = check_dims("grl_swiglu_nt", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    GRL_REQUIRE(out && K > 0 && x && W_gate && W_up, GRL_ERR_ARG, "grl_swiglu_nt: null argument or K == 0");
+    GemmArgs a{};
+    a.A = x; a.W = W_gate; a.W2 = W_up; a.C = out;
+    // the reference applies biases only when both are present (backend/_glu_append.py:68)
+    if (b_gate && b_up) { a.bias = b_gate; a.bias2 = b_up; }
+    a.cache1 = gate_cache; a.cache2 = up_cache;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    return dispatch_types(c, a, in_dtype, out_dtype, EPI_SWIGLU);
+}
+
+extern "C" int grl_gemm_nn(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                           const void* A, const void* B, void* C, void* workspace) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_gemm_nn: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_gemm_nn: bad dtype");
+    int rc = check_dims("grl_gemm_nn", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    if (K == 0) return grl_gemm_nt(c, in_dtype, out_dtype, M, N, 0, A, B, nullptr, C, GRL_EPI_NONE);
+    GRL_REQUIRE(A && B && C, GRL_ERR_ARG, "grl_gemm_nn: null argument");
+    void* ws = workspace;
+    void* own = nullptr;
+    if (!ws) {
+        own = grl_malloc(c, (size_t)K * N * grl_dtype_size(in_dtype));
+        if (!own) return GRL_ERR_OOM;
+        ws = own;
+    }
+    rc = grl_transpose2d(c, in_dtype, K, N, B, ws);   // (K,N) -> (N,K)
+    if (!rc) rc = grl_gemm_nt(c, in_dtype, out_dtype, M, N, K, A, ws, nullptr, C, GRL_EPI_NONE);
+    if (own) grl_free(c, own);   // stream order keeps the block alive until the GEMM has read it
+    return rc;
+}

@@ -1,0 +1,453 @@
+// HBM-bound kernels: LayerNorm(+residual), elementwise add / GELU / SiLU / SwiGLU,
+// dtype casts, RoPE, embedding gather, masked mean pooling, 2-D transpose.
+// Each moves every input byte once and every output byte once; wave64 reductions only.
+#include "common.hpp"
+#include <cmath>
+
+static inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+
+// ------------------------------------------------------------------ 4-element vectors
+template <typename T> struct vec4;
+template <> struct vec4<float> {
+    f32x4 v;
+    __device__ __forceinline__ void load(const float* p) { v = *(const f32x4*)p; }
+    __device__ __forceinline__ void store(float* p) const { *(f32x4*)p = v; }
+    __device__ __forceinline__ float get(int i) const { return v[i]; }
+    __device__ __forceinline__ void set(int i, float f) { v[i] = f; }
+};
+template <> struct vec4<uint16_t> {
+    u32x2 w;
+    __device__ __forceinline__ void load(const uint16_t* p) { w = *(const u32x2*)p; }
+    __device__ __forceinline__ void store(uint16_t* p) const { *(u32x2*)p = w; }
+    __device__ __forceinline__ float get(int i) const {
+        uint32_t x = w[i >> 1];
+        return (i & 1) ? bf16hi(x) : bf16lo(x);
+    }
+    __device__ __forceinline__ void set(int i, float f) {
+        uint32_t b = f32_to_bf16_bits(f);
+        uint32_t x = w[i >> 1];
+        w[i >> 1] = (i & 1) ? ((x & 0x0000ffffu) | (b << 16)) : ((x & 0xffff0000u) | b);
+    }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// ------------------------------------------------------------------ LayerNorm
+// One wave per row.  Rows of up to 64*4*MAXC elements (F % 4 == 0) stay in registers
+// between the mean pass, the variance pass and the normalise pass, so the row is read
+// from HBM exactly once (the reference makes three dispatches over it,
+// shaders/fnn-layernorm.glsl:44-103).
+template <typename T, int MAXC, bool HAS_RES>
+__global__ __launch_bounds__(256) void layernorm_rows_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, const float* __restrict__ gamma,
+    const float* __restrict__ beta, T* __restrict__ y, int64_t rows, int F, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int nch = F >> 2;
+    const T* xr = x + row * (int64_t)F;
+    const T* rr = HAS_RES ? res + row * (int64_t)F : nullptr;
+    float t[MAXC][4];
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        int ch = lane + c * 64;
+        if (ch < nch) {
+            vec4<T> a; a.load(xr + ch * 4);
+            if (HAS_RES) {
+                vec4<T> b; b.load(rr + ch * 4);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) t[c][i] = a.get(i) + b.get(i);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) t[c][i] = a.get(i);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s += t[c][i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t[c][i] = 0.f;
+        }
+    }
+    const float mean = wave_sum(s) / (float)F;
+    float q = 0.f;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        if (lane + c * 64 < nch) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { float d = t[c][i] - mean; q += d * d; }
+        }
+    }
+    const float var = wave_sum(q) / (float)F;
+    const float sd = sqrtf(var + eps);
+    T* yr = y + row * (int64_t)F;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        int ch = lane + c * 64;
+        if (ch < nch) {
+            f32x4 g = *(const f32x4*)(gamma + ch * 4);
+            f32x4 b = *(const f32x4*)(beta + ch * 4);
+            vec4<T> o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o.set(i, g[i] * ((t[c][i] - mean) / sd) + b[i]);
+            o.store(yr + ch * 4);
+        }
+    }
+}
+
+// Any F: three passes over the row from global memory (the second and third hit L2).
+template <typename T, bool HAS_RES>
+__global__ __launch_bounds__(256) void layernorm_rows_generic_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, const float* __restrict__ gamma,
+    const float* __restrict__ beta, T* __restrict__ y, int64_t rows, int F, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * (int64_t)F;
+    const T* rr = HAS_RES ? res + row * (int64_t)F : nullptr;
+    float s = 0.f;
+    for (int f = lane; f < F; f += 64) s += elem<T>::ld(xr + f) + (HAS_RES ? elem<T>::ld(rr + f) : 0.f);
+    const float mean = wave_sum(s) / (float)F;
+    float q = 0.f;
+    for (int f = lane; f < F; f += 64) {
+        float d = elem<T>::ld(xr + f) + (HAS_RES ? elem<T>::ld(rr + f) : 0.f) - mean;
+        q += d * d;
+    }
+    const float sd = sqrtf(wave_sum(q) / (float)F + eps);
+    T* yr = y + row * (int64_t)F;
+    for (int f = lane; f < F; f += 64) {
+        float v = elem<T>::ld(xr + f) + (HAS_RES ? elem<T>::ld(rr + f) : 0.f);
+        elem<T>::st(yr + f, gamma[f] * ((v - mean) / sd) + beta[f]);
+    }
+}
+
+template <typename T>
+static int launch_layernorm(grl_ctx* c, int64_t rows, int64_t F, const void* x, const void* res,
+                            const float* g, const float* b, float eps, void* y) {
+    dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    const T* X = (const T*)x; const T* R = (const T*)res; T* Y = (T*)y;
+    bool fast = (F % 4 == 0) && F <= 64 * 4 * 8 && aligned16(x) && aligned16(y) && aligned16(g) &&
+                aligned16(b) && (!res || aligned16(res)) && ((F * sizeof(T)) % 8 == 0);
+    // bf16 rows need 8-byte alignment of every row start: F*2 % 8 == 0 <=> F % 4 == 0 (checked)
+#define LN_LAUNCH(MAXC)                                                                             \
+    do {                                                                                            \
+        if (res) hipLaunchKernelGGL((layernorm_rows_kernel<T, MAXC, true>), grid, block, 0, c->stream, X, R, g, b, Y, rows, (int)F, eps); \
+        else     hipLaunchKernelGGL((layernorm_rows_kernel<T, MAXC, false>), grid, block, 0, c->stream, X, R, g, b, Y, rows, (int)F, eps); \
+    } while (0)
+    if (fast) {
+        int nch = (int)(F / 4), maxc = (nch + 63) / 64;
+        if (maxc <= 2) LN_LAUNCH(2);
+        else if (maxc <= 3) LN_LAUNCH(3);
+        else if (maxc <= 4) LN_LAUNCH(4);
+        else LN_LAUNCH(8);
+    } else {
+        if (res) hipLaunchKernelGGL((layernorm_rows_generic_kernel<T, true>), grid, block, 0, c->stream, X, R, g, b, Y, rows, (int)F, eps);
+        else     hipLaunchKernelGGL((layernorm_rows_generic_kernel<T, false>), grid, block, 0, c->stream, X, R, g, b, Y, rows, (int)F, eps);
+    }
+#undef LN_LAUNCH
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+extern "C" int grl_layernorm(grl_ctx* c, int dtype, int64_t rows, int64_t F, const void* x,
+                             const void* residual, const float* gamma, const float* beta, float eps, void* y) {
+    GRL_REQUIRE(c && x && gamma && beta && y, GRL_ERR_ARG, "grl_layernorm: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_layernorm: bad dtype %d", dtype);
+    GRL_REQUIRE(rows >= 0 && F > 0 && F < (1 << 30), GRL_ERR_SHAPE, "grl_layernorm: bad shape rows=%lld F=%lld", (long long)rows, (long long)F);
+    GRL_REQUIRE(rows < ((int64_t)1 << 33), GRL_ERR_SHAPE, "grl_layernorm: too many rows");
+    if (rows == 0) return GRL_OK;
+    return dtype == GRL_F32 ? launch_layernorm<float>(c, rows, F, x, residual, gamma, beta, eps, y)
+                            : launch_layernorm<uint16_t>(c, rows, F, x, residual, gamma, beta, eps, y);
+}
+
+// ------------------------------------------------------------------ elementwise
+enum { OP_ADD = 0, OP_GELU = 1, OP_SILU = 2 };
+
+// shaders/activation-swiglu.glsl:40-49: sign-split stable sigmoid
+__device__ __forceinline__ float sigmoid_stable(float v) {
+    if (v >= 0.f) return 1.0f / (1.0f + __expf(-v));
+    float e = __expf(v);
+    return e / (1.0f + e);
+}
+
+template <int OP> __device__ __forceinline__ float ew_apply(float a, float b) {
+    if (OP == OP_ADD) return a + b;
+    if (OP == OP_GELU) return gelu_ref(a);
+    return a * sigmoid_stable(a);   // backend/fnn.py:344-391 (activation_silu): x*sigmoid(x)
+}
+
+template <typename T, int OP, bool VEC>
+__global__ __launch_bounds__(256) void elementwise_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                         T* __restrict__ out, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (VEC) {
+        const int64_t nv = n >> 2;
+        for (int64_t v = i; v < nv; v += stride) {
+            vec4<T> x, y, o;
+            x.load(a + v * 4);
+            if (OP == OP_ADD) y.load(b + v * 4);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) o.set(k, ew_apply<OP>(x.get(k), OP == OP_ADD ? y.get(k) : 0.f));
+            o.store(out + v * 4);
+        }
+        for (int64_t t = (nv << 2) + i; t < n; t += stride)
+            elem<T>::st(out + t, ew_apply<OP>(elem<T>::ld(a + t), OP == OP_ADD ? elem<T>::ld(b + t) : 0.f));
+    } else {
+        for (int64_t t = i; t < n; t += stride)
+            elem<T>::st(out + t, ew_apply<OP>(elem<T>::ld(a + t), OP == OP_ADD ? elem<T>::ld(b + t) : 0.f));
+    }
+}
+
+static inline unsigned ew_grid(int64_t work_items) {
+    int64_t g = (work_items + 255) / 256;
+    const int64_t cap = 256 * 32;   // 256 CUs x enough waves to cover HBM latency; grid-stride beyond
+    if (g > cap) g = cap;
+    if (g < 1) g = 1;
+    return (unsigned)g;
+}
+
+template <typename T, int OP>
+static int launch_ew(grl_ctx* c, int64_t n, const void* a, const void* b, void* out) {
+    bool vec = aligned16(a) && aligned16(out) && (!b || aligned16(b));
+    if (vec) hipLaunchKernelGGL((elementwise_kernel<T, OP, true>), dim3(ew_grid(n / 4 + 1)), dim3(256), 0, c->stream, (const T*)a, (const T*)b, (T*)out, n);
+    else     hipLaunchKernelGGL((elementwise_kernel<T, OP, false>), dim3(ew_grid(n)), dim3(256), 0, c->stream, (const T*)a, (const T*)b, (T*)out, n);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+#define EW_ENTRY(NAME, OP, NEEDS_B)                                                                   \
+    GRL_REQUIRE(c && a && out && (!(NEEDS_B) || b), GRL_ERR_ARG, NAME ": null argument");             \
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, NAME ": bad dtype %d", dtype);                   \
+    GRL_REQUIRE(n >= 0, GRL_ERR_SHAPE, NAME ": negative size");                                       \
+    if (n == 0) return GRL_OK;                                                                        \
+    return dtype == GRL_F32 ? launch_ew<float, OP>(c, n, a, b, out) : launch_ew<uint16_t, OP>(c, n, a, b, out);
+
+extern "C" int grl_add(grl_ctx* c, int dtype, int64_t n, const void* a, const void* b, void* out) { EW_ENTRY("grl_add", OP_ADD, true) }
+extern "C" int grl_gelu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_gelu", OP_GELU, false) }
+extern "C" int grl_silu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_silu", OP_SILU, false) }
+
+// x (rows, 2h) -> y (rows, h)
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_act_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t h) {
+    const int64_t n = rows * h, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        int64_t r = i / h, p = i - r * h;
+        float x1 = elem<T>::ld(x + r * 2 * h + p);
+        float x2 = elem<T>::ld(x + r * 2 * h + h + p);
+        elem<T>::st(y + i, x1 * (x2 * sigmoid_stable(x2)));
+    }
+}
+
+extern "C" int grl_swiglu_act(grl_ctx* c, int dtype, int64_t rows, int64_t h, const void* x, void* y) {
+    GRL_REQUIRE(c && x && y, GRL_ERR_ARG, "grl_swiglu_act: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_swiglu_act: bad dtype %d", dtype);
+    GRL_REQUIRE(rows >= 0 && h >= 0, GRL_ERR_SHAPE, "grl_swiglu_act: negative size");
+    if (rows * h == 0) return GRL_OK;
+    if (dtype == GRL_F32) hipLaunchKernelGGL(swiglu_act_kernel<float>, dim3(ew_grid(rows * h)), dim3(256), 0, c->stream, (const float*)x, (float*)y, rows, h);
+    else hipLaunchKernelGGL(swiglu_act_kernel<uint16_t>, dim3(ew_grid(rows * h)), dim3(256), 0, c->stream, (const uint16_t*)x, (uint16_t*)y, rows, h);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+// ------------------------------------------------------------------ casts
+template <typename S, typename D>
+__global__ __launch_bounds__(256) void cast_kernel(const S* __restrict__ s, D* __restrict__ d, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        elem<D>::st(d + i, elem<S>::ld(s + i));
+}
+
+extern "C" int grl_cast(grl_ctx* c, int sd, int dd, int64_t n, const void* src, void* dst) {
+    GRL_REQUIRE(c && src && dst, GRL_ERR_ARG, "grl_cast: null argument");
+    GRL_REQUIRE(grl_valid_dtype(sd) && grl_valid_dtype(dd), GRL_ERR_ARG, "grl_cast: bad dtype");
+    GRL_REQUIRE(n >= 0, GRL_ERR_SHAPE, "grl_cast: negative size");
+    if (n == 0) return GRL_OK;
+    dim3 g(ew_grid(n)), b(256);
+    if (sd == GRL_F32 && dd == GRL_BF16) hipLaunchKernelGGL((cast_kernel<float, uint16_t>), g, b, 0, c->stream, (const float*)src, (uint16_t*)dst, n);
+    else if (sd == GRL_BF16 && dd == GRL_F32) hipLaunchKernelGGL((cast_kernel<uint16_t, float>), g, b, 0, c->stream, (const uint16_t*)src, (float*)dst, n);
+    else return grl_d2d(c, dst, src, (size_t)n * grl_dtype_size(sd));
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+// ------------------------------------------------------------------ RoPE
+// inv_freq[p] is the correctly rounded fp32 value of base^(fe), fe = fp32(-2*p)/fp32(D), computed
+// on the host in double; the angle is then formed in fp32 exactly as the shaders do:
+//   half style        theta = (pos / scaling) * inv_freq      shaders/rope.glsl:114-118
+//   interleaved style theta = (pos * inv_freq) / scaling      shaders/flash-attention2-rope.glsl:75-78,124-125
+struct RopeFreq { float inv_freq[64]; };
+
+void grl_rope_freqs(RopeFreq* f, int D, float base) {
+    for (int p = 0; p < 64; ++p) {
+        float fe = (-2.0f * (float)p) / (float)D;
+        f->inv_freq[p] = p < D / 2 ? (float)pow((double)base, (double)fe) : 0.f;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kernel(const T* __restrict__ x, const int32_t* __restrict__ pos_ids,
+                                                  T* __restrict__ y, int64_t total_pairs, int S, int H, int D,
+                                                  int style, float scaling, RopeFreq fr) {
+    const int half = D >> 1;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total_pairs; i += stride) {
+        int p = (int)(i % half);
+        int64_t vec = i / half;                 // (b,s,h) flat
+        int64_t bs = vec / H;                   // (b,s) flat
+        int s = (int)(bs % S);
+        float pos = pos_ids ? (float)pos_ids[bs] : (float)s;
+        float theta = style == GRL_ROPE_HALF ? (pos / scaling) * fr.inv_freq[p] : (pos * fr.inv_freq[p]) / scaling;
+        float sn, cs;
+        sincosf(theta, &sn, &cs);
+        int64_t i0, i1;
+        if (style == GRL_ROPE_HALF) { i0 = vec * D + p; i1 = i0 + half; }
+        else { i0 = vec * D + 2 * p; i1 = i0 + 1; }
+        float a = elem<T>::ld(x + i0), b = elem<T>::ld(x + i1);
+        elem<T>::st(y + i0, a * cs - b * sn);
+        elem<T>::st(y + i1, b * cs + a * sn);
+    }
+}
+
+extern "C" int grl_rope(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x,
+                        const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling) {
+    GRL_REQUIRE(c && x && y, GRL_ERR_ARG, "grl_rope: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_rope: bad dtype %d", dtype);
+    GRL_REQUIRE(style == GRL_ROPE_HALF || style == GRL_ROPE_INTERLEAVED, GRL_ERR_ARG, "grl_rope: bad style %d", style);
+    GRL_REQUIRE(B >= 0 && S >= 0 && H >= 0 && D > 0 && D % 2 == 0 && D <= 128, GRL_ERR_SHAPE,
+                "grl_rope: head_dim must be even and <= 128 (got %lld)", (long long)D);
+    GRL_REQUIRE(rope_scaling != 0.f && rope_base > 0.f, GRL_ERR_ARG, "grl_rope: bad base/scaling");
+    GRL_REQUIRE(S < (1LL << 31) && H < (1LL << 31), GRL_ERR_SHAPE, "grl_rope: dimension too large");
+    int64_t pairs = B * S * H * (D / 2);
+    if (pairs == 0) return GRL_OK;
+    RopeFreq fr; grl_rope_freqs(&fr, (int)D, rope_base);
+    dim3 g(ew_grid(pairs)), b(256);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(rope_kernel<float>, g, b, 0, c->stream, (const float*)x, position_ids, (float*)y, pairs, (int)S, (int)H, (int)D, style, rope_scaling, fr);
+    else hipLaunchKernelGGL(rope_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, position_ids, (uint16_t*)y, pairs, (int)S, (int)H, (int)D, style, rope_scaling, fr);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+// cos/sin table (S, D/2) pairs for the fused-RoPE attention kernel, interleaved-style angle.
+__global__ __launch_bounds__(256) void rope_table_kernel(float2* __restrict__ tab, int S, int half, float scaling, RopeFreq fr) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= S * half) return;
+    int s = i / half, p = i - s * half;
+    float theta = ((float)s * fr.inv_freq[p]) / scaling;
+    float sn, cs;
+    sincosf(theta, &sn, &cs);
+    tab[i] = make_float2(cs, sn);
+}
+
+int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling) {
+    RopeFreq fr; grl_rope_freqs(&fr, D, base);
+    int n = S * (D / 2);
+    hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, c->stream, (float2*)tab, S, D / 2, scaling, fr);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+// ------------------------------------------------------------------ embedding gather
+template <typename T>
+__global__ __launch_bounds__(256) void embed_kernel(const int32_t* __restrict__ ids, const float* __restrict__ tok,
+                                                   const float* __restrict__ pos, const float* __restrict__ typ,
+                                                   T* __restrict__ x, int64_t rows, int S, int F, int vocab) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    int id = ids[row];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // the host validates; this only keeps loads in bounds
+    const int s = (int)(row % S);
+    const float* t = tok + (int64_t)id * F;
+    const float* p = pos + (int64_t)s * F;
+    T* o = x + row * (int64_t)F;
+    for (int f = lane; f < F; f += 64) elem<T>::st(o + f, t[f] + typ[f] + p[f]);
+}
+
+extern "C" int grl_embed(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F, int64_t vocab, const int32_t* ids,
+                         const float* tok_emb, const float* pos_emb, const float* type_emb, void* x) {
+    GRL_REQUIRE(c && ids && tok_emb && pos_emb && type_emb && x, GRL_ERR_ARG, "grl_embed: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_embed: bad dtype %d", dtype);
+    GRL_REQUIRE(B >= 0 && S > 0 && F > 0 && vocab > 0 && S < (1LL << 31) && F < (1LL << 31) && vocab < (1LL << 31),
+                GRL_ERR_SHAPE, "grl_embed: bad shape");
+    int64_t rows = B * S;
+    if (rows == 0) return GRL_OK;
+    dim3 g((unsigned)((rows + 3) / 4)), b(256);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(embed_kernel<float>, g, b, 0, c->stream, ids, tok_emb, pos_emb, type_emb, (float*)x, rows, (int)S, (int)F, (int)vocab);
+    else hipLaunchKernelGGL(embed_kernel<uint16_t>, g, b, 0, c->stream, ids, tok_emb, pos_emb, type_emb, (uint16_t*)x, rows, (int)S, (int)F, (int)vocab);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+// ------------------------------------------------------------------ masked mean pool (+ L2 normalise)
+// grid (ceil(F/256), B): thread f sums its feature over the sequence (coalesced across f).
+template <typename T>
+__global__ __launch_bounds__(256) void mean_pool_kernel(const T* __restrict__ x, const float* __restrict__ mask,
+                                                       float* __restrict__ out, int S, int F) {
+    const int f = blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = blockIdx.y;
+    if (f >= F) return;
+    float acc = 0.f, cnt = 0.f;
+    for (int s = 0; s < S; ++s) {
+        float m = mask ? mask[b * S + s] : 1.0f;
+        cnt += m;
+        acc += m * elem<T>::ld(x + (b * S + s) * (int64_t)F + f);
+    }
+    out[b * F + f] = acc / fmaxf(cnt, 1e-9f);
+}
+
+__global__ __launch_bounds__(256) void l2_normalize_kernel(float* __restrict__ v, int F) {
+    __shared__ float part[4];
+    float* r = v + (int64_t)blockIdx.x * F;
+    float s = 0.f;
+    for (int f = threadIdx.x; f < F; f += 256) s += r[f] * r[f];
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    float n = fmaxf(sqrtf(part[0] + part[1] + part[2] + part[3]), 1e-12f);
+    for (int f = threadIdx.x; f < F; f += 256) r[f] = r[f] / n;
+}
+
+extern "C" int grl_mean_pool(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F, const void* x,
+                             const float* mask, float* out, int l2_normalize) {
+    GRL_REQUIRE(c && x && out, GRL_ERR_ARG, "grl_mean_pool: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_mean_pool: bad dtype %d", dtype);
+    GRL_REQUIRE(B >= 0 && B < 65536 && S > 0 && F > 0 && S < (1LL << 31) && F < (1LL << 31), GRL_ERR_SHAPE, "grl_mean_pool: bad shape");
+    if (B == 0) return GRL_OK;
+    dim3 g((unsigned)((F + 255) / 256), (unsigned)B), b(256);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(mean_pool_kernel<float>, g, b, 0, c->stream, (const float*)x, mask, out, (int)S, (int)F);
+    else hipLaunchKernelGGL(mean_pool_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, mask, out, (int)S, (int)F);
+    GRL_CHECK_LAUNCH();
+    if (l2_normalize) {
+        hipLaunchKernelGGL(l2_normalize_kernel, dim3((unsigned)B), dim3(256), 0, c->stream, out, (int)F);
+        GRL_CHECK_LAUNCH();
+    }
+    return GRL_OK;
+}
+
+// ------------------------------------------------------------------ 2-D transpose (for gemm_nn)
+// in (R,C) row-major -> out (C,R); 64x64 tiles through LDS, one extra column against bank conflicts.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t R, int64_t C) {
+    __shared__ T tile[64][65];
+    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int j = ty; j < 64; j += 4)
+        if (r0 + j < R && c0 + tx < C) tile[j][tx] = in[(r0 + j) * C + c0 + tx];
+    __syncthreads();
+    for (int j = ty; j < 64; j += 4)
+        if (c0 + j < C && r0 + tx < R) out[(c0 + j) * R + r0 + tx] = tile[tx][j];
+}
+
+int grl_transpose2d(grl_ctx* c, int dtype, int64_t R, int64_t C, const void* in, void* out) {
+    dim3 g((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64)), b(256);
+    GRL_REQUIRE(g.y < 65536, GRL_ERR_SHAPE, "transpose: too many rows (%lld)", (long long)R);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(transpose_kernel<float>, g, b, 0, c->stream, (const float*)in, (float*)out, R, C);
+    else hipLaunchKernelGGL(transpose_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)in, (uint16_t*)out, R, C);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}

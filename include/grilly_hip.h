@@ -1,0 +1,219 @@
+/*
+ * grilly_hip.h -- C ABI of libgrilly_hip.so: the gfx950 (MI355X) implementation of
+ * grilly's transformer-forward hot path.
+ *
+ * Every launcher works on DEVICE pointers obtained from grl_malloc (or any hipMalloc'd
+ * memory), enqueues on the context's HIP stream and returns immediately; grl_sync()
+ * waits.  All functions return 0 on success or a negative grl_status; the message of
+ * the last failure on the calling thread is returned by grl_last_error().  There is no
+ * CPU fallback anywhere behind this interface.
+ *
+ * Each entry point names the reference (Grillcheese-AI/grilly) interface it stands in
+ * for as  file:line .  The reference drives GLSL compute shaders through Vulkan from
+ * Python; a binding for it is therefore a ctypes stub (see grilly_amd/_lib.py).
+ *
+ * Conventions shared by all launchers
+ *   - tensors are dense, row-major, C-contiguous; sizes are element counts
+ *   - grl_dtype selects the storage type of activations/weights: GRL_F32 or GRL_BF16
+ *     (bfloat16, round-to-nearest-even); accumulation and statistics are always fp32
+ *   - bias / gamma / beta vectors are always fp32
+ *   - "weights (N,K)" means the reference's (out_features, in_features) layout
+ */
+#ifndef GRILLY_HIP_H
+#define GRILLY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct grl_ctx grl_ctx;
+
+typedef enum grl_status {
+    GRL_OK = 0,
+    GRL_ERR_ARG = -1,         /* null pointer, bad enum, non-positive size */
+    GRL_ERR_SHAPE = -2,       /* shape the kernels do not cover (message says which) */
+    GRL_ERR_HIP = -3,         /* a HIP runtime call failed */
+    GRL_ERR_OOM = -4          /* device allocation failed */
+} grl_status;
+
+typedef enum grl_dtype { GRL_F32 = 0, GRL_BF16 = 1 } grl_dtype;
+
+/* epilogue applied to (x.W^T + bias) inside the GEMM kernel, on the fp32 accumulator */
+typedef enum grl_epilogue {
+    GRL_EPI_NONE = 0,
+    GRL_EPI_GELU = 1,   /* tanh GELU with the +-50 clamp rule of shaders/fused-linear-gelu.glsl:45-63 */
+    GRL_EPI_SILU = 2    /* s/(1+exp(-clamp(s,-88,88))), shaders/fused-linear-silu.glsl:43-48 */
+} grl_epilogue;
+
+typedef enum grl_rope_style { GRL_ROPE_NONE = 0, GRL_ROPE_INTERLEAVED = 1, GRL_ROPE_HALF = 2 } grl_rope_style;
+
+typedef struct grl_devinfo {
+    char name[128];
+    char arch[64];
+    int32_t compute_units;
+    int32_t clock_khz;
+    int32_t lds_bytes_per_block;
+    int32_t wavefront;
+    int64_t hbm_bytes;
+} grl_devinfo;
+
+typedef struct grl_pool_stats {
+    int64_t allocations;      /* hipMalloc calls made by the pool */
+    int64_t hits;             /* grl_malloc calls served from a cached block */
+    int64_t misses;           /* grl_malloc calls that had to allocate */
+    int64_t bytes_in_use;
+    int64_t bytes_cached;
+    int64_t bytes_peak;
+} grl_pool_stats;
+
+/* ---- context / runtime --------------------------------------------------------
+ * Replaces VulkanCore (backend/core.py:17-166 create, :423-439 cleanup) and
+ * VulkanPipelines (backend/pipelines.py:97-130): one context = one device + one stream. */
+grl_ctx*    grl_create(int device);
+void        grl_destroy(grl_ctx* ctx);
+const char* grl_last_error(void);
+int         grl_device_info(grl_ctx* ctx, grl_devinfo* out);
+/* the hipStream_t of the context, for callers that record their own events on it */
+void*       grl_stream(grl_ctx* ctx);
+
+/* Device buffers from a power-of-two bucketed caching pool.
+ * Replaces VulkanCore._create_buffer (backend/core.py:304-335) and
+ * BufferPool.acquire/release/get_stats (backend/buffer_pool.py:534-579, 627-640). */
+void* grl_malloc(grl_ctx* ctx, size_t bytes);
+int   grl_free(grl_ctx* ctx, void* ptr);
+int   grl_pool_get_stats(grl_ctx* ctx, grl_pool_stats* out);
+int   grl_pool_trim(grl_ctx* ctx);     /* return cached blocks to the driver */
+
+/* Host <-> device copies (blocking), replacing _upload_buffer / _download_buffer
+ * (backend/core.py:345-360).  grl_sync replaces vkQueueWaitIdle (backend/core.py:418). */
+int grl_h2d(grl_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
+int grl_d2h(grl_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
+int grl_d2d(grl_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes);
+int grl_memset(grl_ctx* ctx, void* dst_dev, int byte, size_t bytes);
+int grl_sync(grl_ctx* ctx);
+
+/* HIP-event stopwatch on the context stream (there is no counterpart in the reference,
+ * which times whole numpy->numpy calls with time.perf_counter). */
+int grl_timer_start(grl_ctx* ctx);
+int grl_timer_stop(grl_ctx* ctx, float* elapsed_ms);   /* synchronises */
+
+/* fp32 <-> bf16 conversion on the device (RNE).  No reference counterpart: the
+ * reference is fp32 only. */
+int grl_cast(grl_ctx* ctx, int src_dtype, int dst_dtype, int64_t n, const void* src, void* dst);
+
+/* ---- GEMM family ---------------------------------------------------------------
+ * C[m,n] = epi( sum_k A[m,k] * W[n,k] + bias[n] )      A (M,K), W (N,K), C (M,N)
+ * Replaces VulkanFNN.linear (backend/fnn.py:1394-1496, shaders/fnn-linear.glsl:33-58),
+ * VulkanFNN.fused_linear_gelu (backend/fnn.py:2022-2123, shaders/fused-linear-gelu.glsl:42-93),
+ * VulkanFNN.fused_linear_silu (backend/fnn.py:2214-2303, shaders/fused-linear-silu.glsl:42-78)
+ * and, with N = 3*H*D and packed [Wq;Wk;Wv], shaders/fused-qkv-projection.glsl:48-74.
+ * in_dtype is the type of A and W, out_dtype the type of C; bias may be NULL. */
+int grl_gemm_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                const void* A, const void* W, const float* bias, void* C, int epilogue);
+
+/* C = A.B with B (K,N) row-major.  Replaces VulkanFNN.gemm (backend/fnn.py:104-166,
+ * shaders/gemm_mnk.glsl:35-88).  workspace must hold K*N elements of in_dtype (the
+ * kernel transposes B once); pass NULL to let the context allocate it from its pool. */
+int grl_gemm_nn(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                const void* A, const void* B, void* C, void* workspace);
+
+/* out[m,n] = (x.Wg^T + bg)[m,n] * silu((x.Wu^T + bu)[m,n]),  silu(u) = u/(1+exp(-u)).
+ * Replaces fused_swiglu (backend/_glu_append.py:8-129, shaders/fused-swiglu.glsl:43-79).
+ * Biases are applied only when both are given, as in the reference (_glu_append.py:68).
+ * gate_cache / up_cache (fp32, (M,N)) receive the pre-activations when non-NULL. */
+int grl_swiglu_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                  const void* x, const void* W_gate, const void* W_up,
+                  const float* b_gate, const float* b_up, void* out,
+                  float* gate_cache, float* up_cache);
+
+/* ---- attention -------------------------------------------------------------------
+ * O[b,i,h,:] = sum_j softmax_j( scale*<Q'[b,i,h],K'[b,j,h]> + (mask[b,j]-1)*1e9 ) V[b,j,h,:]
+ * with Q',K' optionally rotated (RoPE) and, if causal, keys j>i excluded.
+ * Layout of Q,K,V,O: (B,S,H,D).  mask: fp32 (B,S), 1 keep / 0 drop, or NULL.
+ * Replaces VulkanAttention.flash_attention2 (backend/attention.py:361-597; contract in
+ * its docstring :374-395; constants of shaders/flash-attention2.glsl:95,152,214) and
+ * shaders/flash-attention2-rope.glsl:73-148 (interleaved pairs, theta =
+ * pos*base^(-2p/D)/scaling); causal rule of shaders/attention-mask.glsl:42-46.
+ * D must be 32, 64 or 128.  GRL_ROPE_HALF uses the (d, d+D/2) pairing of
+ * shaders/rope.glsl:74-125 and needs a workspace of 2*B*S*H*D elements (NULL = pool). */
+int grl_fa2_fwd(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                const void* Q, const void* K, const void* V, const float* mask, void* O,
+                float scale, int causal, int rope, float rope_base, float rope_scaling,
+                void* workspace);
+
+/* Same as grl_fa2_fwd with explicit position strides (elements between consecutive sequence
+ * positions of one batch entry), so Q, K and V can be the three column blocks of the packed
+ * (B*S, 3*H*D) output of the fused QKV projection (shaders/fused-qkv-projection.glsl:58-70)
+ * without a split copy.  Rotate-half RoPE is not offered here. */
+int grl_fa2_fwd_strided(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                        const void* Q, const void* K, const void* V, const float* mask, void* O,
+                        int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                        float scale, int causal, int rope, float rope_base, float rope_scaling);
+
+/* y = rotate(x) for x (B,S,H,D); position_ids int32 (B,S) or NULL for 0..S-1.
+ * Replaces VulkanAttention.apply_rope (backend/attention.py:599-676, _rope_cpu :795-835,
+ * shaders/rope.glsl:74-125) for style GRL_ROPE_HALF; GRL_ROPE_INTERLEAVED follows
+ * shaders/flash-attention2-rope.glsl:84-90,122-137. */
+int grl_rope(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+             const void* x, const int32_t* position_ids, void* y,
+             int style, float rope_base, float rope_scaling);
+
+/* ---- bandwidth-bound row / element kernels ------------------------------------------
+ * y = gamma*(t-mean)/sqrt(var+eps)+beta per row of F features, t = x (+ residual if given),
+ * biased variance, two-pass statistics in fp32.
+ * Replaces VulkanFNN.layernorm (backend/fnn.py:1285-1389, shaders/fnn-layernorm.glsl:44-103);
+ * the optional residual folds VulkanFNN.residual (backend/fnn.py:1950-2014) into the same
+ * pass, which is how the encoder uses the pair (utils/vulkan_sentence_transformer.py:1004,1026). */
+int grl_layernorm(grl_ctx* ctx, int dtype, int64_t rows, int64_t F, const void* x,
+                  const void* residual, const float* gamma, const float* beta, float eps, void* y);
+
+/* out = a + b.  Replaces VulkanFNN.residual (shaders/fnn-residual.glsl:25-34). */
+int grl_add(grl_ctx* ctx, int dtype, int64_t n, const void* a, const void* b, void* out);
+/* Replaces VulkanFNN.activation_gelu (backend/fnn.py:285-342, shaders/activation-gelu.glsl:23-53). */
+int grl_gelu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
+/* Replaces VulkanFNN.activation_silu (backend/fnn.py:344-391): x*sigmoid(x). */
+int grl_silu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
+/* x (rows, 2h) -> y (rows, h): x1*(x2*sigmoid(x2)), x1 first half.
+ * Replaces VulkanFNN.activation_swiglu (backend/fnn.py:499-572, shaders/activation-swiglu.glsl:21-52). */
+int grl_swiglu_act(grl_ctx* ctx, int dtype, int64_t rows, int64_t h, const void* x, void* y);
+
+/* ---- encoder pre/post steps ------------------------------------------------------------
+ * x[b,s,:] = tok_emb[ids[b,s]] + pos_emb[s] + type_emb[0]   (tables fp32, x of `dtype`).
+ * Replaces the embedding steps of VulkanSentenceTransformer
+ * (utils/vulkan_sentence_transformer.py:563-707). */
+int grl_embed(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t F, int64_t vocab,
+              const int32_t* ids, const float* tok_emb, const float* pos_emb,
+              const float* type_emb, void* x);
+/* out[b,:] = sum_s mask[b,s]*x[b,s,:] / max(sum_s mask[b,s], 1e-9), optionally L2-normalised
+ * (x / max(||x||, 1e-12)); out fp32 (B,F).
+ * Replaces mean pooling + normalise of encode (utils/vulkan_sentence_transformer.py:1177-1201). */
+int grl_mean_pool(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t F, const void* x,
+                  const float* mask, float* out, int l2_normalize);
+
+/* ---- one post-LN BERT encoder layer, device resident ----------------------------------------
+ * x <- LN(x + Wo.Attn(QKV(x); mask) + bo; g1,b1,eps); x <- LN(x + W2.gelu(W1.x+b1)+b2; g2,b2,eps)
+ * Replaces VulkanSentenceTransformer._forward_layer, BERT branch
+ * (utils/vulkan_sentence_transformer.py:972-1035) with the fused QKV projection.
+ * Weights are (out,in) matrices of `dtype`; biases and LN parameters fp32.
+ * workspace: at least grl_bert_layer_workspace(...) bytes. */
+typedef struct grl_bert_layer {
+    const void*  w_qkv;  const float* b_qkv;     /* (3*H*D, d_model), (3*H*D) */
+    const void*  w_o;    const float* b_o;       /* (d_model, H*D) */
+    const float* ln1_g;  const float* ln1_b;
+    const void*  w_ff1;  const float* b_ff1;     /* (d_ff, d_model) */
+    const void*  w_ff2;  const float* b_ff2;     /* (d_model, d_ff) */
+    const float* ln2_g;  const float* ln2_b;
+} grl_bert_layer;
+
+int64_t grl_bert_layer_workspace(int dtype, int64_t B, int64_t S, int64_t H, int64_t D, int64_t d_ff);
+int grl_bert_layer_fwd(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                       int64_t d_ff, const grl_bert_layer* w, const float* mask, float eps,
+                       void* x, void* workspace);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GRILLY_HIP_H */
