@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Headline benchmark: BERT-base-shaped encoder forward (12 post-LN layers, d=768, 12x64 heads,
+FFN 3072 GELU, fused QKV) at batch 128 x seq 512, bf16 storage with fp32 accumulation, on ONE
+MI355X.  A step = one full forward over one synthetic batch already resident in HBM.
+
+Prints one JSON line: encoder tokens/s, plus
+  roofline     -- the dominant kernel (the bf16 MFMA GEMM): algorithmic FLOPs per launch divided
+                  by its average launch duration, measured here with HIP events on the library's
+                  own stream, against the 2.5 PFLOP/s dense bf16 MFMA peak;
+  kernels      -- the same measurement for every kernel of the layer (GEMMs and attention against
+                  the MFMA peak, LayerNorm against 8 TB/s HBM);
+  cpu_baseline -- the C restatement of the reference shaders (oracle/oracle.c) timed on the host
+                  cores on a bounded sample (one sequence through all 12 layers).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16 = 2.5e15      # MI355X dense bf16 MFMA, FLOP/s
+PEAK_FP32 = 157.3e12
+PEAK_HBM = 8.0e12       # B/s
+
+
+def time_launches(core, fn, reps, warm=3):
+    """average milliseconds of one call of fn() (which only enqueues), HIP events on the context stream"""
+    for _ in range(warm):
+        fn()
+    core.sync()
+    core.timer_start()
+    for _ in range(reps):
+        fn()
+    return core.timer_stop() / reps
+
+
+def kernel_table(backend, enc, B, S, reps):
+    """per-kernel average duration of one encoder layer's launches at the benchmark shape"""
+    from grilly_amd import _lib as L
+    cfg, c, lib, code = enc.cfg, backend.core, backend.core.lib, enc.code
+    M, d, ff, H, D = B * S, cfg.d_model, cfg.d_ff, cfg.heads, cfg.head_dim
+    es = 2 if code == L.GRL_BF16 else 4
+    s = enc.layer_structs[0]
+    qkv, attn, ffb = c.alloc(M * 3 * d * es), c.alloc(M * d * es), c.alloc(M * ff * es)
+    proj = c.alloc(M * d * es)
+    x = enc.x
+    peak = PEAK_BF16 if code == L.GRL_BF16 else PEAK_FP32
+    scale = 1.0 / np.sqrt(D)
+    runs = [
+        ("gemm_qkv", "gemm_nt", lambda: lib.grl_gemm_nt(c.ctx, code, code, M, 3 * d, d, x.ptr, s.w_qkv, s.b_qkv, qkv.ptr, 0),
+         2.0 * M * 3 * d * d, (M * d + 3 * d * d + M * 3 * d) * es),
+        ("gemm_out", "gemm_nt", lambda: lib.grl_gemm_nt(c.ctx, code, code, M, d, d, attn.ptr, s.w_o, s.b_o, proj.ptr, 0),
+         2.0 * M * d * d, (2 * M * d + d * d) * es),
+        ("gemm_ffn2", "gemm_nt", lambda: lib.grl_gemm_nt(c.ctx, code, code, M, d, ff, ffb.ptr, s.w_ff2, s.b_ff2, proj.ptr, 0),
+         2.0 * M * d * ff, (M * ff + d * ff + M * d) * es),
+        ("gemm_ffn1_gelu", "gemm_nt_gelu", lambda: lib.grl_gemm_nt(c.ctx, code, code, M, ff, d, x.ptr, s.w_ff1, s.b_ff1, ffb.ptr, 1),
+         2.0 * M * d * ff, (M * d + d * ff + M * ff) * es),
+        ("fa2_fwd", "fa2", lambda: lib.grl_fa2_fwd_strided(c.ctx, code, B, S, H, D, qkv.ptr, qkv.ptr + d * es, qkv.ptr + 2 * d * es,
+                                                           None, attn.ptr, 3 * d, 3 * d, 3 * d, d, scale, 0, 0, 1e4, 1.0),
+         4.0 * B * H * S * S * D, 4 * M * d * es),
+        ("layernorm_residual", "ln", lambda: lib.grl_layernorm(c.ctx, code, M, d, x.ptr, proj.ptr, s.ln1_g, s.ln1_b, cfg.eps, attn.ptr),
+         0.0, 3 * M * d * es),
+    ]
+    out = {}
+    for name, group, fn, flops, nbytes in runs:
+        ms = time_launches(c, fn, reps)
+        rec = {"ms": round(ms, 4), "group": group, "flops": flops, "bytes": nbytes}
+        if flops:
+            rec["tflops"] = round(flops / ms / 1e9, 1)
+            rec["frac_mfma"] = round(flops / (ms * 1e-3) / peak, 4)
+        rec["gbps"] = round(nbytes / ms / 1e6, 1)
+        rec["frac_hbm"] = round(nbytes / (ms * 1e-3) / PEAK_HBM, 4)
+        out[name] = rec
+    for b in (qkv, attn, ffb, proj):
+        b.free()
+    return out
+
+
+def cpu_baseline(cfg, weights, seed):
+    """C restatement of the reference shaders on the host cores: ONE sequence of the workload
+    (S=512) through embeddings + all layers.  tokens/s = 512 / elapsed."""
+    from oracle import oracle_np as O
+    O.build()
+    C = O.COracle()
+    rng = np.random.default_rng(seed)
+    S = 512
+    ids = rng.integers(0, cfg.vocab, (1, S))
+    t0 = time.perf_counter()
+    x = C.layernorm(C.embed(ids, weights["tok_emb"], weights["pos_emb"], weights["type_emb"]),
+                    weights["emb_ln_g"], weights["emb_ln_b"], cfg.eps)
+    for lw in weights["layers"]:
+        x = C.bert_layer(x, lw, None, cfg.heads, cfg.eps)
+    dt = time.perf_counter() - t0
+    return {"value": round(S / dt, 2), "unit": "tokens/s", "cores": C.num_threads(), "kind": "port",
+            "sample": f"1 sequence x {S} tokens through embeddings + {cfg.layers} layers, fp32, "
+                      f"oracle/oracle.c (one-output-per-invocation shader loops, OpenMP over rows); {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--seq", type=int, default=512)
+    ap.add_argument("--kernel-reps", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one MI355X: this path has no multi-GPU leg (data-parallel sharding over "
+                 "batch needs no exchange; see DESIGN.md).  Run with --gpus 1.")
+
+    import grilly_amd
+    from grilly_amd import BertEncoder, random_bert_weights
+    from grilly_amd.encoder import BERT_BASE as cfg
+
+    seed = 20260131 + 3
+    backend = grilly_amd.Compute(0)
+    info = backend.device_info()
+    weights = random_bert_weights(cfg, seed=seed)
+    enc = BertEncoder(backend, cfg, weights, dtype=a.dtype)
+    rng = np.random.default_rng(seed)
+    B, S = a.batch, a.seq
+    ids = rng.integers(0, cfg.vocab, (B, S))
+    enc.set_inputs(ids, None)                 # no padding in this configuration
+
+    for _ in range(a.warmup):
+        enc.launch(pool=True)
+    backend.core.sync()
+    t0 = time.perf_counter()
+    backend.core.timer_start()
+    for _ in range(a.steps):
+        enc.launch(pool=True)
+    ev_ms = backend.core.timer_stop()         # records the stop event and waits for it
+    backend.core.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / a.steps
+    tokens_per_s = B * S * a.steps / wall
+    flops = enc.flops_per_forward(B, S)
+
+    out = {
+        "metric": "encoder tokens/s (BERT-base, L=512)", "value": round(tokens_per_s, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.dtype, "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2]: BERT-base-shaped encoder forward, 12 post-LN layers, d=768, "
+                               "12x64 heads, FFN 3072 GELU, fused QKV, no padding, random init N(0,0.02)",
+                   "batch": B, "seq_len": S, "tokens_per_step": B * S, "flops_per_step": flops},
+        "event_ms_per_step": round(ev_ms / a.steps, 3),
+        "model_tflops": round(flops / (ms_per_step * 1e-3) / 1e12, 1),
+        "device": info,
+    }
+    peak = PEAK_BF16 if a.dtype == "bf16" else PEAK_FP32
+    if not a.no_kernels:
+        kt = kernel_table(backend, enc, B, S, a.kernel_reps)
+        out["kernels"] = kt
+        # dominant kernel = the plain (no activation) GEMM instantiation, launched three times per layer
+        # (QKV, out-proj, FFN2): average FLOPs per launch over average duration per launch
+        g = [kt[k] for k in ("gemm_qkv", "gemm_out", "gemm_ffn2")]
+        avg_flops = sum(r["flops"] for r in g) / 3
+        avg_ms = sum(r["ms"] for r in g) / 3
+        ach = avg_flops / (avg_ms * 1e-3) / 1e12
+        out["roofline"] = {"kernel": "gemm_nt_kernel<bf16,bf16,256,256,2,2,EPI_NONE>" if a.dtype == "bf16" else "gemm_nt_kernel<f32,f32,256,256,2,2,EPI_NONE>",
+                           "bound": "mfma", "achieved": round(ach, 1), "peak": peak / 1e12, "unit": "TFLOP/s",
+                           "frac": round(ach * 1e12 / peak, 4), "traffic": None,
+                           "avg_launch_ms": round(avg_ms, 4), "flops_per_launch": avg_flops,
+                           "launches_per_step": 3 * cfg.layers}
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, weights, seed)
+    backend.cleanup()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

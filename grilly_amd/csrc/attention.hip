@@ -51,7 +51,7 @@ template <> struct Slab<float> {
     static __device__ __forceinline__ void run(const u32x4& a, const u32x4& b, f32x16& acc) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a[e]), __builtin_bit_cast(float, b[e]), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u2f(a[e]), u2f(b[e]), acc, 0, 0, 0);
     }
 };
 
@@ -61,7 +61,7 @@ template <> __device__ __forceinline__ u32x4 rope_chunk<float>(u32x4 v, const fl
     u32x4 o;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        float x0 = __builtin_bit_cast(float, v[2 * i]), x1 = __builtin_bit_cast(float, v[2 * i + 1]);
+        float x0 = u2f(v[2 * i]), x1 = u2f(v[2 * i + 1]);
         o[2 * i] = __builtin_bit_cast(uint32_t, x0 * cs[i].x - x1 * cs[i].y);
         o[2 * i + 1] = __builtin_bit_cast(uint32_t, x0 * cs[i].y + x1 * cs[i].x);
     }

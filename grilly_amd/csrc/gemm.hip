@@ -65,7 +65,7 @@ template <> struct MfmaSlab<float> {      // fp32: 16 B = 4 values, each feeds o
     static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, w[e]), __builtin_bit_cast(float, x[e]), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u2f(w[e]), u2f(x[e]), acc, 0, 0, 0);
     }
 };
 

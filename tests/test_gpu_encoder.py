@@ -1,0 +1,98 @@
+"""GPU parity of the encoder forward (post-LN BERT layer recipe of the reference's
+VulkanSentenceTransformer) against the float64 oracle of the same recipe."""
+import numpy as np
+import pytest
+
+from conftest import TOL_F32, TOL_BF16, rng_for
+from oracle import oracle_np as O
+from grilly_amd import BertEncoder, EncoderConfig, random_bert_weights
+
+pytestmark = pytest.mark.gpu
+
+
+def truth_encoder(w, cfg, ids, mask, quant=None):
+    qf = (lambda a: a) if quant is None else (lambda a: quant(np.asarray(a, np.float32)).astype(np.float64))
+    wq = lambda a: a if quant is None else quant(a)
+    x = qf(O.truth_embed(ids, w["tok_emb"], w["pos_emb"], w["type_emb"]))
+    x = qf(O.truth_layernorm(x, w["emb_ln_g"], w["emb_ln_b"], cfg.eps))
+    for lw in w["layers"]:
+        lw = {k: (wq(v) if k.startswith("w_") else v) for k, v in lw.items()}
+        x = O.truth_bert_layer(x, lw, mask, cfg.heads, cfg.eps, quant)
+    return x
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_small_encoder_parity(backend, dtype):
+    cfg = EncoderConfig(layers=2, d_model=128, heads=4, d_ff=512, vocab=500, max_pos=64)
+    w = random_bert_weights(cfg, seed=3)
+    rng = np.random.default_rng(3)
+    for lw in w["layers"]:      # non-trivial biases and LayerNorm parameters
+        for k in ("b_qkv", "b_o", "b_ff1", "b_ff2", "ln1_b", "ln2_b"):
+            lw[k] = (rng.standard_normal(lw[k].shape) * 0.05).astype(np.float32)
+        for k in ("ln1_g", "ln2_g"):
+            lw[k] = (1 + rng.standard_normal(lw[k].shape) * 0.05).astype(np.float32)
+    B, S = 2, 16
+    ids = rng.integers(0, cfg.vocab, (B, S))
+    mask = (np.arange(S)[None] < np.array([16, 9])[:, None]).astype(np.float32)
+    enc = BertEncoder(backend, cfg, w, dtype=dtype)
+    h = enc.forward(ids, mask, pool=False)
+    quant = O.bf16_round if dtype == "bf16" else None
+    ref = truth_encoder(w, cfg, ids, mask, quant)
+    assert h.shape == (B, S, cfg.d_model)
+    assert O.max_rel(h, ref) < (TOL_F32 if dtype == "fp32" else TOL_BF16)
+    pooled = enc.forward(ids, mask, pool=True)
+    assert O.max_rel(pooled, O.truth_mean_pool(h, mask)) < 1e-4
+    np.testing.assert_allclose(np.linalg.norm(pooled, axis=1), 1.0, atol=1e-5)
+    with pytest.raises(IndexError):
+        enc.forward(np.full((1, 4), cfg.vocab), None)
+    with pytest.raises(ValueError):
+        enc.forward(np.zeros((1, 65), np.int64), None)
+
+
+def test_minilm_shaped_encoder_fp32(backend, corc):
+    # BASELINE config 2 architecture (6 post-LN layers, d=384, 12x32, FFN 1536, GELU, fp32, padding mask
+    # with lengths in [32,256], vocab 30522) at reduced batch so the CPU oracle finishes in seconds
+    from grilly_amd.encoder import MINILM_L6 as cfg
+    w = random_bert_weights(cfg, seed=20260133)
+    rng = rng_for(2)
+    B, S = 2, 256
+    ids = rng.integers(0, cfg.vocab, (B, S))
+    lens = rng.integers(32, 257, B)
+    mask = (np.arange(S)[None] < lens[:, None]).astype(np.float32)
+    enc = BertEncoder(backend, cfg, w, dtype="fp32")
+    h = enc.forward(ids, mask, pool=False)
+    # C oracle (fp32 shader order), layer by layer
+    x = corc.layernorm(corc.embed(ids, w["tok_emb"], w["pos_emb"], w["type_emb"]), w["emb_ln_g"], w["emb_ln_b"], cfg.eps)
+    for lw in w["layers"]:
+        x = corc.bert_layer(x, lw, mask, cfg.heads, cfg.eps)
+    assert O.max_rel(h, x) < TOL_F32
+    assert O.max_rel(h, truth_encoder(w, cfg, ids, mask)) < TOL_F32
+
+
+def test_bert_base_layer_bf16_full_width(backend):
+    # BASELINE config 3 architecture (d=768, 12x64, FFN 3072, fused QKV), one layer at full width, reduced batch
+    cfg = EncoderConfig(layers=1)
+    w = random_bert_weights(cfg, seed=20260134)
+    rng = rng_for(3)
+    B, S = 2, 512
+    ids = rng.integers(0, cfg.vocab, (B, S))
+    enc = BertEncoder(backend, cfg, w, dtype="bf16")
+    h = enc.forward(ids, None, pool=False)
+    ref = truth_encoder(w, cfg, ids, None, O.bf16_round)
+    assert O.max_rel(h, ref) < TOL_BF16
+    # post-LN with gamma=1, beta=0: every row has mean 0 and variance ~1
+    assert np.abs(h.mean(-1)).max() < 2e-2 and np.abs(h.var(-1) - 1).max() < 5e-2
+
+
+def test_encoder_batch_independence_full_config(backend):
+    # full BERT-base depth (12 layers) in bf16: sequences are independent, so a batch run equals per-sequence runs
+    cfg = EncoderConfig()
+    w = random_bert_weights(cfg, seed=1)
+    rng = np.random.default_rng(1)
+    ids = rng.integers(0, cfg.vocab, (3, 512))
+    enc = BertEncoder(backend, cfg, w, dtype="bf16")
+    full = enc.forward(ids, None, pool=True)
+    one = enc.forward(ids[1:2], None, pool=True)
+    assert np.isfinite(full).all()
+    np.testing.assert_allclose(full[1:2], one, atol=2e-3)
+    np.testing.assert_allclose(np.linalg.norm(full, axis=1), 1.0, atol=1e-4)

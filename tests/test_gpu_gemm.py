@@ -1,0 +1,195 @@
+"""GPU parity of the GEMM family against the oracle (float64 closed form of the reference
+shaders), called through the numpy facade which goes through the C ABI.
+Tolerances: max|y-ref|/max|ref| <= 1e-4 on the fp32 path, <= 2e-2 on the bf16 path."""
+import numpy as np
+import pytest
+
+from conftest import TOL_F32, TOL_BF16, rng_for
+from oracle import oracle_np as O
+
+pytestmark = pytest.mark.gpu
+
+
+def tol(dtype):
+    return TOL_F32 if dtype == "fp32" else TOL_BF16
+
+
+def prep(dtype, *arrs):
+    """the bf16 path's oracle consumes the bf16-rounded inputs"""
+    return [O.bf16_round(a) if dtype == "bf16" else a for a in arrs]
+
+
+SHAPES = [
+    (32, 384, 128),      # BASELINE config 1
+    (1, 8, 4), (3, 16, 5), (33, 40, 17), (64, 128, 256),      # reference test_gemm_backward shape + ragged edges
+    (130, 264, 250), (257, 72, 513), (300, 2056, 129),
+    (1024, 384, 1536),   # MiniLM FFN1 slice
+    (2048, 768, 768), (4096, 768, 2304),                      # BERT-base out-proj / QKV (big-tile kernel)
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_linear_parity(backend, dtype, M, K, N):
+    rng = np.random.default_rng(M * 7 + K * 3 + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    W = rng.standard_normal((N, K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    x, W = prep(dtype, x, W)
+    y = backend.fnn.linear(x, W, b, dtype=dtype)
+    assert y.shape == (M, N) and y.dtype == np.float32 and y.flags.c_contiguous
+    assert O.max_rel(y, O.truth_linear(x, W, b)) < tol(dtype)
+    y0 = backend.fnn.linear(x, W, dtype=dtype)
+    assert O.max_rel(y0, O.truth_linear(x, W)) < tol(dtype)
+
+
+def test_config1_linear_then_swiglu(backend, corc):
+    # BASELINE config 1: x[32,384].W[384,128]+b (W given as (in,out) -> passed transposed), then swiglu
+    rng = rng_for(1)
+    x = rng.standard_normal((32, 384)).astype(np.float32)
+    W = rng.standard_normal((384, 128)).astype(np.float32)
+    b = np.zeros(128, np.float32)
+    y = backend.fnn.linear(x, W.T.copy(), b)
+    assert O.max_rel(y, x.astype(np.float64) @ W.astype(np.float64)) < TOL_F32
+    assert O.max_rel(y, corc.linear(x, W.T.copy(), b)) < TOL_F32          # shader-order fp32 restatement
+    z = backend.fnn.activation_swiglu(y)
+    assert z.shape == (32, 64)
+    assert O.max_rel(z, O.truth_swiglu_act(y)) < TOL_F32
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("epi", ["gelu", "silu"])
+@pytest.mark.parametrize("M,K,N", [(5, 24, 7), (129, 136, 260), (2048, 768, 3072)])
+def test_fused_linear_parity(backend, dtype, epi, M, K, N):
+    rng = np.random.default_rng(11 + M + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    W = (rng.standard_normal((N, K)) * 0.2).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    x, W = prep(dtype, x, W)
+    fn = backend.fnn.fused_linear_gelu if epi == "gelu" else backend.fnn.fused_linear_silu
+    y = fn(x, W, b, dtype=dtype)
+    assert O.max_rel(y, O.truth_linear(x, W, b, epi)) < tol(dtype)
+
+
+def test_fused_epilogue_clamp_edges(backend):
+    # drive the pre-activation to the +-50 (gelu) and +-88 (silu) edges through a 1-wide GEMM
+    s = np.array([0.0, 1.0, -1.0, 49.5, 50.5, -49.5, -50.5, 87.0, 89.0, -87.0, -89.0, -120.0, 300.0], np.float32)
+    x = np.zeros((len(s), 8), np.float32); x[:, 0] = s
+    W = np.zeros((4, 8), np.float32); W[:, 0] = 1
+    g = backend.fnn.fused_linear_gelu(x, W)
+    np.testing.assert_allclose(g[:, 0], O.truth_gelu(s), rtol=1e-5, atol=1e-6)
+    assert g[0, 0] == 0.0 and g[4, 0] == 50.5 and g[6, 0] == 0.0
+    si = backend.fnn.fused_linear_silu(x, W)
+    np.testing.assert_allclose(si[:, 0], O.truth_silu_clamped(s), rtol=1e-5, atol=1e-30)
+    ga = backend.fnn.activation_gelu(s)
+    np.testing.assert_allclose(ga, O.truth_gelu(s), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("M,K,N,bias", [(6, 20, 10, True), (70, 72, 33, False), (513, 264, 130, True), (2048, 512, 1408, False)])
+def test_fused_swiglu_parity(backend, dtype, M, K, N, bias):
+    rng = np.random.default_rng(M + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    Wg = (rng.standard_normal((N, K)) * 0.1).astype(np.float32)
+    Wu = (rng.standard_normal((N, K)) * 0.1).astype(np.float32)
+    bg = rng.standard_normal(N).astype(np.float32) if bias else None
+    bu = rng.standard_normal(N).astype(np.float32) if bias else None
+    x, Wg, Wu = prep(dtype, x, Wg, Wu)
+    t_out, t_g, t_u = O.truth_fused_swiglu(x, Wg, Wu, bg, bu)
+    out, g, u = backend.fnn.fused_swiglu(x, Wg, Wu, bg, bu, return_cache=True, dtype=dtype)
+    assert out.shape == (M, N)
+    assert O.max_rel(out, t_out) < tol(dtype)
+    assert O.max_rel(g, t_g) < tol(dtype) and O.max_rel(u, t_u) < tol(dtype)
+    out2 = backend.fnn.fused_swiglu(x, Wg, Wu, bg, bu, dtype=dtype)
+    np.testing.assert_array_equal(out2, out)          # deterministic, cache stores do not disturb the result
+    # a single bias is ignored, as in the reference
+    np.testing.assert_array_equal(backend.fnn.fused_swiglu(x, Wg, Wu, bg, None, dtype=dtype),
+                                  backend.fnn.fused_swiglu(x, Wg, Wu, dtype=dtype))
+
+
+def test_fused_swiglu_always_2d_and_config4_convention(backend):
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((2, 5, 16)).astype(np.float32)
+    Wg = rng.standard_normal((12, 16)).astype(np.float32); Wu = rng.standard_normal((12, 16)).astype(np.float32)
+    out = backend.fnn.fused_swiglu(x, Wg, Wu)
+    assert out.shape == (10, 12)
+    # BASELINE config 4 wants silu(x.Wg)*(x.Wu): pass W_gate:=Wu, W_up:=Wg
+    want = O.truth_silu(x.reshape(10, 16).astype(np.float64) @ Wg.T) * (x.reshape(10, 16).astype(np.float64) @ Wu.T)
+    assert O.max_rel(backend.fnn.fused_swiglu(x, Wu, Wg), want) < TOL_F32
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_gemm_nn_and_transposed_view(backend, dtype):
+    rng = np.random.default_rng(8)
+    A = rng.standard_normal((65, 40)).astype(np.float32)
+    B = rng.standard_normal((40, 77)).astype(np.float32)
+    A, B = prep(dtype, A, B)
+    assert O.max_rel(backend.fnn.gemm(A, B, dtype=dtype), O.truth_gemm(A, B)) < tol(dtype)
+    W = np.ascontiguousarray(B.T)                 # nn.Linear calls gemm(x, W.T) with a transposed view
+    assert O.max_rel(backend.fnn.gemm(A, W.T, dtype=dtype), O.truth_gemm(A, B)) < tol(dtype)
+    if dtype == "fp32":
+        np.testing.assert_array_equal(backend.fnn.gemm(np.array([[1, 2], [3, 4]], np.float32), np.array([[5, 6], [7, 8]], np.float32)),
+                                      np.array([[19, 22], [43, 50]], np.float32))     # reference tests/test_pytorch_ops.py:42-48
+
+
+def test_qkv_projection_equals_three_linears(backend):
+    rng = np.random.default_rng(9)
+    H, D, K = 4, 32, 96
+    x = rng.standard_normal((3, 7, K)).astype(np.float32)
+    Ws = [rng.standard_normal((H * D, K)).astype(np.float32) * 0.1 for _ in range(3)]
+    bs = [rng.standard_normal(H * D).astype(np.float32) for _ in range(3)]
+    qkv = backend.fnn.fused_qkv_projection(x, np.concatenate(Ws), np.concatenate(bs), num_heads=H, head_dim=D)
+    assert qkv.shape == (3, 7, 3 * H * D)
+    for i in range(3):
+        assert O.max_rel(qkv[..., i * H * D:(i + 1) * H * D], O.truth_linear(x, Ws[i], bs[i])) < TOL_F32
+    with pytest.raises(ValueError):
+        backend.fnn.fused_qkv_projection(x, np.concatenate(Ws), None, num_heads=5, head_dim=D)
+
+
+def test_shapes_dtypes_and_errors(backend):
+    rng = np.random.default_rng(10)
+    W = rng.standard_normal((6, 8)).astype(np.float32)
+    x3 = rng.standard_normal((2, 3, 8))                       # float64 in -> float32 out, leading dims kept
+    y = backend.fnn.linear(x3, W)
+    assert y.shape == (2, 3, 6) and y.dtype == np.float32
+    assert O.max_rel(y, O.truth_linear(x3, W)) < TOL_F32
+    assert backend.fnn.fused_linear_gelu(x3[0, 0], W).shape == (1, 6)     # rank-1 -> (1,N) (reference fnn.py:2055-2060)
+    assert backend.fnn.fused_linear_silu(x3, W).shape == (2, 3, 6)
+    xs = np.asfortranarray(rng.standard_normal((5, 8)).astype(np.float32))   # non-contiguous input is copied
+    assert O.max_rel(backend.fnn.linear(xs, W), O.truth_linear(xs, W)) < TOL_F32
+    before = x3.copy(); backend.fnn.linear(x3, W); np.testing.assert_array_equal(x3, before)   # inputs untouched
+    with pytest.raises(ValueError):
+        backend.fnn.linear(rng.standard_normal((4, 7)), W)
+    with pytest.raises(ValueError):
+        backend.fnn.linear(x3, W, np.zeros(5))
+    with pytest.raises(AssertionError):
+        backend.fnn.gemm(np.zeros((2, 3)), np.zeros((4, 5)))
+    with pytest.raises(ValueError):
+        backend.fnn.linear(x3, W, dtype="fp16")
+    assert backend.fnn.linear(np.zeros((0, 8), np.float32), W).shape == (0, 6)      # empty batch
+
+
+def test_full_size_properties_bert_ffn1(backend):
+    # BASELINE config 3 shape (one GEMM at full size, bf16): linearity + a row-sample against the oracle
+    rng = rng_for(3)
+    M, K, N = 65536, 768, 3072
+    x = O.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    W = O.bf16_round((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+    y = backend.fnn.linear(x, W, dtype="bf16")
+    rows = rng.integers(0, M, 64)
+    assert O.max_rel(y[rows], O.truth_linear(x[rows], W)) < TOL_BF16
+    # scaling the input by 2 (exact in bf16) scales the output by exactly 2
+    y2 = backend.fnn.linear(2 * x[:4096], W, dtype="bf16")
+    np.testing.assert_array_equal(y2, 2 * y[:4096])
+    # every tile was written: no row is left at its allocation value
+    assert np.isfinite(y).all() and (np.abs(y).max(axis=1) > 0).all()
+
+
+def test_buffer_pool_stats(backend):
+    s0 = backend.fnn.buffer_pool.get_stats()
+    x = np.ones((16, 16), np.float32)
+    for _ in range(20):
+        backend.fnn.linear(x, x)
+    s1 = backend.fnn.get_buffer_pool_stats()
+    assert s1["hits"] - s0["hits"] >= 60 and s1["allocations"] - s0["allocations"] < 10    # reference claims <10 allocs / 100 ops
+    assert 0.0 <= s1["hit_rate"] <= 1.0 and s1["bytes_in_use"] == s0["bytes_in_use"]

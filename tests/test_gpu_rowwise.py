@@ -1,0 +1,151 @@
+"""GPU parity of the HBM-bound kernels: LayerNorm(+residual), residual add, GELU, SiLU,
+SwiGLU activation, casts, embedding gather, masked mean pooling."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import TOL_F32, TOL_BF16
+from oracle import oracle_np as O
+from grilly_amd import _lib as L
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("shape", [(100,), (7, 384), (4, 16, 768), (3, 5, 1024), (2, 2048), (5, 2052), (9, 333), (2, 4100)])
+def test_layernorm_parity(backend, corc, dtype, shape):
+    rng = np.random.default_rng(sum(shape))
+    x = (rng.standard_normal(shape) * 3 + 1).astype(np.float32)
+    if dtype == "bf16":
+        x = O.bf16_round(x)
+    F = shape[-1]
+    g = rng.standard_normal(F).astype(np.float32); b = rng.standard_normal(F).astype(np.float32)
+    y = backend.fnn.layernorm(x, g, b, dtype=dtype)
+    assert y.shape == x.shape
+    assert O.max_rel(y, O.truth_layernorm(x, g, b)) < (TOL_F32 if dtype == "fp32" else TOL_BF16)
+    if dtype == "fp32":
+        assert O.max_rel(y, corc.layernorm(x, g, b)) < 1e-5
+        y0 = backend.fnn.layernorm(x)          # gamma/beta default to ones/zeros; reference test: mean~0, std~1
+        assert np.abs(y0.mean(-1)).max() < 1e-4 and np.abs(y0.std(-1) - 1).max() < 1e-2
+        assert O.max_rel(backend.fnn.layernorm(x, g, b, eps=0.5), O.truth_layernorm(x, g, b, eps=0.5)) < TOL_F32
+
+
+def test_layernorm_constant_row_and_rank_check(backend):
+    beta = np.arange(16, dtype=np.float32)
+    y = backend.fnn.layernorm(np.full((3, 16), 2.5, np.float32), np.ones(16), beta)
+    np.testing.assert_allclose(y, np.tile(beta, (3, 1)), atol=1e-6)
+    with pytest.raises(ValueError):
+        backend.fnn.layernorm(np.zeros((2, 2, 2, 8), np.float32))
+    with pytest.raises(ValueError):
+        backend.fnn.layernorm(np.zeros((2, 8), np.float32), np.ones(7))
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_layernorm_with_residual_device_api(backend, dtype):
+    # the fused residual+LayerNorm entry point the encoder layer uses, called on device pointers
+    rng = np.random.default_rng(5)
+    rows, F = 1000, 768
+    x = rng.standard_normal((rows, F)).astype(np.float32); r = rng.standard_normal((rows, F)).astype(np.float32)
+    if dtype == "bf16":
+        x, r = O.bf16_round(x), O.bf16_round(r)
+    g = rng.standard_normal(F).astype(np.float32); b = rng.standard_normal(F).astype(np.float32)
+    c = backend.core
+    code = L.GRL_BF16 if dtype == "bf16" else L.GRL_F32
+    dx, dr, dg, db = c.upload(x, code), c.upload(r, code), c.upload(g), c.upload(b)
+    L.check(c.lib.grl_layernorm(c.ctx, code, rows, F, dx.ptr, dr.ptr, dg.ptr, db.ptr, 1e-5, dx.ptr))    # in place
+    y = c.download(dx, (rows, F), code)
+    assert O.max_rel(y, O.truth_layernorm(x, g, b, residual=r)) < (TOL_F32 if dtype == "fp32" else TOL_BF16)
+    for t in (dx, dr, dg, db):
+        t.free()
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("n", [1, 5, 1023, 4096, 100003])
+def test_elementwise_parity(backend, dtype, n):
+    rng = np.random.default_rng(n)
+    a = (rng.standard_normal(n) * 4).astype(np.float32); b = rng.standard_normal(n).astype(np.float32)
+    if dtype == "bf16":
+        a, b = O.bf16_round(a), O.bf16_round(b)
+    t = TOL_F32 if dtype == "fp32" else TOL_BF16
+    r = backend.fnn.residual(a, b, dtype=dtype)
+    if dtype == "fp32":
+        np.testing.assert_array_equal(r, a + b)                       # exact
+    else:
+        np.testing.assert_array_equal(r, O.bf16_round(a + b))         # one RNE rounding of the exact fp32 sum
+    assert O.max_rel(backend.fnn.activation_gelu(a, dtype=dtype), O.truth_gelu(a)) < t
+    assert O.max_rel(backend.fnn.activation_silu(a, dtype=dtype), O.truth_silu(a)) < t
+
+
+def test_activation_edges(backend):
+    x = np.array([0.0, 1.0, -1.0, 49.9, 50.1, -50.1, 88.5, -88.5, -200.0, 200.0], np.float32)
+    g = backend.fnn.activation_gelu(x)
+    assert g[0] == 0.0 and g[1] > 0                                  # reference tests/test_gpu_operations.py:109-118
+    np.testing.assert_allclose(g, O.truth_gelu(x), rtol=1e-5, atol=1e-6)
+    s = backend.fnn.activation_silu(x)
+    np.testing.assert_allclose(s, O.truth_silu(x), rtol=1e-5, atol=1e-30)
+    assert np.isfinite(s).all()
+
+
+@pytest.mark.parametrize("shape", [(32,), (8, 64), (2, 3, 128), (5, 4098)])
+def test_activation_swiglu(backend, shape):
+    rng = np.random.default_rng(shape[-1])
+    x = rng.standard_normal(shape).astype(np.float32)
+    y = backend.fnn.activation_swiglu(x)
+    h = shape[-1] // 2
+    assert y.shape == shape[:-1] + (h,)
+    x1, x2 = x[..., :h], x[..., h:]
+    np.testing.assert_allclose(y, x1 * x2 / (1.0 + np.exp(-x2)), rtol=1e-5, atol=1e-6)      # reference test formula
+    with pytest.raises(ValueError):
+        backend.fnn.activation_swiglu(np.zeros((2, 5), np.float32))
+
+
+def test_casts_are_rne(backend):
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.standard_normal(5000).astype(np.float32) * 100,
+                        np.array([1.00390625, 1.005859375, 0.0, -0.0, 3.3895314e38, 1e-39], np.float32)])
+    c = backend.core
+    d = c.upload(x, L.GRL_BF16)
+    np.testing.assert_array_equal(c.download(d, x.shape, L.GRL_BF16), O.bf16_round(x))
+    d.free()
+
+
+def test_embed_and_mean_pool(backend):
+    rng = np.random.default_rng(2)
+    B, S, F, V = 3, 50, 384, 1000
+    tok = rng.standard_normal((V, F)).astype(np.float32); pos = rng.standard_normal((64, F)).astype(np.float32)
+    typ = rng.standard_normal((2, F)).astype(np.float32)
+    ids = rng.integers(0, V, (B, S)).astype(np.int32)
+    c = backend.core
+    dt, dp, dty, di = c.upload(tok), c.upload(pos), c.upload(typ), c.upload_raw(ids)
+    dx = c.alloc(B * S * F * 4)
+    L.check(c.lib.grl_embed(c.ctx, L.GRL_F32, B, S, F, V, di.ptr, dt.ptr, dp.ptr, dty.ptr, dx.ptr))
+    x = c.download(dx, (B, S, F))
+    np.testing.assert_allclose(x, O.truth_embed(ids, tok, pos, typ), atol=1e-6)
+    m = (np.arange(S)[None] < np.array([50, 1, 17])[:, None]).astype(np.float32)
+    dm = c.upload(m); do = c.alloc(B * F * 4)
+    L.check(c.lib.grl_mean_pool(c.ctx, L.GRL_F32, B, S, F, dx.ptr, dm.ptr, do.ptr, 1))
+    assert O.max_rel(c.download(do, (B, F)), O.truth_mean_pool(x, m)) < 1e-5
+    L.check(c.lib.grl_mean_pool(c.ctx, L.GRL_F32, B, S, F, dx.ptr, None, do.ptr, 0))
+    assert O.max_rel(c.download(do, (B, F)), O.truth_mean_pool(x, None, l2=False)) < 1e-5
+    for t in (dt, dp, dty, di, dx, dm, do):
+        t.free()
+
+
+def test_c_abi_argument_errors(backend):
+    c = backend.core
+    lib = c.lib
+    buf = c.alloc(1024)
+    assert lib.grl_gemm_nt(c.ctx, 5, 0, 4, 4, 4, buf.ptr, buf.ptr, None, buf.ptr, 0) == L.ERR_ARG
+    assert lib.grl_gemm_nt(c.ctx, 0, 0, 4, 4, 4, buf.ptr, buf.ptr, None, buf.ptr, 9) == L.ERR_ARG
+    assert lib.grl_gemm_nt(c.ctx, 0, 0, -1, 4, 4, buf.ptr, buf.ptr, None, buf.ptr, 0) == L.ERR_SHAPE
+    assert lib.grl_gemm_nt(c.ctx, 0, 0, 4, 4, 4, None, buf.ptr, None, buf.ptr, 0) == L.ERR_ARG
+    assert lib.grl_fa2_fwd(c.ctx, 0, 1, 8, 1, 48, buf.ptr, buf.ptr, buf.ptr, None, buf.ptr, 1.0, 0, 0, 1e4, 1.0, None) == L.ERR_SHAPE
+    assert "head_dim" in L.last_error()
+    assert lib.grl_layernorm(c.ctx, 0, 4, 0, buf.ptr, None, buf.ptr, buf.ptr, 1e-5, buf.ptr) == L.ERR_SHAPE
+    assert lib.grl_free(c.ctx, ctypes.c_void_p(12345)) == L.ERR_ARG          # foreign pointer
+    # an impossible allocation reports out-of-memory instead of crashing
+    assert lib.grl_malloc(c.ctx, 1 << 50) is None and "hipMalloc" in L.last_error()
+    buf.free()
+    info = backend.device_info()
+    assert info["arch"].startswith("gfx950") and info["wavefront"] == 64 and info["compute_units"] > 0

@@ -1,0 +1,263 @@
+"""Pins the oracle (oracle/oracle.c and oracle/oracle_np.py) without a GPU:
+reference-held known answers, closed forms, invariants, and C (fp32 shader order) vs
+float64 truth.  A plausible mistake (dropped term, wrong sign/index, transposed operand)
+fails at least one check here."""
+import numpy as np
+import pytest
+
+from oracle import oracle_np as O
+
+
+def rel(a, b):
+    return O.max_rel(a, b)
+
+
+# ---------------------------------------------------------------- reference-held known answers
+def test_matmul_known_answer(corc):
+    # reference tests/test_pytorch_ops.py:42-48
+    A = np.array([[1, 2], [3, 4]], np.float32); B = np.array([[5, 6], [7, 8]], np.float32)
+    want = np.array([[19, 22], [43, 50]], np.float32)
+    assert np.array_equal(corc.gemm(A, B), want)
+    assert np.array_equal(O.truth_gemm(A, B), want)
+    # linear takes (out,in): x.W^T with W = B^T is the same product (catches a transposed operand)
+    assert np.array_equal(corc.linear(A, B.T.copy()), want)
+    assert not np.array_equal(corc.linear(A, B), want)
+
+
+def test_gelu_known_points(corc):
+    # reference tests/test_gpu_operations.py:109-118: gelu(0)=0, gelu(1)>0
+    x = np.array([0.0, 1.0, -1.0, 6.0, 50.0, 50.5, -50.5, -60.0, 100.0], np.float32)
+    y = corc.gelu(x)
+    assert y[0] == 0.0 and y[1] > 0
+    assert abs(y[1] - 0.8411919906082768) < 1e-6        # tanh-GELU(1), closed form
+    assert abs(y[2] + 0.15880800939172324) < 1e-6
+    assert abs(y[3] - 6.0) < 1e-5                        # gelu(x) -> x
+    assert y[5] == 50.5 and y[6] == 0.0 and y[7] == 0.0 and y[8] == 100.0   # |x|>50 branch
+    assert rel(y, O.truth_gelu(x)) < 1e-6
+
+
+def test_swiglu_reference_formula(corc):
+    # reference tests/test_gpu_operations.py:169-195: x1 * x2/(1+exp(-x2)), 2-D and 1-D
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((8, 64)).astype(np.float32)
+    want = x[:, :32] * (x[:, 32:] / (1.0 + np.exp(-x[:, 32:])))
+    np.testing.assert_allclose(corc.swiglu_act(x), want, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(O.truth_swiglu_act(x), want, rtol=1e-5, atol=1e-6)
+    x1 = rng.standard_normal(32).astype(np.float32)
+    np.testing.assert_allclose(corc.swiglu_act(x1[None])[0], x1[:16] * x1[16:] / (1 + np.exp(-x1[16:])), rtol=1e-5, atol=1e-6)
+    # operand order matters: silu is on the SECOND half
+    assert rel(corc.swiglu_act(x), x[:, 32:] * (x[:, :32] / (1.0 + np.exp(-x[:, :32])))) > 1e-2
+
+
+def test_layernorm_reference_moments(corc):
+    # reference tests/test_gpu_operations.py:197-205: |mean|<0.1, |std-1|<0.1 on 100 randoms
+    rng = np.random.default_rng(42)
+    x = rng.standard_normal(100).astype(np.float32) * 3 + 2
+    y = corc.layernorm(x[None], np.ones(100), np.zeros(100))[0]
+    assert abs(y.mean()) < 1e-5 and abs(y.std() - 1) < 1e-3
+    # constant row -> beta; biased variance with eps inside the root
+    beta = rng.standard_normal(16).astype(np.float32)
+    y = corc.layernorm(np.full((1, 16), 3.25, np.float32), rng.standard_normal(16), beta)
+    np.testing.assert_allclose(y[0], beta, atol=1e-6)
+    x = np.array([[1.0, 3.0]], np.float32)      # mean 2, biased var 1
+    np.testing.assert_allclose(corc.layernorm(x, np.ones(2), np.zeros(2), eps=3.0)[0], [-0.5, 0.5], atol=1e-6)
+    np.testing.assert_allclose(O.truth_layernorm(x, eps=3.0)[0], [-0.5, 0.5], atol=1e-12)
+
+
+def test_linear_nn_module_tolerance(corc):
+    # reference tests/test_gemm_backward.py:42-154: x.W^T+b vs numpy, rtol 1e-4 / atol 1e-5, (64,128->256)
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((64, 128)).astype(np.float32)
+    W = (rng.standard_normal((256, 128)) * 0.1).astype(np.float32)
+    b = rng.standard_normal(256).astype(np.float32)
+    np.testing.assert_allclose(corc.linear(x, W, b), x @ W.T + b, rtol=1e-4, atol=1e-4)
+    assert rel(corc.linear(x, W, b), O.truth_linear(x, W, b)) < 1e-6
+
+
+# ---------------------------------------------------------------- GEMM family invariants
+def test_linear_invariants(corc):
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((5, 7)).astype(np.float32); x2 = rng.standard_normal((5, 7)).astype(np.float32)
+    W = rng.standard_normal((3, 7)).astype(np.float32); b = rng.standard_normal(3).astype(np.float32)
+    # bias only when x = 0
+    np.testing.assert_array_equal(corc.linear(np.zeros_like(x), W, b), np.tile(b, (5, 1)))
+    # linearity in x (no bias)
+    np.testing.assert_allclose(corc.linear(x + x2, W), corc.linear(x, W) + corc.linear(x2, W), atol=1e-5)
+    # gemm(x, W.T) == linear(x, W)
+    np.testing.assert_allclose(corc.gemm(x, W.T.copy()), corc.linear(x, W), atol=1e-6)
+    # brute-force python loop in the shader's order reproduces it bit for bit
+    want = np.zeros((5, 3), np.float32)
+    for m in range(5):
+        for n in range(3):
+            s = np.float32(0)
+            for k in range(7):
+                s = np.float32(s + np.float32(x[m, k] * W[n, k]))
+            want[m, n] = np.float32(s + b[n])
+    np.testing.assert_array_equal(corc.linear(x, W, b), want)
+
+
+def test_fused_epilogues_equal_composition(corc):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((9, 33)).astype(np.float32) * 2
+    W = rng.standard_normal((17, 33)).astype(np.float32); b = rng.standard_normal(17).astype(np.float32)
+    lin = corc.linear(x, W, b)
+    # the reference's own fallback: fused == activation(linear) (backend/fnn.py:2043-2046)
+    np.testing.assert_array_equal(corc.linear(x, W, b, "gelu"), corc.gelu(lin))
+    assert rel(corc.linear(x, W, b, "gelu"), O.truth_linear(x, W, b, "gelu")) < 1e-5
+    assert rel(corc.linear(x, W, b, "silu"), O.truth_linear(x, W, b, "silu")) < 1e-5
+    # silu(0)=0 and the +-88 clamp keeps large negatives finite and tiny
+    s = corc.linear(np.array([[0.0], [-100.0], [100.0]], np.float32), np.ones((1, 1), np.float32), None, "silu")
+    assert s[0, 0] == 0.0 and np.isfinite(s[1, 0]) and abs(s[1, 0]) < 1e-30 and s[2, 0] == 100.0
+
+
+def test_fused_swiglu_conventions(corc):
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((6, 20)).astype(np.float32)
+    Wg = rng.standard_normal((10, 20)).astype(np.float32); Wu = rng.standard_normal((10, 20)).astype(np.float32)
+    bg = rng.standard_normal(10).astype(np.float32); bu = rng.standard_normal(10).astype(np.float32)
+    out, g, u = corc.fused_swiglu(x, Wg, Wu, bg, bu)
+    t_out, t_g, t_u = O.truth_fused_swiglu(x, Wg, Wu, bg, bu)
+    assert rel(out, t_out) < 1e-5 and rel(g, t_g) < 1e-6 and rel(u, t_u) < 1e-6
+    # identity with the unfused pair: activation_swiglu(concat[gate, up])
+    np.testing.assert_allclose(out, corc.swiglu_act(np.concatenate([g, u], 1)), rtol=1e-5, atol=1e-6)
+    # SiLU sits on the UP projection, not the gate
+    assert rel(out, t_u * O.truth_silu(t_g)) > 1e-2
+    # one bias alone is ignored (reference _glu_append.py:68)
+    o1, _, _ = corc.fused_swiglu(x, Wg, Wu, bg, None)
+    o0, _, _ = corc.fused_swiglu(x, Wg, Wu, None, None)
+    np.testing.assert_array_equal(o1, o0)
+
+
+def test_qkv_is_concat_of_three_linears(corc):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((4, 12)).astype(np.float32)
+    Ws = [rng.standard_normal((8, 12)).astype(np.float32) for _ in range(3)]
+    bs = [rng.standard_normal(8).astype(np.float32) for _ in range(3)]
+    packed = corc.linear(x, np.concatenate(Ws, 0), np.concatenate(bs, 0))
+    for i in range(3):
+        np.testing.assert_array_equal(packed[:, 8 * i:8 * i + 8], corc.linear(x, Ws[i], bs[i]))
+
+
+# ---------------------------------------------------------------- attention
+def _qkv(rng, B, S, H, D):
+    return [rng.standard_normal((B, S, H, D)).astype(np.float32) for _ in range(3)]
+
+
+def test_attention_known_answers(corc):
+    rng = np.random.default_rng(6)
+    # S=1 -> O=V
+    q, k, v = _qkv(rng, 2, 1, 3, 8)
+    np.testing.assert_allclose(corc.attention(q, k, v), v, atol=1e-6)
+    # all scores equal (q=0) -> mean of V over keys
+    q, k, v = _qkv(rng, 1, 5, 2, 8)
+    np.testing.assert_allclose(corc.attention(np.zeros_like(q), k, v), np.broadcast_to(v.mean(1, keepdims=True), v.shape), atol=1e-6)
+    # two equal keys -> (v1+v2)/2, which the reference's racy shader would NOT produce (v1/2+v2/4)
+    k2 = np.repeat(k[:, :1], 2, 1); v2 = v[:, :2]; q2 = q[:, :2]
+    want = np.broadcast_to((v2[:, :1] + v2[:, 1:2]) / 2, v2.shape)
+    np.testing.assert_allclose(corc.attention(q2, k2, v2), want, atol=1e-6)
+    np.testing.assert_allclose(O.truth_attention(q2, k2, v2), want, atol=1e-12)
+    # mask keeping a single key -> that V row
+    m = np.zeros((1, 5), np.float32); m[0, 3] = 1
+    np.testing.assert_allclose(corc.attention(q, k, v, mask=m), np.broadcast_to(v[:, 3:4], v.shape), atol=1e-6)
+    # causal: row 0 sees only key 0; last row equals the unmasked result
+    oc = corc.attention(q, k, v, causal=True)
+    np.testing.assert_allclose(oc[:, 0], v[:, 0], atol=1e-6)
+    np.testing.assert_allclose(oc[:, -1], corc.attention(q, k, v)[:, -1], atol=1e-6)
+    # fully masked row degenerates to the uniform mean (mask bias added in fp32)
+    z = np.zeros((1, 5), np.float32)
+    np.testing.assert_allclose(corc.attention(q, k, v, mask=z), np.broadcast_to(v.mean(1, keepdims=True), v.shape), atol=1e-6)
+    np.testing.assert_allclose(O.truth_attention(q, k, v, mask=z), np.broadcast_to(v.astype(np.float64).mean(1, keepdims=True), v.shape), atol=1e-12)
+
+
+def test_attention_c_vs_truth_and_invariants(corc):
+    rng = np.random.default_rng(7)
+    B, S, H, D = 2, 37, 3, 32
+    q, k, v = _qkv(rng, B, S, H, D)
+    lens = np.array([37, 20])
+    m = (np.arange(S)[None] < lens[:, None]).astype(np.float32)
+    for kw in ({}, {"mask": m}, {"causal": True}, {"scale": 0.3}, {"mask": m, "causal": True}):
+        assert rel(corc.attention(q, k, v, **kw), O.truth_attention(q, k, v, **kw)) < 2e-6, kw
+    # layout check: heads are independent and live in axis 2 -- permuting heads permutes the output
+    perm = [2, 0, 1]
+    np.testing.assert_allclose(corc.attention(q[:, :, perm], k[:, :, perm], v[:, :, perm]), corc.attention(q, k, v)[:, :, perm], atol=1e-6)
+    # permutation equivariance over keys (unmasked)
+    p = rng.permutation(S)
+    np.testing.assert_allclose(corc.attention(q, k[:, p], v[:, p]), corc.attention(q, k, v), atol=2e-6)
+    # softmax shift invariance: adding c*q-independent constant to all scores (k -> k + t with q.t const) -- use scale of V instead:
+    np.testing.assert_allclose(corc.attention(q, k, 2 * v), 2 * corc.attention(q, k, v), atol=1e-5)
+
+
+def test_rope_properties(corc):
+    rng = np.random.default_rng(8)
+    B, S, H, D = 1, 9, 2, 16
+    x = rng.standard_normal((B, S, H, D)).astype(np.float32)
+    for style in ("half", "interleaved"):
+        y = corc.rope(x, style)
+        np.testing.assert_allclose(y[:, 0], x[:, 0], atol=1e-7)            # position 0 is unrotated
+        np.testing.assert_allclose(np.linalg.norm(y, axis=-1), np.linalg.norm(x, axis=-1), rtol=1e-5)   # rotation
+        assert rel(y, O.truth_rope(x, style=style)) < 1e-6
+        # scores depend only on the relative position: same vector pair at (i,j) and (i+3,j+3)
+        a = np.tile(x[:, :1], (1, S, 1, 1)); ya = corc.rope(a, style)
+        d1 = (ya[0, 1, 0] * ya[0, 4, 0]).sum(); d2 = (ya[0, 4, 0] * ya[0, 7, 0]).sum()
+        assert abs(d1 - d2) < 1e-4
+    # the two conventions differ, and are related by the even/odd <-> first/second-half permutation
+    yh, yi = corc.rope(x, "half"), corc.rope(x, "interleaved")
+    assert rel(yh, yi) > 1e-2
+    perm = np.concatenate([np.arange(0, D, 2), np.arange(1, D, 2)])
+    np.testing.assert_allclose(corc.rope(x[..., perm], "half"), yi[..., perm], atol=1e-6)
+    # explicit pair check against capsule_transformer-style formula (pairs 2i,2i+1; theta=pos*base^(-2i/D))
+    pos, i = 5, 3
+    th = pos * 10000.0 ** (-2 * i / D)
+    x0, x1 = x[0, pos, 1, 2 * i], x[0, pos, 1, 2 * i + 1]
+    np.testing.assert_allclose(yi[0, pos, 1, 2 * i:2 * i + 2], [x0 * np.cos(th) - x1 * np.sin(th), x0 * np.sin(th) + x1 * np.cos(th)], atol=1e-5)
+    # scaling divides the position; position_ids override arange
+    np.testing.assert_allclose(corc.rope(x, "half", scaling=2.0)[:, 2 * np.arange(4)], corc.rope(x, "half")[:, np.arange(4)] * 0 + corc.rope(x[:, 2 * np.arange(4)], "half", position_ids=np.arange(4)[None]), atol=1e-6)
+    # attention with rope == attention on pre-rotated q,k; V is never rotated
+    q, k, v = _qkv(rng, 1, 9, 2, 16)
+    for style in ("half", "interleaved"):
+        np.testing.assert_allclose(corc.attention(q, k, v, rope=style), corc.attention(corc.rope(q, style), corc.rope(k, style), v), atol=1e-6)
+        assert rel(corc.attention(q, k, v, rope=style, causal=True), O.truth_attention(q, k, v, rope=style, causal=True)) < 2e-6
+
+
+# ---------------------------------------------------------------- encoder pieces
+def test_embed_pool_and_layer(corc):
+    rng = np.random.default_rng(9)
+    B, S, H, D, ff, V = 2, 16, 2, 32, 128, 50
+    d = H * D
+    tok = rng.standard_normal((V, d)).astype(np.float32); pos = rng.standard_normal((32, d)).astype(np.float32)
+    typ = rng.standard_normal((2, d)).astype(np.float32)
+    ids = rng.integers(0, V, (B, S))
+    x = corc.embed(ids, tok, pos, typ)
+    np.testing.assert_allclose(x, tok[ids] + typ[0] + pos[:S][None], atol=1e-6)
+    assert rel(x, O.truth_embed(ids, tok, pos, typ)) < 1e-6
+    m = (np.arange(S)[None] < np.array([16, 5])[:, None]).astype(np.float32)
+    pooled = corc.mean_pool(x, m)
+    np.testing.assert_allclose(np.linalg.norm(pooled, axis=1), 1.0, atol=1e-6)
+    want = x[1, :5].mean(0); want /= np.linalg.norm(want)
+    np.testing.assert_allclose(pooled[1], want, atol=1e-6)
+    assert rel(pooled, O.truth_mean_pool(x, m)) < 1e-6
+
+    n = lambda *s: (rng.standard_normal(s) * 0.05).astype(np.float32)
+    w = {"w_qkv": n(3 * d, d), "b_qkv": n(3 * d), "w_o": n(d, d), "b_o": n(d), "ln1_g": 1 + n(d), "ln1_b": n(d),
+         "w_ff1": n(ff, d), "b_ff1": n(ff), "w_ff2": n(d, ff), "b_ff2": n(d), "ln2_g": 1 + n(d), "ln2_b": n(d)}
+    y = corc.bert_layer(x, w, m, H)
+    assert rel(y, O.truth_bert_layer(x, w, m, H)) < 1e-5
+    # post-LN: every output row is an affine map of a normalised row
+    z = (y - w["ln2_b"]) / w["ln2_g"]
+    assert np.abs(z.mean(-1)).max() < 1e-4 and np.abs(z.var(-1) - 1).max() < 1e-2
+
+
+def test_bf16_rounding_helpers():
+    x = np.array([1.0, 1.00390625, 1.005859375, -2.5, 3.1415927, 0.0, 1e-40, np.inf], np.float32)
+    r = O.bf16_round(x)
+    assert r[0] == 1.0 and r[3] == -2.5 and r[5] == 0.0 and np.isinf(r[7])
+    assert r[1] == 1.0            # tie -> even (mantissa 0)
+    assert r[2] == 1.0078125      # 1.005859375 is the tie between 1.00390625 (odd) and 1.0078125 (even)
+    assert abs(r[4] - 3.140625) < 1e-7
+    np.testing.assert_array_equal(O.from_bf16_bits(O.to_bf16_bits(x[:6])), r[:6])
+    try:
+        import torch
+        t = torch.tensor(x[:5]).to(torch.bfloat16).to(torch.float32).numpy()
+        np.testing.assert_array_equal(t, r[:5])
+    except ImportError:
+        pass
