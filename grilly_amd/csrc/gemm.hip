@@ -21,6 +21,7 @@
 // therefore hit eight different slots = all 32 banks once, for the reads as for the writes.
 #include "common.hpp"
 #include <type_traits>
+#include <cstdlib>
 
 int grl_transpose2d(grl_ctx* c, int dtype, int64_t R, int64_t C, const void* in, void* out);
 
@@ -85,6 +86,75 @@ template <> __device__ __forceinline__ void store4<float>(float* p, float a, flo
 template <> __device__ __forceinline__ void store4<uint16_t>(uint16_t* p, float a, float b, float c, float d) {
     u32x2 v = {pack_bf16x2(a, b), pack_bf16x2(c, d)};
     *(u32x2*)p = v;
+}
+
+// ---- direct epilogue: lane (li, lg) holds, for output row m = .. + li, the columns
+// n = .. + 8*q + 4*lg + {0..3} in accumulator registers 4q..4q+3 and stores them itself
+// (8- or 16-byte stores).  Every index into the accumulators is a compile-time constant so
+// they stay in registers.  Used for ragged N, for the SwiGLU pre-activation outputs and by the
+// staged kernel.
+template <typename OutT, int TM, int TN, int TNO, int WM, int WNO, int EPI, bool DUAL>
+__device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const GemmArgs& p, int m0, int n0, int wm, int wn, int li, int lg) {
+    OutT* C = (OutT*)p.C;
+    const bool vec_ok = (p.N & 3) == 0;
+    static_for<TM>([&](auto ia) {
+        constexpr int a = decltype(ia)::value;
+        const int m = m0 + wm * WM + a * 32 + li;
+        static_for<TNO>([&](auto ib) {
+            constexpr int b = decltype(ib)::value;
+            static_for<4>([&](auto iq) {
+                constexpr int q = decltype(iq)::value;
+                const int n = n0 + wn * WNO + b * 32 + 8 * q + 4 * lg;
+                if (m < p.M && n < p.N) {
+                    float v[4], u[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = acc[a][b][4 * q + e];
+                        u[e] = DUAL ? acc[a][DUAL ? b + TNO : b][4 * q + e] : 0.f;
+                    }
+                    const int64_t o = (int64_t)m * p.N + n;
+                    if (vec_ok) {
+                        if (p.bias) {
+                            f32x4 bv = *(const f32x4*)(p.bias + n);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] += bv[e];
+                        }
+                        if (DUAL) {
+                            if (p.bias2) {
+                                f32x4 bv = *(const f32x4*)(p.bias2 + n);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) u[e] += bv[e];
+                            }
+                            if (p.cache1) store4<float>(p.cache1 + o, v[0], v[1], v[2], v[3]);
+                            if (p.cache2) store4<float>(p.cache2 + o, u[0], u[1], u[2], u[3]);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(u[e]);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
+                        }
+                        store4<OutT>(C + o, v[0], v[1], v[2], v[3]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (n + e < p.N) {
+                                float x = v[e] + (p.bias ? p.bias[n + e] : 0.f);
+                                if (DUAL) {
+                                    float y = u[e] + (p.bias2 ? p.bias2[n + e] : 0.f);
+                                    if (p.cache1) p.cache1[o + e] = x;
+                                    if (p.cache2) p.cache2[o + e] = y;
+                                    x = x * silu_plain(y);
+                                } else {
+                                    x = epi_apply<EPI>(x);
+                                }
+                                elem<OutT>::st(C + o + e, x);
+                            }
+                        }
+                    }
+                }
+            });
+        });
+    });
 }
 
 // BN counts LDS rows of the weight tile; with DUAL it is 2x the output-column count of the
@@ -216,69 +286,196 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
         __syncthreads();
     }
 
-    // ---- epilogue: lane (li, lg) holds, for output row m = .. + li, the columns
-    // n = .. + 8*q + 4*lg + {0..3} in accumulator registers 4q..4q+3.  Every index into the
-    // accumulators is a compile-time constant so they stay in registers.
-    OutT* C = (OutT*)p.C;
-    const bool vec_ok = (p.N & 3) == 0;
-    static_for<TM>([&](auto ia) {
-        constexpr int a = decltype(ia)::value;
-        const int m = m0 + wm * WM + a * 32 + li;
-        static_for<TNO>([&](auto ib) {
-            constexpr int b = decltype(ib)::value;
-            static_for<4>([&](auto iq) {
-                constexpr int q = decltype(iq)::value;
-                const int n = n0 + wn * WNO + b * 32 + 8 * q + 4 * lg;
-                if (m < p.M && n < p.N) {
-                    float v[4], u[4];
+    epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
+}
+
+// =====================================================================================
+// Second generation main kernel: global -> LDS without passing through registers.
+//
+//   buffer_load_dwordx4 ... lds   writes each wave's 64 x 16 B straight into 1 KiB of LDS
+//   (8 tile rows); the lane -> chunk assignment carries the XOR swizzle, so the LDS image is
+//   the same as in the staged kernel above and the MFMA fragment reads are unchanged.
+//   No staging VGPRs, no ds_write, no select: the slab t+1 transfer runs entirely under the
+//   MFMAs of slab t.  8 waves per 256x256 tile (2 per SIMD) so that one wave's LDS waits and
+//   its epilogue arithmetic hide under the other's matrix work.
+//
+//   Needs K to be a whole number of 128-byte slabs (the transfer cannot zero a K tail);
+//   M and N are free: rows past the edge are out of range for the buffer resource, read as
+//   zero, and feed only accumulators that are never stored.
+//
+//   Epilogue: accumulators -> bias/activation -> OutT -> LDS (row-major, padded) -> 16-byte
+//   row-contiguous global stores, 32 output rows per wave-row at a time.
+// =====================================================================================
+template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL>
+__global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p) {
+    constexpr int NW = WGM * WGN, NT = NW * 64;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int BNO = DUAL ? BN / 2 : BN;
+    constexpr int WNO = DUAL ? WN / 2 : WN;
+    constexpr int TNO = DUAL ? TN / 2 : TN;
+    constexpr int GA = BM / 8 / NW, GB = BN / 8 / NW;      // 8-row groups per wave
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "row groups must divide over the waves");
+    static_assert(!DUAL || (NW % 2 == 0), "the two weights split the waves evenly");
+    constexpr int STAGE = (BM + BN) * 128;
+    constexpr int OES = (int)sizeof(OutT);
+    constexpr int CROW = BNO * OES + 16;                    // padded LDS row of the output staging
+    static_assert(WGM * 32 * CROW <= 2 * STAGE, "output staging must fit in the operand buffers");
+    __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int li = lane & 31, lg = lane >> 5;
+
+    int tile_m, tile_n;
+    {
+        const int nb = gridDim.x, pid = blockIdx.x;
+        const int per = nb >> 3, rem = nb & 7, xcd = pid & 7, loc = pid >> 3;
+        const int npid = xcd * per + (xcd < rem ? xcd : rem) + loc;
+        constexpr int GROUP = 8;
+        const int width = GROUP * p.tiles_n;
+        const int first_m = (npid / width) * GROUP;
+        const int gsize = p.tiles_m - first_m < GROUP ? p.tiles_m - first_m : GROUP;
+        tile_m = first_m + (npid % width) % gsize;
+        tile_n = (npid % width) / gsize;
+    }
+    const int m0 = tile_m * BM, n0 = tile_n * BNO;
+
+    const int64_t rowbytes = (int64_t)p.K * (int64_t)sizeof(T);
+    auto make_rsrc = [&](const void* base, int first_row, int rows_total) {
+        int64_t left = (int64_t)(rows_total - first_row) * rowbytes;
+        if (left < 0) left = 0;
+        uint32_t nrec = left > 0xffffffffLL ? 0xffffffffu : (uint32_t)left;
+        return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base + (int64_t)first_row * rowbytes), 0, (int)nrec, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(p.A, m0, p.M);
+    // with two weights the lower half of the waves fetches the gate rows, the upper half the up rows
+    const bool second = DUAL && (wave >= NW / 2);
+    const __amdgpu_buffer_rsrc_t rsW = make_rsrc(second ? p.W2 : p.W, n0, p.N);
+    const int lr = lane >> 3, ls = lane & 7;
+    // lane -> (row lr of the group, chunk ls ^ lr): LDS slot ls of row r holds chunk ls ^ (r & 7)
+    const int lane_off = lr * (int)rowbytes + ((ls ^ lr) << 4);
+    const int a_row0 = wave * GA * 8;                                    // first A tile row of this wave
+    const int b_row0_lds = wave * GB * 8;                                // LDS row in the weight region
+    const int b_row0_glb = second ? b_row0_lds - BNO : b_row0_lds;       // row relative to n0 in its matrix
+
+    auto issue = [&](int kt) {
+        char* st = lds + (kt & 1) * STAGE;
+        const int sbyte = kt * 128;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        v[e] = acc[a][b][4 * q + e];
-                        u[e] = DUAL ? acc[a][DUAL ? b + TNO : b][4 * q + e] : 0.f;
-                    }
-                    const int64_t o = (int64_t)m * p.N + n;
-                    if (vec_ok) {
+        for (int j = 0; j < GA; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (__attribute__((address_space(3))) void*)(st + (a_row0 + j * 8) * 128), 16,
+                                                 lane_off + (a_row0 + j * 8) * (int)rowbytes, sbyte, 0, 0);
+#pragma unroll
+        for (int j = 0; j < GB; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (__attribute__((address_space(3))) void*)(st + BM * 128 + (b_row0_lds + j * 8) * 128), 16,
+                                                 lane_off + (b_row0_glb + j * 8) * (int)rowbytes, sbyte, 0, 0);
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+    int rowX[TM], rowW[TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a) rowX[a] = wm * WM + a * 32 + li;
+#pragma unroll
+    for (int b = 0; b < TN; ++b) {
+        int base = DUAL ? ((b >= TNO ? BNO : 0) + wn * WNO + (b % TNO) * 32) : (wn * WN + b * 32);
+        rowW[b] = base + li;
+    }
+
+    constexpr int BKE = 128 / (int)sizeof(T);
+    const int KT = p.K / BKE;
+    issue(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's transfers have landed
+    __syncthreads();                         // ... and everybody else's
+    for (int kt = 0; kt < KT; ++kt) {
+        if (kt + 1 < KT) issue(kt + 1);
+        const char* s = lds + (kt & 1) * STAGE;
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            const int ch = 2 * sl + lg;
+            u32x4 xf[TM], wf[TN];
+#pragma unroll
+            for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ (rowX[a] & 7)) << 4));
+#pragma unroll
+            for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ (rowW[b] & 7)) << 4));
+            static_for<TM>([&](auto ia) {
+                static_for<TN>([&](auto ib) {
+                    MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
+                });
+            });
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+    }
+
+    OutT* C = (OutT*)p.C;
+    const bool staged = ((int64_t)p.N * OES) % 16 == 0 && !p.cache1 && !p.cache2;
+    if (staged) {
+        // ---- LDS-staged epilogue, one 32-row band of every wave-row per pass
+        constexpr int CPR = BNO * OES / 16;                  // 16-byte chunks per output row
+        constexpr int EPCO = 16 / OES;
+        static_for<TM>([&](auto ia) {
+            constexpr int a = decltype(ia)::value;
+            char* crow = lds + (wm * 32 + li) * CROW;
+            static_for<TNO>([&](auto ib) {
+                constexpr int b = decltype(ib)::value;
+                static_for<4>([&](auto iq) {
+                    constexpr int q = decltype(iq)::value;
+                    const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
+                    const int n = n0 + nl;
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e];
+                    if (n < p.N) {     // N % 4 == 0 here, so the 4 columns are in or out together
                         if (p.bias) {
                             f32x4 bv = *(const f32x4*)(p.bias + n);
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] += bv[e];
                         }
                         if (DUAL) {
+                            float u[4];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) u[e] = acc[a][DUAL ? b + TNO : b][4 * q + e];
                             if (p.bias2) {
                                 f32x4 bv = *(const f32x4*)(p.bias2 + n);
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) u[e] += bv[e];
                             }
-                            if (p.cache1) store4<float>(p.cache1 + o, v[0], v[1], v[2], v[3]);
-                            if (p.cache2) store4<float>(p.cache2 + o, u[0], u[1], u[2], u[3]);
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(u[e]);
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
                         }
-                        store4<OutT>(C + o, v[0], v[1], v[2], v[3]);
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            if (n + e < p.N) {
-                                float x = v[e] + (p.bias ? p.bias[n + e] : 0.f);
-                                if (DUAL) {
-                                    float y = u[e] + (p.bias2 ? p.bias2[n + e] : 0.f);
-                                    if (p.cache1) p.cache1[o + e] = x;
-                                    if (p.cache2) p.cache2[o + e] = y;
-                                    x = x * silu_plain(y);
-                                } else {
-                                    x = epi_apply<EPI>(x);
-                                }
-                                elem<OutT>::st(C + o + e, x);
-                            }
-                        }
                     }
-                }
+                    store4<OutT>((OutT*)(crow + nl * OES), v[0], v[1], v[2], v[3]);
+                });
             });
+            __syncthreads();
+            constexpr int TOTAL = WGM * 32 * CPR;
+#pragma unroll
+            for (int i = 0; i < (TOTAL + NT - 1) / NT; ++i) {
+                const int id = tid + i * NT;
+                if (TOTAL % NT == 0 || id < TOTAL) {
+                    const int r = id / CPR, cc = id % CPR;
+                    const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
+                    const int n = n0 + cc * EPCO;
+                    if (m < p.M && n < p.N)
+                        *(u32x4*)(C + (int64_t)m * p.N + n) = *(const u32x4*)(lds + r * CROW + cc * 16);
+                }
+            }
+            __syncthreads();
         });
-    });
+    } else {
+        epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
+    }
 }
 
 // ---- any shape / any alignment: one thread per output, ascending-k fp32 sum (the summation
@@ -320,16 +517,36 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
         GRL_CHECK_LAUNCH();
         return GRL_OK;
     }
-    // big tile when it fills the 256 CUs at least ~once, else the small tile for more workgroups
+    // Tile choice.  The direct-to-LDS kernel needs whole 128-byte K slabs; the 256x256 tile is
+    // used once it yields enough workgroups to occupy most of the 256 CUs, else 128x128 tiles.
+    // GRL_GEMM_VARIANT (1..4) forces one variant, for tuning runs.
+    static const int forced = [] { const char* e = getenv("GRL_GEMM_VARIANT"); return e ? atoi(e) : 0; }();
+    const int64_t bke = 128 / (int64_t)sizeof(T);
     const int64_t big_m = (a.M + 255) / 256, big_n = (a.N + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
-    if (big_m * big_n >= 192) {
-        a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
-        hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 256, 256, 2, 2, EPI, DUAL>), dim3((unsigned)(big_m * big_n)), dim3(256), 0, c->stream, a);
-    } else {
-        const int64_t sm = (a.M + 127) / 128, sn = (a.N + (DUAL ? 63 : 127)) / (DUAL ? 64 : 128);
-        GRL_REQUIRE(sm * sn < (1LL << 31), GRL_ERR_SHAPE, "gemm: too many tiles");
-        a.tiles_m = (int)sm; a.tiles_n = (int)sn;
-        hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)(sm * sn)), dim3(256), 0, c->stream, a);
+    const int64_t sm = (a.M + 127) / 128, sn = (a.N + (DUAL ? 63 : 127)) / (DUAL ? 64 : 128);
+    GRL_REQUIRE(sm * sn < (1LL << 31), GRL_ERR_SHAPE, "gemm: too many tiles");
+    GRL_REQUIRE(a.K * (int64_t)sizeof(T) * 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: K too large (256 rows must span < 2 GiB)");
+    const bool slabs = a.K % bke == 0;
+    const bool big = big_m * big_n >= 192;
+    int variant = slabs ? (big ? 3 : 4) : (big ? 1 : 2);
+    if (forced >= 1 && forced <= 4 && (slabs || forced <= 2)) variant = forced;
+    switch (variant) {
+        case 1:
+            a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
+            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 256, 256, 2, 2, EPI, DUAL>), dim3((unsigned)(big_m * big_n)), dim3(256), 0, c->stream, a);
+            break;
+        case 2:
+            a.tiles_m = (int)sm; a.tiles_n = (int)sn;
+            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)(sm * sn)), dim3(256), 0, c->stream, a);
+            break;
+        case 3:
+            a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
+            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 256, 256, 2, 4, EPI, DUAL>), dim3((unsigned)(big_m * big_n)), dim3(512), 0, c->stream, a);
+            break;
+        default:
+            a.tiles_m = (int)sm; a.tiles_n = (int)sn;
+            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)(sm * sn)), dim3(256), 0, c->stream, a);
+            break;
     }
     GRL_CHECK_LAUNCH();
     return GRL_OK;
