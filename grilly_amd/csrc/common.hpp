@@ -79,9 +79,12 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
     return __builtin_bit_cast(float, (uint32_t)b << 16);
 }
-// two floats -> packed pair of bf16 (lo in bits 0..15)
+// two floats -> packed pair of bf16 (lo in bits 0..15); one v_cvt_pk_bf16_f32 (RNE) on gfx950
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+    f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 // bit reinterpretation through a by-value copy: __builtin_bit_cast applied directly to an
 // element of an ext_vector (v[i]) reads element 0 whatever i is.
@@ -109,11 +112,23 @@ __device__ __forceinline__ float gelu_ref(float x) {
     if (fabsf(x) > 50.0f) r = x > 0.0f ? x : 0.0f;
     return r;
 }
-// shaders/fused-linear-silu.glsl:43-48
+// Fast forms for GEMM epilogues: v_exp_f32 (base 2) and v_rcp_f32, both within 1 ulp, instead
+// of the multi-instruction IEEE division.
+// shaders/fused-linear-silu.glsl:43-48: x * 1/(1+exp(-clamp(x,-88,88)))
 __device__ __forceinline__ float silu_clamped(float x) {
-    float c = fminf(fmaxf(x, -88.0f), 88.0f);
-    return x * (1.0f / (1.0f + __expf(-c)));
+    float c = __builtin_amdgcn_fmed3f(x, -88.0f, 88.0f);
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * c));
 }
-// shaders/fused-swiglu.glsl:44-46
-__device__ __forceinline__ float silu_plain(float x) { return x / (1.0f + __expf(-x)); }
+// shaders/fused-swiglu.glsl:44-46: x/(1+exp(-x)); exp overflow gives x*0 = -0 like the division
+__device__ __forceinline__ float silu_plain(float x) {
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+// shaders/fused-linear-gelu.glsl:45-63 rewritten with tanh(u) = 2/(1+exp(-2u)) - 1:
+//   0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (c + 0.044715 c^3), c = clamp(x, +-50).
+// For |x| > 50 the exponential saturates to 0 / +inf, which yields x and (-)0: the shader's rule.
+__device__ __forceinline__ float gelu_fast(float x) {
+    float c = __builtin_amdgcn_fmed3f(x, -50.0f, 50.0f);
+    float e = c * (-2.302208198f + -0.10294324f * (c * c));     // -2u*log2(e)
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e));
+}
 #endif

@@ -22,6 +22,7 @@
 #include "common.hpp"
 #include <type_traits>
 #include <cstdlib>
+#include <algorithm>
 
 int grl_transpose2d(grl_ctx* c, int dtype, int64_t R, int64_t C, const void* in, void* out);
 
@@ -41,16 +42,7 @@ struct GemmArgs {
 enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
 
 template <int EPI> __device__ __forceinline__ float epi_apply(float v) {
-    if (EPI == EPI_GELU) {
-        // same closed form as gelu_ref, with tanh(u) = 1 - 2/(exp(2u)+1): one v_exp instead of
-        // the library tanhf; absolute error ~1e-7, and the +-50 rule is kept.
-        float c = fminf(fmaxf(v, -50.0f), 50.0f);
-        float inner = 0.7978845608028654f * (c + 0.044715f * (c * c * c));
-        float t = 1.0f - 2.0f / (__expf(2.0f * inner) + 1.0f);
-        float r = 0.5f * v * (1.0f + t);
-        if (fabsf(v) > 50.0f) r = v > 0.0f ? v : 0.0f;
-        return r;
-    }
+    if (EPI == EPI_GELU) return gelu_fast(v);
     if (EPI == EPI_SILU) return silu_clamped(v);
     return v;
 }
@@ -290,21 +282,26 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
 }
 
 // =====================================================================================
-// Second generation main kernel: global -> LDS without passing through registers.
+// Main kernel: persistent workgroups, global -> LDS without passing through registers.
 //
 //   buffer_load_dwordx4 ... lds   writes each wave's 64 x 16 B straight into 1 KiB of LDS
 //   (8 tile rows); the lane -> chunk assignment carries the XOR swizzle, so the LDS image is
 //   the same as in the staged kernel above and the MFMA fragment reads are unchanged.
 //   No staging VGPRs, no ds_write, no select: the slab t+1 transfer runs entirely under the
-//   MFMAs of slab t.  8 waves per 256x256 tile (2 per SIMD) so that one wave's LDS waits and
-//   its epilogue arithmetic hide under the other's matrix work.
+//   MFMAs of slab t.  8 waves per 256x256 tile (2 per SIMD) so that one wave's LDS waits hide
+//   under the other's matrix work.
+//
+//   One workgroup per CU walks over its tiles.  When a tile's K loop ends, the first slab of
+//   the NEXT tile is already requested into LDS stage 0 before the epilogue starts, so its
+//   HBM/L2 latency hides under the epilogue, which stages the output through LDS stage 1.
 //
 //   Needs K to be a whole number of 128-byte slabs (the transfer cannot zero a K tail);
 //   M and N are free: rows past the edge are out of range for the buffer resource, read as
 //   zero, and feed only accumulators that are never stored.
 //
-//   Epilogue: accumulators -> bias/activation -> OutT -> LDS (row-major, padded) -> 16-byte
-//   row-contiguous global stores, 32 output rows per wave-row at a time.
+//   Epilogue: accumulators -> bias/activation -> OutT -> LDS (row-major, 16-byte chunks XOR
+//   swizzled by row) -> 16-byte row-contiguous global stores, 32 output rows per wave-row
+//   per pass, two staging regions used alternately so a pass costs one barrier.
 // =====================================================================================
 template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL>
 __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p) {
@@ -319,27 +316,31 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     static_assert(!DUAL || (NW % 2 == 0), "the two weights split the waves evenly");
     constexpr int STAGE = (BM + BN) * 128;
     constexpr int OES = (int)sizeof(OutT);
-    constexpr int CROW = BNO * OES + 16;                    // padded LDS row of the output staging
-    static_assert(WGM * 32 * CROW <= 2 * STAGE, "output staging must fit in the operand buffers");
+    constexpr int CROWB = BNO * OES;                        // bytes per staged output row
+    constexpr int CPR = CROWB / 16;                         // 16-byte chunks per staged row
+    constexpr int RG = WGM * 32 * CROWB;                    // one staging region
+    constexpr int NREG = 2 * RG <= STAGE ? 2 : 1;
+    static_assert(RG <= STAGE && (CPR & (CPR - 1)) == 0, "output staging must fit in LDS stage 1");
     __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
     const int li = lane & 31, lg = lane >> 5;
+    const int ntiles = p.tiles_m * p.tiles_n;
 
-    int tile_m, tile_n;
-    {
-        const int nb = gridDim.x, pid = blockIdx.x;
-        const int per = nb >> 3, rem = nb & 7, xcd = pid & 7, loc = pid >> 3;
+    // workgroup id -> tile: give each XCD (workgroup ids are dealt round-robin over the 8 XCDs,
+    // and the persistent stride is a multiple of 8) a contiguous run of tiles, walked in bands
+    // of 8 tile-rows so that the 32 CUs of an XCD share few A and W row panels in their L2.
+    auto tile_of = [&](int pid, int& m0, int& n0) {
+        const int per = ntiles >> 3, rem = ntiles & 7, xcd = pid & 7, loc = pid >> 3;
         const int npid = xcd * per + (xcd < rem ? xcd : rem) + loc;
         constexpr int GROUP = 8;
         const int width = GROUP * p.tiles_n;
         const int first_m = (npid / width) * GROUP;
         const int gsize = p.tiles_m - first_m < GROUP ? p.tiles_m - first_m : GROUP;
-        tile_m = first_m + (npid % width) % gsize;
-        tile_n = (npid % width) / gsize;
-    }
-    const int m0 = tile_m * BM, n0 = tile_n * BNO;
+        m0 = (first_m + (npid % width) % gsize) * BM;
+        n0 = ((npid % width) / gsize) * BNO;
+    };
 
     const int64_t rowbytes = (int64_t)p.K * (int64_t)sizeof(T);
     auto make_rsrc = [&](const void* base, int first_row, int rows_total) {
@@ -348,10 +349,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
         uint32_t nrec = left > 0xffffffffLL ? 0xffffffffu : (uint32_t)left;
         return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base + (int64_t)first_row * rowbytes), 0, (int)nrec, 0x00020000);
     };
-    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(p.A, m0, p.M);
     // with two weights the lower half of the waves fetches the gate rows, the upper half the up rows
     const bool second = DUAL && (wave >= NW / 2);
-    const __amdgpu_buffer_rsrc_t rsW = make_rsrc(second ? p.W2 : p.W, n0, p.N);
+    const void* Wsrc = second ? p.W2 : p.W;
     const int lr = lane >> 3, ls = lane & 7;
     // lane -> (row lr of the group, chunk ls ^ lr): LDS slot ls of row r holds chunk ls ^ (r & 7)
     const int lane_off = lr * (int)rowbytes + ((ls ^ lr) << 4);
@@ -359,26 +359,18 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     const int b_row0_lds = wave * GB * 8;                                // LDS row in the weight region
     const int b_row0_glb = second ? b_row0_lds - BNO : b_row0_lds;       // row relative to n0 in its matrix
 
-    auto issue = [&](int kt) {
+    auto issue = [&](__amdgpu_buffer_rsrc_t rsA, __amdgpu_buffer_rsrc_t rsW, int kt) {
         char* st = lds + (kt & 1) * STAGE;
         const int sbyte = kt * 128;
 #pragma unroll
         for (int j = 0; j < GA; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (__attribute__((address_space(3))) void*)(st + (a_row0 + j * 8) * 128), 16,
-                                                 lane_off + (a_row0 + j * 8) * (int)rowbytes, sbyte, 0, 0);
+                                                     lane_off + (a_row0 + j * 8) * (int)rowbytes, sbyte, 0, 0);
 #pragma unroll
         for (int j = 0; j < GB; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (__attribute__((address_space(3))) void*)(st + BM * 128 + (b_row0_lds + j * 8) * 128), 16,
-                                                 lane_off + (b_row0_glb + j * 8) * (int)rowbytes, sbyte, 0, 0);
+                                                     lane_off + (b_row0_glb + j * 8) * (int)rowbytes, sbyte, 0, 0);
     };
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int a = 0; a < TM; ++a)
-#pragma unroll
-        for (int b = 0; b < TN; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
     int rowX[TM], rowW[TN];
 #pragma unroll
@@ -391,90 +383,124 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
 
     constexpr int BKE = 128 / (int)sizeof(T);
     const int KT = p.K / BKE;
-    issue(0);
-    __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's transfers have landed
-    __syncthreads();                         // ... and everybody else's
-    for (int kt = 0; kt < KT; ++kt) {
-        if (kt + 1 < KT) issue(kt + 1);
-        const char* s = lds + (kt & 1) * STAGE;
-#pragma unroll
-        for (int sl = 0; sl < 4; ++sl) {
-            const int ch = 2 * sl + lg;
-            u32x4 xf[TM], wf[TN];
-#pragma unroll
-            for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ (rowX[a] & 7)) << 4));
-#pragma unroll
-            for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ (rowW[b] & 7)) << 4));
-            static_for<TM>([&](auto ia) {
-                static_for<TN>([&](auto ib) {
-                    MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
-                });
-            });
-        }
-        __builtin_amdgcn_s_waitcnt(0x0f70);
-        __syncthreads();
-    }
-
     OutT* C = (OutT*)p.C;
     const bool staged = ((int64_t)p.N * OES) % 16 == 0 && !p.cache1 && !p.cache2;
-    if (staged) {
-        // ---- LDS-staged epilogue, one 32-row band of every wave-row per pass
-        constexpr int CPR = BNO * OES / 16;                  // 16-byte chunks per output row
-        constexpr int EPCO = 16 / OES;
-        static_for<TM>([&](auto ia) {
-            constexpr int a = decltype(ia)::value;
-            char* crow = lds + (wm * 32 + li) * CROW;
-            static_for<TNO>([&](auto ib) {
-                constexpr int b = decltype(ib)::value;
-                static_for<4>([&](auto iq) {
-                    constexpr int q = decltype(iq)::value;
-                    const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
-                    const int n = n0 + nl;
-                    float v[4];
+
+    int pid = blockIdx.x;
+    int m0, n0;
+    tile_of(pid, m0, n0);
+    __amdgpu_buffer_rsrc_t rsA = make_rsrc(p.A, m0, p.M);
+    __amdgpu_buffer_rsrc_t rsW = make_rsrc(Wsrc, n0, p.N);
+    issue(rsA, rsW, 0);
+
+    for (;;) {
+        f32x16 acc[TM][TN];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e];
-                    if (n < p.N) {     // N % 4 == 0 here, so the 4 columns are in or out together
-                        if (p.bias) {
-                            f32x4 bv = *(const f32x4*)(p.bias + n);
+        for (int a = 0; a < TM; ++a)
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] += bv[e];
-                        }
-                        if (DUAL) {
-                            float u[4];
+            for (int b = 0; b < TN; ++b)
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) u[e] = acc[a][DUAL ? b + TNO : b][4 * q + e];
-                            if (p.bias2) {
-                                f32x4 bv = *(const f32x4*)(p.bias2 + n);
+                for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's transfers (and earlier stores) are done
+        __syncthreads();                         // ... and everybody else's; all staging reads of the last tile too
+        for (int kt = 0; kt < KT; ++kt) {
+            if (kt + 1 < KT) issue(rsA, rsW, kt + 1);
+            const char* s = lds + (kt & 1) * STAGE;
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) u[e] += bv[e];
-                            }
+            for (int sl = 0; sl < 4; ++sl) {
+                const int ch = 2 * sl + lg;
+                u32x4 xf[TM], wf[TN];
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(u[e]);
-                        } else {
+                for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ (rowX[a] & 7)) << 4));
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
-                        }
-                    }
-                    store4<OutT>((OutT*)(crow + nl * OES), v[0], v[1], v[2], v[3]);
+                for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ (rowW[b] & 7)) << 4));
+                static_for<TM>([&](auto ia) {
+                    static_for<TN>([&](auto ib) {
+                        MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
+                    });
                 });
-            });
+            }
+            __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();
-            constexpr int TOTAL = WGM * 32 * CPR;
+        }
+
+        // both LDS stages are free now: request the next tile's first slab into stage 0
+        const int npid = pid + (int)gridDim.x;
+        const bool has_next = npid < ntiles;
+        int m0n = 0, n0n = 0;
+        __amdgpu_buffer_rsrc_t rsAn = rsA, rsWn = rsW;
+        if (has_next) {
+            tile_of(npid, m0n, n0n);
+            rsAn = make_rsrc(p.A, m0n, p.M);
+            rsWn = make_rsrc(Wsrc, n0n, p.N);
+            issue(rsAn, rsWn, 0);
+        }
+
+        if (staged) {
+            // ---- LDS-staged epilogue in stage 1, one 32-row band of every wave-row per pass
+            constexpr int EPCO = 16 / OES;
+            char* stg = lds + STAGE;
+            static_for<TM>([&](auto ia) {
+                constexpr int a = decltype(ia)::value;
+                char* reg = stg + (NREG == 2 ? (a & 1) * RG : 0);
+                const int r_w = wm * 32 + li;
+                char* crow = reg + r_w * CROWB;
+                static_for<TNO>([&](auto ib) {
+                    constexpr int b = decltype(ib)::value;
+                    static_for<4>([&](auto iq) {
+                        constexpr int q = decltype(iq)::value;
+                        const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
+                        const int n = n0 + nl;
+                        float v[4];
 #pragma unroll
-            for (int i = 0; i < (TOTAL + NT - 1) / NT; ++i) {
-                const int id = tid + i * NT;
-                if (TOTAL % NT == 0 || id < TOTAL) {
+                        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e];
+                        if (n < p.N) {     // N % 4 == 0 here, so the 4 columns are in or out together
+                            if (p.bias) {
+                                f32x4 bv = *(const f32x4*)(p.bias + n);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) v[e] += bv[e];
+                            }
+                            if (DUAL) {
+                                float u[4];
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) u[e] = acc[a][DUAL ? b + TNO : b][4 * q + e];
+                                if (p.bias2) {
+                                    f32x4 bv = *(const f32x4*)(p.bias2 + n);
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) u[e] += bv[e];
+                                }
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(u[e]);
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
+                            }
+                        }
+                        const int byte = nl * OES;
+                        const int chunk = (byte >> 4) ^ (r_w & (CPR - 1));
+                        store4<OutT>((OutT*)(crow + (chunk << 4) + (byte & 15)), v[0], v[1], v[2], v[3]);
+                    });
+                });
+                __syncthreads();
+                constexpr int TOTAL = WGM * 32 * CPR;
+                static_assert(TOTAL % NT == 0, "staged chunks divide over the threads");
+#pragma unroll
+                for (int i = 0; i < TOTAL / NT; ++i) {
+                    const int id = tid + i * NT;
                     const int r = id / CPR, cc = id % CPR;
                     const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
                     const int n = n0 + cc * EPCO;
                     if (m < p.M && n < p.N)
-                        *(u32x4*)(C + (int64_t)m * p.N + n) = *(const u32x4*)(lds + r * CROW + cc * 16);
+                        *(u32x4*)(C + (int64_t)m * p.N + n) = *(const u32x4*)(reg + r * CROWB + ((cc ^ (r & (CPR - 1))) << 4));
                 }
-            }
-            __syncthreads();
-        });
-    } else {
-        epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
+                if (NREG == 1) __syncthreads();
+            });
+        } else {
+            epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
+        }
+        if (!has_next) break;
+        pid = npid; m0 = m0n; n0 = n0n; rsA = rsAn; rsW = rsWn;
     }
 }
 
@@ -528,6 +554,7 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     GRL_REQUIRE(a.K * (int64_t)sizeof(T) * 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: K too large (256 rows must span < 2 GiB)");
     const bool slabs = a.K % bke == 0;
     const bool big = big_m * big_n >= 192;
+    const int64_t cus = c->prop.multiProcessorCount;     // one 128 KiB-LDS workgroup per CU, two of the 64 KiB ones
     int variant = slabs ? (big ? 3 : 4) : (big ? 1 : 2);
     if (forced >= 1 && forced <= 4 && (slabs || forced <= 2)) variant = forced;
     switch (variant) {
@@ -541,11 +568,11 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
             break;
         case 3:
             a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
-            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 256, 256, 2, 4, EPI, DUAL>), dim3((unsigned)(big_m * big_n)), dim3(512), 0, c->stream, a);
+            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 256, 256, 2, 4, EPI, DUAL>), dim3((unsigned)std::min<int64_t>(big_m * big_n, cus)), dim3(512), 0, c->stream, a);
             break;
         default:
             a.tiles_m = (int)sm; a.tiles_n = (int)sn;
-            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)(sm * sn)), dim3(256), 0, c->stream, a);
+            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)std::min<int64_t>(sm * sn, 2 * cus)), dim3(256), 0, c->stream, a);
             break;
     }
     GRL_CHECK_LAUNCH();
