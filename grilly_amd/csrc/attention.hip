@@ -20,8 +20,11 @@
 //   out = acc / max(sum, 1e-10) ; causal keys (k > q) and keys >= S are excluded outright.
 #include "common.hpp"
 #include <type_traits>
+#include <algorithm>
 
 int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling);
+int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                     const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling);
 
 struct FaArgs {
     const void* Q; const void* K; const void* V;
@@ -345,6 +348,260 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
     }
 }
 
+// =====================================================================================
+// bf16 kernel, second generation.
+//
+//   K and V tiles (64 keys) go HBM -> LDS by buffer_load ... lds (no staging registers), both
+//   row-major [key][d] with the 16-byte chunks XOR-swizzled by key, double buffered.
+//   S^T = K.Q^T reads K with ds_read_b128; O^T += V^T.P^T reads V with the transposing
+//   ds_read_b64_tr_b16: inside a 16-lane group, source lane j points at
+//   V[k0 + j/4][d0 + 4*(j%4) ..] and result lane i receives V[k0 .. k0+3][d0 + i], i.e. four
+//   consecutive keys of ONE head dimension -- the MFMA operand -- without any shuffling.
+//   Softmax works in the base-2 domain: p = exp2(s*scale*log2e - m), one v_exp_f32 per score.
+//   About 130-190 VGPRs, so 2-3 workgroups share a CU and one wave's softmax VALU work
+//   overlaps another's MFMAs.
+//   RoPE: each Q row is rotated once as it is loaded; K is rotated once per row by the host
+//   wrapper into a workspace (rotating K inside the kernel would redo it for every query block).
+// =====================================================================================
+struct Fa16Args {
+    const uint16_t* Q; const uint16_t* K; const uint16_t* V;
+    const float* mask; uint16_t* O; const float2* rope;
+    int B, S, H;
+    float scale;
+    int causal;
+    int64_t q_stride, k_stride, v_stride, o_stride;
+};
+
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+
+template <int D, bool ROPE_Q>
+__global__ __launch_bounds__(256) void fa2_bf16_kernel(Fa16Args p) {
+    constexpr int RB = D * 2, NCH = RB / 16, NS = D / 16;
+    constexpr int KT = 64, NKB = 2, DT = D / 32;
+    constexpr int TILE = KT * RB;
+    constexpr int NI = TILE / 1024 / 4;           // DMA instructions per wave per tile and operand
+    constexpr int RPI = 1024 / RB;                // tile rows per DMA instruction
+    static_assert(TILE % 4096 == 0, "tile must split over 4 waves in 1 KiB transfers");
+    __shared__ __attribute__((aligned(1024))) char ldsK[2][TILE];
+    __shared__ __attribute__((aligned(1024))) char ldsV[2][TILE];
+    __shared__ __attribute__((aligned(16))) float ldsBias[2][KT];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 31, lg = lane >> 5;
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int qb = p.causal ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    const int q0 = qb * 128, S = p.S;
+    const int qi = q0 + wave * 32 + li;
+    const int qc = qi < S ? qi : S - 1;
+    const uint16_t* Qg = p.Q + (int64_t)b * S * p.q_stride + h * D;
+
+    u32x4 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int c = 2 * s + lg;
+        u32x4 v = *(const u32x4*)(Qg + (int64_t)qc * p.q_stride + c * 8);
+        if (ROPE_Q) {
+            float2 cs[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cs[i] = p.rope[(int64_t)qc * (D / 2) + c * 4 + i];
+            v = rope_chunk<uint16_t>(v, cs);
+        }
+        qf[s] = v;
+    }
+
+    int nkt = (S + KT - 1) / KT;
+    if (p.causal) {
+        int last = (q0 + 127 < S - 1 ? q0 + 127 : S - 1) / KT + 1;
+        nkt = nkt < last ? nkt : last;
+    }
+
+    // buffer resources cover this (batch, head)'s rows 0..S-1; rows >= S are out of range
+    auto make_rsrc = [&](const uint16_t* base, int64_t stride) {
+        int64_t bytes = (int64_t)(S - 1) * stride * 2 + RB;
+        uint32_t nrec = bytes > 0xffffffffLL ? 0xffffffffu : (uint32_t)bytes;
+        return __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)b * S * stride + h * D), 0, (int)nrec, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t rsK = make_rsrc(p.K, p.k_stride);
+    const __amdgpu_buffer_rsrc_t rsV = make_rsrc(p.V, p.v_stride);
+    const int kstride_b = (int)p.k_stride * 2, vstride_b = (int)p.v_stride * 2;
+    // lane -> (row, slot) inside one 1 KiB transfer; the slot holds chunk slot ^ swizzle(row)
+    const int t_row = lane / NCH, t_slot = lane % NCH;
+
+    auto issue = [&](int kt) {
+        const int st = kt & 1, k0 = kt * KT;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int inst = wave * NI + j;
+            const int row = inst * RPI + t_row;
+            const int chunk = NCH >= 8 ? (t_slot ^ (row & 7)) : (t_slot ^ ((row >> 1) & 3));
+            const int rowg = k0 + row;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsK, (__attribute__((address_space(3))) void*)(ldsK[st] + inst * 1024), 16,
+                                                     rowg * kstride_b + chunk * 16, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsV, (__attribute__((address_space(3))) void*)(ldsV[st] + inst * 1024), 16,
+                                                     rowg * vstride_b + chunk * 16, 0, 0, 0);
+        }
+        if (tid < KT) {
+            const int kk = k0 + tid;
+            float bv = 0.f;
+            if (p.mask && kk < S) bv = (p.mask[(int64_t)b * S + kk] - 1.0f) * 1e9f * 1.4426950408889634f;
+            if (kk >= S) bv = -__builtin_inff();
+            ldsBias[st][tid] = bv;
+        }
+    };
+
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[t][r] = 0.f;
+    float m_run = -1.4426950408889634e10f, l_run = 0.f;     // -1e10 in the base-2 domain
+    const float c2 = p.scale * 1.4426950408889634f;
+
+    issue(0);
+    for (int kt = 0; kt < nkt; ++kt) {
+        const int st = kt & 1, k0 = kt * KT;
+        __builtin_amdgcn_s_waitcnt(0x0f70);     // vmcnt(0): tile kt has landed (this wave's part)
+        __syncthreads();                        // everybody's part; and tile kt-1 is no longer read
+        if (kt + 1 < nkt) issue(kt + 1);
+        char* Kb = ldsK[st];
+        char* Vb = ldsV[st];
+        if (k0 + KT > S) {
+            // last, partial tile: rows >= S hold whatever the out-of-range transfer left; clear them
+            const int first = S - k0;
+            for (int i = tid; i < (KT - first) * NCH; i += 256) {
+                const u32x4 zero = {0u, 0u, 0u, 0u};
+                *(u32x4*)(Kb + first * RB + i * 16) = zero;
+                *(u32x4*)(Vb + first * RB + i * 16) = zero;
+            }
+            __syncthreads();
+        }
+
+        f32x16 sacc[NKB];
+        sfor<NKB>([&](auto it) {
+            constexpr int t = decltype(it)::value;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[t][r] = 0.f;
+            const int key = 32 * t + li;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const int c = 2 * s + lg;
+                const int slot = NCH >= 8 ? (c ^ (key & 7)) : (c ^ ((key >> 1) & 3));
+                u32x4 kf = *(const u32x4*)(Kb + key * RB + slot * 16);
+                Slab<uint16_t>::run(kf, qf[s], sacc[t]);
+            }
+        });
+
+        // ---- scores in the base-2 domain, running max
+        const bool diag = p.causal && (k0 + KT - 1 > q0 + wave * 32);
+        const bool biased = p.mask != nullptr || (k0 + KT > S);
+        float mx = -__builtin_inff();
+        if (biased || diag) {
+            sfor<NKB>([&](auto it) {
+                constexpr int t = decltype(it)::value;
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd) {
+                    const int kl = 32 * t + 8 * qd + 4 * lg;
+                    f32x4 bias = *(const f32x4*)(&ldsBias[st][kl]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float s = sacc[t][4 * qd + e] * c2 + bias[e];
+                        if (diag && (k0 + kl + e > qi)) s = -__builtin_inff();
+                        sacc[t][4 * qd + e] = s;
+                    }
+                }
+            });
+        } else {
+            sfor<NKB>([&](auto it) {
+                constexpr int t = decltype(it)::value;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[t][r] *= c2;
+            });
+        }
+        sfor<NKB>([&](auto it) {
+            constexpr int t = decltype(it)::value;
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) mx = __builtin_fmaxf(mx, __builtin_fmaxf(sacc[t][r], sacc[t][r + 1]));
+        });
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.f;
+        sfor<NKB>([&](auto it) {
+            constexpr int t = decltype(it)::value;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float pv = __builtin_amdgcn_exp2f(sacc[t][r] - m_new);
+                sacc[t][r] = pv;
+                psum += pv;
+            }
+        });
+        l_run = l_run * alpha + psum;
+        sfor<DT>([&](auto idt) {
+            constexpr int dt = decltype(idt)::value;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        });
+
+        // ---- O^T += V^T . P^T; V operand through the transposing LDS read
+        // source role of this lane inside its 16-lane group: key row j/4, 4 dims at 4*(j%4)
+        const int j16 = lane & 15, grp = lane >> 4;
+        sfor<NKB>([&](auto it) {
+            constexpr int t = decltype(it)::value;
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                u32x4 pf;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) pf[e] = pack_bf16x2(sacc[t][8 * hh + 2 * e], sacc[t][8 * hh + 2 * e + 1]);
+                // keys of MFMA k-index (g, e): 32t + 16hh + 8*(e/4) + 4g + e%4, g = lane/32
+                const int kA = 32 * t + 16 * hh + 4 * (grp >> 1) + (j16 >> 2);
+                sfor<DT>([&](auto idt) {
+                    constexpr int dt = decltype(idt)::value;
+                    const int dcol = 32 * dt + 16 * (grp & 1) + 4 * (j16 & 3);     // first of 4 dims this lane points at
+                    const int ch = dcol >> 3, sub = (dcol & 7) * 2;
+                    auto addr = [&](int key) {
+                        const int slot = NCH >= 8 ? (ch ^ (key & 7)) : (ch ^ ((key >> 1) & 3));
+                        return (__attribute__((address_space(3))) s16x4_t*)(Vb + key * RB + slot * 16 + sub);
+                    };
+                    s16x4_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16(addr(kA));
+                    s16x4_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16(addr(kA + 8));
+                    u32x2 wa = __builtin_bit_cast(u32x2, va), wb = __builtin_bit_cast(u32x2, vb);
+                    u32x4 vf = {wa[0], wa[1], wb[0], wb[1]};
+                    Slab<uint16_t>::run(vf, pf, oacc[dt]);
+                });
+            }
+        });
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / fmaxf(l_tot, 1e-10f);
+    if (qi < S) {
+        uint16_t* Og = p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
+        sfor<DT>([&](auto idt) {
+            constexpr int dt = decltype(idt)::value;
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int d = 32 * dt + 8 * qd + 4 * lg;
+                fa_store4<uint16_t>(Og + d, oacc[dt][4 * qd] * inv, oacc[dt][4 * qd + 1] * inv, oacc[dt][4 * qd + 2] * inv, oacc[dt][4 * qd + 3] * inv);
+            }
+        });
+    }
+}
+
+template <int D>
+static int launch_fa16(grl_ctx* c, const FaArgs& a, bool rope_q) {
+    Fa16Args f{};
+    f.Q = (const uint16_t*)a.Q; f.K = (const uint16_t*)a.K; f.V = (const uint16_t*)a.V;
+    f.mask = a.mask; f.O = (uint16_t*)a.O; f.rope = a.rope;
+    f.B = a.B; f.S = a.S; f.H = a.H; f.scale = a.scale; f.causal = a.causal;
+    f.q_stride = a.q_stride; f.k_stride = a.k_stride; f.v_stride = a.v_stride; f.o_stride = a.o_stride;
+    dim3 grid((unsigned)((a.S + 127) / 128), (unsigned)a.H, (unsigned)a.B), block(256);
+    if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true>), grid, block, 0, c->stream, f);
+    else hipLaunchKernelGGL((fa2_bf16_kernel<D, false>), grid, block, 0, c->stream, f);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
 template <typename T, int D>
 static int launch_fa(grl_ctx* c, FaArgs& a, bool rope) {
     dim3 grid((unsigned)((a.S + 127) / 128), (unsigned)a.H, (unsigned)a.B), block(256);
@@ -379,34 +636,44 @@ static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t
     a.B = (int)B; a.S = (int)S; a.H = (int)H; a.scale = scale; a.causal = causal ? 1 : 0;
     a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.o_stride = o_stride;
 
-    void* own = nullptr;
+    GRL_REQUIRE(S * std::max(std::max(q_stride, k_stride), std::max(v_stride, o_stride)) * es < (1LL << 31), GRL_ERR_SHAPE,
+                "%s: one batch entry must span less than 2 GiB", who);
+    void* own = nullptr;      // RoPE table or rotate-half workspace
+    void* own2 = nullptr;     // rotated K of the bf16 fused path
     int rc = GRL_OK;
     if (rope == GRL_ROPE_HALF) {
         // (d, d+D/2) pairs straddle MFMA chunks: rotate Q and K once into a workspace with the
         // standalone kernel, then run the plain kernel on the rotated copies.
-        GRL_REQUIRE(q_stride == hd && k_stride == hd, GRL_ERR_SHAPE, "%s: rotate-half RoPE needs contiguous Q and K", who);
         const size_t n = (size_t)B * S * H * D, bytes = n * grl_dtype_size(dtype);
         char* ws = (char*)workspace;
         if (!ws) { own = grl_malloc(c, 2 * bytes); if (!own) return GRL_ERR_OOM; ws = (char*)own; }
-        rc = grl_rope(c, dtype, B, S, H, D, Q, nullptr, ws, GRL_ROPE_HALF, rope_base, rope_scaling);
-        if (!rc) rc = grl_rope(c, dtype, B, S, H, D, K, nullptr, ws + bytes, GRL_ROPE_HALF, rope_base, rope_scaling);
-        a.Q = ws; a.K = ws + bytes;
+        rc = grl_rope_strided(c, dtype, B, S, H, D, Q, q_stride, nullptr, ws, GRL_ROPE_HALF, rope_base, rope_scaling);
+        if (!rc) rc = grl_rope_strided(c, dtype, B, S, H, D, K, k_stride, nullptr, ws + bytes, GRL_ROPE_HALF, rope_base, rope_scaling);
+        a.Q = ws; a.K = ws + bytes; a.q_stride = hd; a.k_stride = hd;
     } else if (rope == GRL_ROPE_INTERLEAVED) {
         const size_t bytes = (size_t)S * (D / 2) * sizeof(float2);
         own = grl_malloc(c, bytes);
         if (!own) return GRL_ERR_OOM;
         rc = grl_build_rope_table(c, (float*)own, (int)S, (int)D, rope_base, rope_scaling);
         a.rope = (const float2*)own;
+        if (!rc && dtype == GRL_BF16) {
+            // every K row is rotated exactly once here; the kernel rotates Q rows as it loads them
+            own2 = grl_malloc(c, (size_t)B * S * H * D * 2);
+            if (!own2) { grl_free(c, own); return GRL_ERR_OOM; }
+            rc = grl_rope_strided(c, dtype, B, S, H, D, K, k_stride, nullptr, own2, GRL_ROPE_INTERLEAVED, rope_base, rope_scaling);
+            a.K = own2; a.k_stride = hd;
+        }
     }
     const bool fused = rope == GRL_ROPE_INTERLEAVED;
     if (!rc) {
         if (dtype == GRL_F32) {
             rc = D == 32 ? launch_fa<float, 32>(c, a, fused) : D == 64 ? launch_fa<float, 64>(c, a, fused) : launch_fa<float, 128>(c, a, fused);
         } else {
-            rc = D == 32 ? launch_fa<uint16_t, 32>(c, a, fused) : D == 64 ? launch_fa<uint16_t, 64>(c, a, fused) : launch_fa<uint16_t, 128>(c, a, fused);
+            rc = D == 32 ? launch_fa16<32>(c, a, fused) : D == 64 ? launch_fa16<64>(c, a, fused) : launch_fa16<128>(c, a, fused);
         }
     }
-    if (own) grl_free(c, own);   // stream order keeps it alive until the kernel has finished
+    if (own) grl_free(c, own);   // stream order keeps the blocks alive until the kernel has finished
+    if (own2) grl_free(c, own2);
     return rc;
 }
 

@@ -292,7 +292,7 @@ void grl_rope_freqs(RopeFreq* f, int D, float base) {
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kernel(const T* __restrict__ x, const int32_t* __restrict__ pos_ids,
                                                   T* __restrict__ y, int64_t total_pairs, int S, int H, int D,
-                                                  int style, float scaling, RopeFreq fr) {
+                                                  int style, float scaling, RopeFreq fr, int64_t x_stride) {
     const int half = D >> 1;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total_pairs; i += stride) {
@@ -304,17 +304,28 @@ __global__ __launch_bounds__(256) void rope_kernel(const T* __restrict__ x, cons
         float theta = style == GRL_ROPE_HALF ? (pos / scaling) * fr.inv_freq[p] : (pos * fr.inv_freq[p]) / scaling;
         float sn, cs;
         sincosf(theta, &sn, &cs);
+        const int hh = (int)(vec - bs * H);
+        const int64_t xin = bs * x_stride + (int64_t)hh * D;     // input may be strided by position
         int64_t i0, i1;
-        if (style == GRL_ROPE_HALF) { i0 = vec * D + p; i1 = i0 + half; }
-        else { i0 = vec * D + 2 * p; i1 = i0 + 1; }
-        float a = elem<T>::ld(x + i0), b = elem<T>::ld(x + i1);
-        elem<T>::st(y + i0, a * cs - b * sn);
-        elem<T>::st(y + i1, b * cs + a * sn);
+        if (style == GRL_ROPE_HALF) { i0 = p; i1 = p + half; }
+        else { i0 = 2 * p; i1 = i0 + 1; }
+        float a = elem<T>::ld(x + xin + i0), b = elem<T>::ld(x + xin + i1);
+        elem<T>::st(y + vec * D + i0, a * cs - b * sn);
+        elem<T>::st(y + vec * D + i1, b * cs + a * sn);
     }
 }
 
+int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                     const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling);
+
 extern "C" int grl_rope(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x,
                         const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling) {
+    return grl_rope_strided(c, dtype, B, S, H, D, x, H * D, position_ids, y, style, rope_base, rope_scaling);
+}
+
+// x may have a position stride larger than H*D (a column block of a packed QKV buffer); y is dense
+int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                     const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling) {
     GRL_REQUIRE(c && x && y, GRL_ERR_ARG, "grl_rope: null argument");
     GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_rope: bad dtype %d", dtype);
     GRL_REQUIRE(style == GRL_ROPE_HALF || style == GRL_ROPE_INTERLEAVED, GRL_ERR_ARG, "grl_rope: bad style %d", style);
@@ -326,8 +337,8 @@ extern "C" int grl_rope(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, 
     if (pairs == 0) return GRL_OK;
     RopeFreq fr; grl_rope_freqs(&fr, (int)D, rope_base);
     dim3 g(ew_grid(pairs)), b(256);
-    if (dtype == GRL_F32) hipLaunchKernelGGL(rope_kernel<float>, g, b, 0, c->stream, (const float*)x, position_ids, (float*)y, pairs, (int)S, (int)H, (int)D, style, rope_scaling, fr);
-    else hipLaunchKernelGGL(rope_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, position_ids, (uint16_t*)y, pairs, (int)S, (int)H, (int)D, style, rope_scaling, fr);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(rope_kernel<float>, g, b, 0, c->stream, (const float*)x, position_ids, (float*)y, pairs, (int)S, (int)H, (int)D, style, rope_scaling, fr, x_stride);
+    else hipLaunchKernelGGL(rope_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, position_ids, (uint16_t*)y, pairs, (int)S, (int)H, (int)D, style, rope_scaling, fr, x_stride);
     GRL_CHECK_LAUNCH();
     return GRL_OK;
 }
