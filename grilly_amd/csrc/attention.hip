@@ -21,6 +21,7 @@
 #include "common.hpp"
 #include <type_traits>
 #include <algorithm>
+#include <cstdlib>
 
 int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling);
 int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
@@ -374,44 +375,49 @@ struct Fa16Args {
 
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 
-template <int D, bool ROPE_Q>
-__global__ __launch_bounds__(256) void fa2_bf16_kernel(Fa16Args p) {
+// s_waitcnt with vmcnt = N and the other counters left open (gfx9 encoding)
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+template <int IPT, int MAXT> __device__ __forceinline__ void wait_tiles_outstanding(int tiles) {
+    // allow `tiles` later tiles (IPT transfers each) to be still in flight; loads return in order
+    if constexpr (MAXT >= 0) {
+        if (tiles >= MAXT) wait_vmcnt<IPT * MAXT>();
+        else wait_tiles_outstanding<IPT, MAXT - 1>(tiles);
+    }
+}
+
+template <int D, bool ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK>
+__global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
+    // QT = 32-query MFMA tiles per wave (every K / V fragment read from LDS feeds QT MFMAs),
+    // NW waves per workgroup, NSTG-deep ring of 64-key K/V tiles in LDS (NSTG-1 tiles in flight).
     constexpr int RB = D * 2, NCH = RB / 16, NS = D / 16;
     constexpr int KT = 64, NKB = 2, DT = D / 32;
     constexpr int TILE = KT * RB;
-    constexpr int NI = TILE / 1024 / 4;           // DMA instructions per wave per tile and operand
-    constexpr int RPI = 1024 / RB;                // tile rows per DMA instruction
-    static_assert(TILE % 4096 == 0, "tile must split over 4 waves in 1 KiB transfers");
-    __shared__ __attribute__((aligned(1024))) char ldsK[2][TILE];
-    __shared__ __attribute__((aligned(1024))) char ldsV[2][TILE];
-    __shared__ __attribute__((aligned(16))) float ldsBias[2][KT];
+    constexpr int NT = NW * 64;
+    constexpr int TPO = TILE / 1024;              // 1 KiB transfers per tile and operand
+    constexpr int IPT = 2 * TPO / NW + (HAS_MASK ? 1 : 0);   // transfers per wave per tile (K, V, mask)
+    constexpr int RPI = 1024 / RB;                // tile rows per transfer
+    constexpr int QW = 32 * QT, QB = NW * QW;     // queries per wave / per workgroup
+    static_assert((2 * TPO) % NW == 0 && 2 * TPO >= NW, "transfers must divide over the waves");
+    static_assert(IPT * (NSTG - 1) < 64, "vmcnt is a 6-bit counter");
+    // ONE LDS array with manual offsets: with several __shared__ objects the compiler tracks the
+    // LDS-DMA transfers per object and puts a full vmcnt(0) in front of every LDS read of a ring
+    // that has a transfer in flight, which would serialise the prefetch.
+    constexpr int OFF_V = NSTG * TILE, OFF_M = 2 * NSTG * TILE;
+    __shared__ __attribute__((aligned(1024))) char lds[2 * NSTG * TILE + NSTG * 1024];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lg = lane >> 5;
     const int b = blockIdx.z, h = blockIdx.y;
     const int qb = p.causal ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
-    const int q0 = qb * 128, S = p.S;
-    const int qi = q0 + wave * 32 + li;
-    const int qc = qi < S ? qi : S - 1;
+    const int q0 = qb * QB, S = p.S;
+    const int qw0 = q0 + wave * QW;               // first query of this wave
     const uint16_t* Qg = p.Q + (int64_t)b * S * p.q_stride + h * D;
-
-    u32x4 qf[NS];
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        const int c = 2 * s + lg;
-        u32x4 v = *(const u32x4*)(Qg + (int64_t)qc * p.q_stride + c * 8);
-        if (ROPE_Q) {
-            float2 cs[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) cs[i] = p.rope[(int64_t)qc * (D / 2) + c * 4 + i];
-            v = rope_chunk<uint16_t>(v, cs);
-        }
-        qf[s] = v;
-    }
 
     int nkt = (S + KT - 1) / KT;
     if (p.causal) {
-        int last = (q0 + 127 < S - 1 ? q0 + 127 : S - 1) / KT + 1;
+        int last = (q0 + QB - 1 < S - 1 ? q0 + QB - 1 : S - 1) / KT + 1;
         nkt = nkt < last ? nkt : last;
     }
 
@@ -423,124 +429,186 @@ __global__ __launch_bounds__(256) void fa2_bf16_kernel(Fa16Args p) {
     };
     const __amdgpu_buffer_rsrc_t rsK = make_rsrc(p.K, p.k_stride);
     const __amdgpu_buffer_rsrc_t rsV = make_rsrc(p.V, p.v_stride);
+    const __amdgpu_buffer_rsrc_t rsM = __builtin_amdgcn_make_buffer_rsrc((void*)(p.mask ? p.mask + (int64_t)b * S : (const float*)p.Q), 0, HAS_MASK ? S * 4 : 0, 0x00020000);
     const int kstride_b = (int)p.k_stride * 2, vstride_b = (int)p.v_stride * 2;
     // lane -> (row, slot) inside one 1 KiB transfer; the slot holds chunk slot ^ swizzle(row)
     const int t_row = lane / NCH, t_slot = lane % NCH;
 
     auto issue = [&](int kt) {
-        const int st = kt & 1, k0 = kt * KT;
+        const int st = kt % NSTG, k0 = kt * KT;
 #pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            const int inst = wave * NI + j;
+        for (int j = 0; j < 2 * TPO / NW; ++j) {
+            const int g = wave * (2 * TPO / NW) + j;                 // transfer id within the tile: K first, then V
+            const bool isv = g >= TPO;
+            const int inst = isv ? g - TPO : g;
             const int row = inst * RPI + t_row;
             const int chunk = NCH >= 8 ? (t_slot ^ (row & 7)) : (t_slot ^ ((row >> 1) & 3));
             const int rowg = k0 + row;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsK, (__attribute__((address_space(3))) void*)(ldsK[st] + inst * 1024), 16,
-                                                     rowg * kstride_b + chunk * 16, 0, 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsV, (__attribute__((address_space(3))) void*)(ldsV[st] + inst * 1024), 16,
-                                                     rowg * vstride_b + chunk * 16, 0, 0, 0);
+            if (isv)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsV, (__attribute__((address_space(3))) void*)(lds + OFF_V + st * TILE + inst * 1024), 16,
+                                                         rowg * vstride_b + chunk * 16, 0, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsK, (__attribute__((address_space(3))) void*)(lds + st * TILE + inst * 1024), 16,
+                                                         rowg * kstride_b + chunk * 16, 0, 0, 0);
         }
-        if (tid < KT) {
-            const int kk = k0 + tid;
-            float bv = 0.f;
-            if (p.mask && kk < S) bv = (p.mask[(int64_t)b * S + kk] - 1.0f) * 1e9f * 1.4426950408889634f;
-            if (kk >= S) bv = -__builtin_inff();
-            ldsBias[st][tid] = bv;
-        }
+        // raw mask values of the tile's 64 keys (256 B; the transfer unit is 1 KiB per wave, lanes
+        // past the tile read further mask entries or out of range, which nobody uses).  Every wave
+        // issues it so that all waves count the same number of transfers per tile.
+        if (HAS_MASK)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsM, (__attribute__((address_space(3))) void*)(lds + OFF_M + st * 1024), 16,
+                                                     (k0 + lane * 4) * 4, 0, 0, 0);
     };
 
-    f32x16 oacc[DT];
+    f32x16 oacc[QT][DT];
+    float m_run[QT], l_run[QT];
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
+    for (int t = 0; t < QT; ++t) {
+        m_run[t] = -1.4426950408889634e10f;      // -1e10 in the base-2 domain
+        l_run[t] = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[t][r] = 0.f;
-    float m_run = -1.4426950408889634e10f, l_run = 0.f;     // -1e10 in the base-2 domain
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[t][d][r] = 0.f;
+    }
     const float c2 = p.scale * 1.4426950408889634f;
 
-    issue(0);
+    for (int t = 0; t < NSTG - 1 && t < nkt; ++t) issue(t);
+
+    // this wave's queries as MFMA "B" operand: slab s holds dims (2s+lg)*8 .. +7 of query li.
+    // Loaded after the first tiles were requested so that both latencies overlap; the explicit
+    // wait below retires these loads before the loop, which lets the waits inside the loop count
+    // only the tile transfers issued there.
+    u32x4 qf[QT][NS];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        const int qi = qw0 + 32 * t + li;
+        const int qc = qi < S ? qi : S - 1;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int c = 2 * s + lg;
+            u32x4 v = *(const u32x4*)(Qg + (int64_t)qc * p.q_stride + c * 8);
+            if (ROPE_Q) {
+                float2 cs[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) cs[i] = p.rope[(int64_t)qc * (D / 2) + c * 4 + i];
+                v = rope_chunk<uint16_t>(v, cs);
+            }
+            qf[t][s] = v;
+        }
+    }
+
+    wait_vmcnt<0>();
+
     for (int kt = 0; kt < nkt; ++kt) {
-        const int st = kt & 1, k0 = kt * KT;
-        __builtin_amdgcn_s_waitcnt(0x0f70);     // vmcnt(0): tile kt has landed (this wave's part)
-        __syncthreads();                        // everybody's part; and tile kt-1 is no longer read
-        if (kt + 1 < nkt) issue(kt + 1);
-        char* Kb = ldsK[st];
-        char* Vb = ldsV[st];
+        const int st = kt % NSTG, k0 = kt * KT;
+        // tiles kt+1 .. kt+NSTG-2 may still be in flight; tile kt (this wave's part) must have landed
+        wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1 - kt);
+        // barrier without a memory fence (a fence would wait for every transfer in flight): LDS
+        // writes of this wave are drained by lgkmcnt(0), its tile transfers by the wait above
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (kt + NSTG - 1 < nkt) issue(kt + NSTG - 1);   // into the stage tile kt-1 has just left
+        char* Kb = lds + st * TILE;
+        char* Vb = lds + OFF_V + st * TILE;
+        const float* Mb = (const float*)(lds + OFF_M + st * 1024);
         if (k0 + KT > S) {
             // last, partial tile: rows >= S hold whatever the out-of-range transfer left; clear them
             const int first = S - k0;
-            for (int i = tid; i < (KT - first) * NCH; i += 256) {
+            for (int i = tid; i < (KT - first) * NCH; i += NT) {
                 const u32x4 zero = {0u, 0u, 0u, 0u};
                 *(u32x4*)(Kb + first * RB + i * 16) = zero;
                 *(u32x4*)(Vb + first * RB + i * 16) = zero;
             }
-            __syncthreads();
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
+        // a wave whose queries all precede this tile has nothing to add (causal): it only keeps the barriers
+        if (p.causal && k0 > qw0 + QW - 1) continue;
 
-        f32x16 sacc[NKB];
+        f32x16 sacc[QT][NKB];
         sfor<NKB>([&](auto it) {
             constexpr int t = decltype(it)::value;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[t][r] = 0.f;
+            for (int u = 0; u < QT; ++u)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[u][t][r] = 0.f;
             const int key = 32 * t + li;
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 const int c = 2 * s + lg;
                 const int slot = NCH >= 8 ? (c ^ (key & 7)) : (c ^ ((key >> 1) & 3));
                 u32x4 kf = *(const u32x4*)(Kb + key * RB + slot * 16);
-                Slab<uint16_t>::run(kf, qf[s], sacc[t]);
+                sfor<QT>([&](auto iu) { Slab<uint16_t>::run(kf, qf[decltype(iu)::value][s], sacc[decltype(iu)::value][t]); });
             }
         });
 
-        // ---- scores in the base-2 domain, running max
-        const bool diag = p.causal && (k0 + KT - 1 > q0 + wave * 32);
-        const bool biased = p.mask != nullptr || (k0 + KT > S);
-        float mx = -__builtin_inff();
-        if (biased || diag) {
-            sfor<NKB>([&](auto it) {
-                constexpr int t = decltype(it)::value;
+        // ---- softmax in the base-2 domain: p = exp2(s*c2 + bias - m)
+        const bool diag = p.causal && (k0 + KT - 1 > qw0);
+        const bool tail = k0 + KT > S;
+        const bool biased = HAS_MASK || tail;
+        sfor<QT>([&](auto iu) {
+            constexpr int u = decltype(iu)::value;
+            const int qi = qw0 + 32 * u + li;
+            float mx = -__builtin_inff();
+            if (biased || diag) {
+                sfor<NKB>([&](auto it) {
+                    constexpr int t = decltype(it)::value;
 #pragma unroll
-                for (int qd = 0; qd < 4; ++qd) {
-                    const int kl = 32 * t + 8 * qd + 4 * lg;
-                    f32x4 bias = *(const f32x4*)(&ldsBias[st][kl]);
+                    for (int qd = 0; qd < 4; ++qd) {
+                        const int kl = 32 * t + 8 * qd + 4 * lg;
+                        f32x4 mk = {1.f, 1.f, 1.f, 1.f};
+                        if (HAS_MASK) mk = *(const f32x4*)(Mb + kl);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        float s = sacc[t][4 * qd + e] * c2 + bias[e];
-                        if (diag && (k0 + kl + e > qi)) s = -__builtin_inff();
-                        sacc[t][4 * qd + e] = s;
+                        for (int e = 0; e < 4; ++e) {
+                            // (mask-1)*1e9 as the shader forms it, then into the base-2 domain
+                            float sv = sacc[u][t][4 * qd + e] * c2;
+                            if (HAS_MASK) sv += ((mk[e] - 1.0f) * 1e9f) * 1.4426950408889634f;
+                            if ((diag && (k0 + kl + e > qi)) || (tail && (k0 + kl + e >= S))) sv = -__builtin_inff();
+                            sacc[u][t][4 * qd + e] = sv;
+                            mx = __builtin_fmaxf(mx, sv);
+                        }
                     }
-                }
-            });
-        } else {
+                });
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const float m_new = fmaxf(m_run[u], mx);
+                sfor<NKB>([&](auto it) {
+                    constexpr int t = decltype(it)::value;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sacc[u][t][r] = __builtin_amdgcn_exp2f(sacc[u][t][r] - m_new);
+                });
+                mx = m_new;
+            } else {
+                // plain tile: the max is taken on the raw products (c2 > 0) and the scale rides in the fma
+                sfor<NKB>([&](auto it) {
+                    constexpr int t = decltype(it)::value;
+#pragma unroll
+                    for (int r = 0; r < 16; r += 2) mx = __builtin_fmaxf(mx, __builtin_fmaxf(sacc[u][t][r], sacc[u][t][r + 1]));
+                });
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const float m_new = fmaxf(m_run[u], mx * c2);
+                const float nm = -m_new;
+                sfor<NKB>([&](auto it) {
+                    constexpr int t = decltype(it)::value;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sacc[u][t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][t][r], c2, nm));
+                });
+                mx = m_new;
+            }
+            float psum = 0.f;
             sfor<NKB>([&](auto it) {
                 constexpr int t = decltype(it)::value;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[t][r] *= c2;
+                for (int r = 0; r < 16; ++r) psum += sacc[u][t][r];
             });
-        }
-        sfor<NKB>([&](auto it) {
-            constexpr int t = decltype(it)::value;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[u] - mx);
+            l_run[u] = l_run[u] * alpha + psum;
+            // rescale the output only when some row of the wave raised its maximum
+            if (__builtin_amdgcn_ballot_w64(mx != m_run[u]) != 0) {
+                sfor<DT>([&](auto idt) {
+                    constexpr int dt = decltype(idt)::value;
 #pragma unroll
-            for (int r = 0; r < 16; r += 2) mx = __builtin_fmaxf(mx, __builtin_fmaxf(sacc[t][r], sacc[t][r + 1]));
-        });
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.f;
-        sfor<NKB>([&](auto it) {
-            constexpr int t = decltype(it)::value;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float pv = __builtin_amdgcn_exp2f(sacc[t][r] - m_new);
-                sacc[t][r] = pv;
-                psum += pv;
+                    for (int r = 0; r < 16; ++r) oacc[u][dt][r] *= alpha;
+                });
             }
-        });
-        l_run = l_run * alpha + psum;
-        sfor<DT>([&](auto idt) {
-            constexpr int dt = decltype(idt)::value;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+            m_run[u] = mx;
         });
 
         // ---- O^T += V^T . P^T; V operand through the transposing LDS read
@@ -550,9 +618,11 @@ __global__ __launch_bounds__(256) void fa2_bf16_kernel(Fa16Args p) {
             constexpr int t = decltype(it)::value;
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
-                u32x4 pf;
+                u32x4 pf[QT];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) pf[e] = pack_bf16x2(sacc[t][8 * hh + 2 * e], sacc[t][8 * hh + 2 * e + 1]);
+                for (int u = 0; u < QT; ++u)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) pf[u][e] = pack_bf16x2(sacc[u][t][8 * hh + 2 * e], sacc[u][t][8 * hh + 2 * e + 1]);
                 // keys of MFMA k-index (g, e): 32t + 16hh + 8*(e/4) + 4g + e%4, g = lane/32
                 const int kA = 32 * t + 16 * hh + 4 * (grp >> 1) + (j16 >> 2);
                 sfor<DT>([&](auto idt) {
@@ -567,25 +637,43 @@ __global__ __launch_bounds__(256) void fa2_bf16_kernel(Fa16Args p) {
                     s16x4_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16(addr(kA + 8));
                     u32x2 wa = __builtin_bit_cast(u32x2, va), wb = __builtin_bit_cast(u32x2, vb);
                     u32x4 vf = {wa[0], wa[1], wb[0], wb[1]};
-                    Slab<uint16_t>::run(vf, pf, oacc[dt]);
+                    sfor<QT>([&](auto iu) { Slab<uint16_t>::run(vf, pf[decltype(iu)::value], oacc[decltype(iu)::value][dt]); });
                 });
             }
         });
     }
 
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = 1.0f / fmaxf(l_tot, 1e-10f);
-    if (qi < S) {
-        uint16_t* Og = p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
-        sfor<DT>([&](auto idt) {
-            constexpr int dt = decltype(idt)::value;
 #pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const int d = 32 * dt + 8 * qd + 4 * lg;
-                fa_store4<uint16_t>(Og + d, oacc[dt][4 * qd] * inv, oacc[dt][4 * qd + 1] * inv, oacc[dt][4 * qd + 2] * inv, oacc[dt][4 * qd + 3] * inv);
-            }
-        });
+    for (int u = 0; u < QT; ++u) {
+        const int qi = qw0 + 32 * u + li;
+        const float l_tot = l_run[u] + __shfl_xor(l_run[u], 32, 64);
+        const float inv = 1.0f / fmaxf(l_tot, 1e-10f);
+        if (qi < S) {
+            uint16_t* Og = p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd) {
+                    const int d = 32 * dt + 8 * qd + 4 * lg;
+                    fa_store4<uint16_t>(Og + d, oacc[u][dt][4 * qd] * inv, oacc[u][dt][4 * qd + 1] * inv, oacc[u][dt][4 * qd + 2] * inv, oacc[u][dt][4 * qd + 3] * inv);
+                }
+        }
     }
+}
+
+template <int D, int QT, int NW, int NSTG>
+static int launch_fa16_cfg(grl_ctx* c, const Fa16Args& f, bool rope_q) {
+    const int qb = 32 * QT * NW;
+    dim3 grid((unsigned)((f.S + qb - 1) / qb), (unsigned)f.H, (unsigned)f.B), block(NW * 64);
+    if (f.mask) {
+        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, true>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, true>), grid, block, 0, c->stream, f);
+    } else {
+        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, false>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, false>), grid, block, 0, c->stream, f);
+    }
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
 }
 
 template <int D>
@@ -595,11 +683,15 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, bool rope_q) {
     f.mask = a.mask; f.O = (uint16_t*)a.O; f.rope = a.rope;
     f.B = a.B; f.S = a.S; f.H = a.H; f.scale = a.scale; f.causal = a.causal;
     f.q_stride = a.q_stride; f.k_stride = a.k_stride; f.v_stride = a.v_stride; f.o_stride = a.o_stride;
-    dim3 grid((unsigned)((a.S + 127) / 128), (unsigned)a.H, (unsigned)a.B), block(256);
-    if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true>), grid, block, 0, c->stream, f);
-    else hipLaunchKernelGGL((fa2_bf16_kernel<D, false>), grid, block, 0, c->stream, f);
-    GRL_CHECK_LAUNCH();
-    return GRL_OK;
+    // GRL_FA_CFG forces a configuration, for tuning runs:
+    //   1: 8 waves x 32 queries, deep ring   3: 4 waves x 32 queries, 4 stages
+    static const int forced = [] { const char* e = getenv("GRL_FA_CFG"); return e ? atoi(e) : 0; }();
+    int cfg = forced == 1 || forced == 3 ? forced : (a.S > 128 ? 1 : 3);
+    constexpr int DEEP = D == 128 ? 4 : 8;        // 128 KiB of K/V tiles: D=128 -> 4 x 32 KiB, else 8 x 16 (8) KiB
+    switch (cfg) {
+        case 1: return launch_fa16_cfg<D, 1, 8, DEEP>(c, f, rope_q);
+        default: return launch_fa16_cfg<D, 1, 4, 4>(c, f, rope_q);
+    }
 }
 
 template <typename T, int D>
