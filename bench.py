@@ -10,7 +10,7 @@ Prints one JSON line: encoder tokens/s, plus
   kernels      -- the same measurement for every kernel of the layer (GEMMs and attention against
                   the MFMA peak, LayerNorm against 8 TB/s HBM);
   cpu_baseline -- the C restatement of the reference shaders (oracle/oracle.c) timed on the host
-                  cores on a bounded sample (one sequence through all 12 layers).
+                  cores on a bounded sample (--cpu-sequences of the 128 sequences through all 12 layers).
 """
 import argparse
 import ctypes
@@ -40,7 +40,7 @@ def time_launches(core, fn, reps, warm=3):
     return core.timer_stop() / reps
 
 
-def kernel_table(backend, enc, B, S, reps):
+def kernel_table(backend, enc, B, S, reps, only=None):
     """per-kernel average duration of one encoder layer's launches at the benchmark shape"""
     from grilly_amd import _lib as L
     cfg, c, lib, code = enc.cfg, backend.core, backend.core.lib, enc.code
@@ -69,6 +69,8 @@ def kernel_table(backend, enc, B, S, reps):
     ]
     out = {}
     for name, group, fn, flops, nbytes in runs:
+        if only and name not in only:
+            continue
         ms = time_launches(c, fn, reps)
         rec = {"ms": round(ms, 4), "group": group, "flops": flops, "bytes": nbytes}
         if flops:
@@ -82,23 +84,23 @@ def kernel_table(backend, enc, B, S, reps):
     return out
 
 
-def cpu_baseline(cfg, weights, seed):
-    """C restatement of the reference shaders on the host cores: ONE sequence of the workload
-    (S=512) through embeddings + all layers.  tokens/s = 512 / elapsed."""
+def cpu_baseline(cfg, weights, seed, nseq):
+    """C restatement of the reference shaders on the host cores: `nseq` sequences of the workload
+    (S=512 each) through embeddings + all layers.  tokens/s = nseq*512 / elapsed."""
     from oracle import oracle_np as O
     O.build()
     C = O.COracle()
     rng = np.random.default_rng(seed)
     S = 512
-    ids = rng.integers(0, cfg.vocab, (1, S))
+    ids = rng.integers(0, cfg.vocab, (nseq, S))
     t0 = time.perf_counter()
     x = C.layernorm(C.embed(ids, weights["tok_emb"], weights["pos_emb"], weights["type_emb"]),
                     weights["emb_ln_g"], weights["emb_ln_b"], cfg.eps)
     for lw in weights["layers"]:
         x = C.bert_layer(x, lw, None, cfg.heads, cfg.eps)
     dt = time.perf_counter() - t0
-    return {"value": round(S / dt, 2), "unit": "tokens/s", "cores": C.num_threads(), "kind": "port",
-            "sample": f"1 sequence x {S} tokens through embeddings + {cfg.layers} layers, fp32, "
+    return {"value": round(nseq * S / dt, 2), "unit": "tokens/s", "cores": C.num_threads(), "kind": "port",
+            "sample": f"{nseq} of the 128 sequences x {S} tokens through embeddings + {cfg.layers} layers, fp32, "
                       f"oracle/oracle.c (one-output-per-invocation shader loops, OpenMP over rows); {dt:.1f} s"}
 
 
@@ -113,10 +115,14 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "copy"],
+                    help="forward: the benchmark; gemm / copy: only launch the dominant GEMM kernel at its three "
+                         "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs)")
+    ap.add_argument("--cpu-sequences", type=int, default=12)
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one MI355X: this path has no multi-GPU leg (data-parallel sharding over "
-                 "batch needs no exchange; see DESIGN.md).  Run with --gpus 1.")
+                 "batch needs no exchange between GPUs).  Run with --gpus 1.")
 
     import grilly_amd
     from grilly_amd import BertEncoder, random_bert_weights
@@ -125,12 +131,28 @@ def main():
     seed = 20260131 + 3
     backend = grilly_amd.Compute(0)
     info = backend.device_info()
+    if a.mode == "copy":
+        # calibration for the HBM counters: a copy kernel that reads 1 GiB and writes 1 GiB per launch
+        c, nbytes = backend.core, 1 << 30
+        src, dst = c.alloc(nbytes), c.alloc(nbytes)
+        c.lib.grl_memset(c.ctx, src.ptr, 1, nbytes)
+        ms = time_launches(c, lambda: c.lib.grl_d2d(c.ctx, dst.ptr, src.ptr, nbytes), a.kernel_reps)
+        print(json.dumps({"mode": "copy", "kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes,
+                          "ms": round(ms, 4), "gbps": round(2 * nbytes / ms / 1e6, 1), "launches": a.kernel_reps + 3}))
+        backend.cleanup()
+        return
     weights = random_bert_weights(cfg, seed=seed)
     enc = BertEncoder(backend, cfg, weights, dtype=a.dtype)
     rng = np.random.default_rng(seed)
     B, S = a.batch, a.seq
     ids = rng.integers(0, cfg.vocab, (B, S))
     enc.set_inputs(ids, None)                 # no padding in this configuration
+
+    if a.mode == "gemm":
+        kt = kernel_table(backend, enc, B, S, a.kernel_reps, only=("gemm_qkv", "gemm_out", "gemm_ffn2"))
+        print(json.dumps({"mode": "gemm", "kernels": kt, "launches_each": a.kernel_reps + 3}))
+        backend.cleanup()
+        return
 
     for _ in range(a.warmup):
         enc.launch(pool=True)
@@ -167,13 +189,13 @@ def main():
         avg_flops = sum(r["flops"] for r in g) / 3
         avg_ms = sum(r["ms"] for r in g) / 3
         ach = avg_flops / (avg_ms * 1e-3) / 1e12
-        out["roofline"] = {"kernel": "gemm_nt_kernel<bf16,bf16,256,256,2,2,EPI_NONE>" if a.dtype == "bf16" else "gemm_nt_kernel<f32,f32,256,256,2,2,EPI_NONE>",
+        out["roofline"] = {"kernel": "gemm_nt_dma_kernel<bf16,bf16,256,256,2,4,EPI_NONE>" if a.dtype == "bf16" else "gemm_nt_dma_kernel<f32,f32,256,256,2,4,EPI_NONE>",
                            "bound": "mfma", "achieved": round(ach, 1), "peak": peak / 1e12, "unit": "TFLOP/s",
                            "frac": round(ach * 1e12 / peak, 4), "traffic": None,
                            "avg_launch_ms": round(avg_ms, 4), "flops_per_launch": avg_flops,
                            "launches_per_step": 3 * cfg.layers}
     if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, weights, seed)
+        out["cpu_baseline"] = cpu_baseline(cfg, weights, seed, a.cpu_sequences)
     backend.cleanup()
     print(json.dumps(out))
 

@@ -172,9 +172,14 @@ extern "C" int grl_d2h(grl_ctx* c, void* dst, const void* src, size_t bytes) {
     GRL_CHECK_HIP(hipStreamSynchronize(c->stream));
     return GRL_OK;
 }
+int grl_copy_kernel_launch(grl_ctx* c, void* dst, const void* src, size_t bytes);
+
 extern "C" int grl_d2d(grl_ctx* c, void* dst, const void* src, size_t bytes) {
     GRL_REQUIRE(c && (bytes == 0 || (dst && src)), GRL_ERR_ARG, "grl_d2d: null argument");
     if (!bytes) return GRL_OK;
+    // a plain copy kernel when everything is 16-byte granular (ordinary kernel launch on the
+    // context stream), else the runtime's copy
+    if ((((uintptr_t)dst | (uintptr_t)src | bytes) & 15u) == 0) return grl_copy_kernel_launch(c, dst, src, bytes);
     GRL_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, c->stream));
     return GRL_OK;
 }

@@ -37,6 +37,7 @@ struct GemmArgs {
     float* cache2;       // fp32 (M,N) pre-activation of W2 (SwiGLU up) or null
     int M, N, K;
     int tiles_m, tiles_n;
+    int group;           // tile-rows per band of the tile walk
 };
 
 enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
@@ -334,7 +335,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     auto tile_of = [&](int pid, int& m0, int& n0) {
         const int per = ntiles >> 3, rem = ntiles & 7, xcd = pid & 7, loc = pid >> 3;
         const int npid = xcd * per + (xcd < rem ? xcd : rem) + loc;
-        constexpr int GROUP = 8;
+        const int GROUP = p.group;
         const int width = GROUP * p.tiles_n;
         const int first_m = (npid / width) * GROUP;
         const int gsize = p.tiles_m - first_m < GROUP ? p.tiles_m - first_m : GROUP;
@@ -547,6 +548,9 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     // used once it yields enough workgroups to occupy most of the 256 CUs, else 128x128 tiles.
     // GRL_GEMM_VARIANT (1..4) forces one variant, for tuning runs.
     static const int forced = [] { const char* e = getenv("GRL_GEMM_VARIANT"); return e ? atoi(e) : 0; }();
+    // band height of the tile walk: rows of 8 KiB and more do better with narrow bands (measured)
+    static const int group = [] { const char* e = getenv("GRL_GEMM_GROUP"); return e ? atoi(e) : 0; }();
+    a.group = group > 0 ? group : (a.K * (int64_t)sizeof(T) >= 8192 ? 2 : 8);
     const int64_t bke = 128 / (int64_t)sizeof(T);
     const int64_t big_m = (a.M + 255) / 256, big_n = (a.N + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
     const int64_t sm = (a.M + 127) / 128, sn = (a.N + (DUAL ? 63 : 127)) / (DUAL ? 64 : 128);

@@ -254,6 +254,20 @@ extern "C" int grl_swiglu_act(grl_ctx* c, int dtype, int64_t rows, int64_t h, co
     return GRL_OK;
 }
 
+// ------------------------------------------------------------------ plain copy
+// 16 bytes per lane per step, grid-stride; moves every byte once in and once out.
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n16) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+int grl_copy_kernel_launch(grl_ctx* c, void* dst, const void* src, size_t bytes) {
+    const int64_t n16 = (int64_t)(bytes / 16);
+    hipLaunchKernelGGL(copy_kernel, dim3(ew_grid(n16)), dim3(256), 0, c->stream, (const u32x4*)src, (u32x4*)dst, n16);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
 // ------------------------------------------------------------------ casts
 template <typename S, typename D>
 __global__ __launch_bounds__(256) void cast_kernel(const S* __restrict__ s, D* __restrict__ d, int64_t n) {
