@@ -387,12 +387,12 @@ template <int IPT, int MAXT> __device__ __forceinline__ void wait_tiles_outstand
     }
 }
 
-template <int D, bool ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK>
+template <int D, bool ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK, int KT>
 __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
     // QT = 32-query MFMA tiles per wave (every K / V fragment read from LDS feeds QT MFMAs),
     // NW waves per workgroup, NSTG-deep ring of 64-key K/V tiles in LDS (NSTG-1 tiles in flight).
     constexpr int RB = D * 2, NCH = RB / 16, NS = D / 16;
-    constexpr int KT = 64, NKB = 2, DT = D / 32;
+    constexpr int NKB = KT / 32, DT = D / 32;     // KT keys per tile (64 or 128)
     constexpr int TILE = KT * RB;
     constexpr int NT = NW * 64;
     constexpr int TPO = TILE / 1024;              // 1 KiB transfers per tile and operand
@@ -459,12 +459,15 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
                                                      (k0 + lane * 4) * 4, 0, 0, 0);
     };
 
-    f32x16 oacc[QT][DT];
-    float m_run[QT], l_run[QT];
+    // lacc: row sums of P, accumulated by the matrix core against an all-ones operand (every
+    // register of a lane then holds the full sum for that lane's query); only register 0 is kept exact
+    f32x16 oacc[QT][DT], lacc[QT];
+    float m_run[QT];
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
         m_run[t] = -1.4426950408889634e10f;      // -1e10 in the base-2 domain
-        l_run[t] = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) lacc[t][r] = 0.f;
 #pragma unroll
         for (int d = 0; d < DT; ++d)
 #pragma unroll
@@ -472,12 +475,12 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
     }
     const float c2 = p.scale * 1.4426950408889634f;
 
-    for (int t = 0; t < NSTG - 1 && t < nkt; ++t) issue(t);
+    issue(0);
 
     // this wave's queries as MFMA "B" operand: slab s holds dims (2s+lg)*8 .. +7 of query li.
-    // Loaded after the first tiles were requested so that both latencies overlap; the explicit
-    // wait below retires these loads before the loop, which lets the waits inside the loop count
-    // only the tile transfers issued there.
+    // Loaded right after the first tile was requested and before the rest of the ring, so the
+    // counted wait below (transfers return in order) retires tile 0 and these loads together while
+    // the later tiles are still in flight; inside the loop only tile transfers remain to be counted.
     u32x4 qf[QT][NS];
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
@@ -497,7 +500,8 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
         }
     }
 
-    wait_vmcnt<0>();
+    for (int t = 1; t < NSTG - 1 && t < nkt; ++t) issue(t);
+    wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1);
 
     for (int kt = 0; kt < nkt; ++kt) {
         const int st = kt % NSTG, k0 = kt * KT;
@@ -544,6 +548,7 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
         const bool diag = p.causal && (k0 + KT - 1 > qw0);
         const bool tail = k0 + KT > S;
         const bool biased = HAS_MASK || tail;
+        float pmul[QT], pneg[QT];     // p = exp2(score * pmul + pneg), formed block by block below
         sfor<QT>([&](auto iu) {
             constexpr int u = decltype(iu)::value;
             const int qi = qw0 + 32 * u + li;
@@ -568,13 +573,8 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
                     }
                 });
                 mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m_run[u], mx);
-                sfor<NKB>([&](auto it) {
-                    constexpr int t = decltype(it)::value;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) sacc[u][t][r] = __builtin_amdgcn_exp2f(sacc[u][t][r] - m_new);
-                });
-                mx = m_new;
+                mx = fmaxf(m_run[u], mx);
+                pmul[u] = 1.0f;          // scores are already scaled and biased
             } else {
                 // plain tile: the max is taken on the raw products (c2 > 0) and the scale rides in the fma
                 sfor<NKB>([&](auto it) {
@@ -583,25 +583,14 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
                     for (int r = 0; r < 16; r += 2) mx = __builtin_fmaxf(mx, __builtin_fmaxf(sacc[u][t][r], sacc[u][t][r + 1]));
                 });
                 mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m_run[u], mx * c2);
-                const float nm = -m_new;
-                sfor<NKB>([&](auto it) {
-                    constexpr int t = decltype(it)::value;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) sacc[u][t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][t][r], c2, nm));
-                });
-                mx = m_new;
+                mx = fmaxf(m_run[u], mx * c2);
+                pmul[u] = c2;
             }
-            float psum = 0.f;
-            sfor<NKB>([&](auto it) {
-                constexpr int t = decltype(it)::value;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) psum += sacc[u][t][r];
-            });
+            pneg[u] = -mx;
             const float alpha = __builtin_amdgcn_exp2f(m_run[u] - mx);
-            l_run[u] = l_run[u] * alpha + psum;
-            // rescale the output only when some row of the wave raised its maximum
+            // rescale the running output and sum only when some row of the wave raised its maximum
             if (__builtin_amdgcn_ballot_w64(mx != m_run[u]) != 0) {
+                lacc[u][0] *= alpha;
                 sfor<DT>([&](auto idt) {
                     constexpr int dt = decltype(idt)::value;
 #pragma unroll
@@ -618,11 +607,20 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
             constexpr int t = decltype(it)::value;
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
+                // exponentials of this 16-key slab only: they are independent of the MFMAs of the previous
+                // slab, which lets the VALU work run under the matrix work instead of ahead of it
                 u32x4 pf[QT];
 #pragma unroll
                 for (int u = 0; u < QT; ++u)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) pf[u][e] = pack_bf16x2(sacc[u][t][8 * hh + 2 * e], sacc[u][t][8 * hh + 2 * e + 1]);
+                    for (int e = 0; e < 4; ++e) {
+                        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][t][8 * hh + 2 * e], pmul[u], pneg[u]));
+                        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][t][8 * hh + 2 * e + 1], pmul[u], pneg[u]));
+                        pf[u][e] = pack_bf16x2(p0, p1);
+                    }
+                // row sums: P^T against an all-ones (bf16 1.0) operand
+                const u32x4 ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+                sfor<QT>([&](auto iu) { Slab<uint16_t>::run(ones, pf[decltype(iu)::value], lacc[decltype(iu)::value]); });
                 // keys of MFMA k-index (g, e): 32t + 16hh + 8*(e/4) + 4g + e%4, g = lane/32
                 const int kA = 32 * t + 16 * hh + 4 * (grp >> 1) + (j16 >> 2);
                 sfor<DT>([&](auto idt) {
@@ -646,8 +644,7 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
 #pragma unroll
     for (int u = 0; u < QT; ++u) {
         const int qi = qw0 + 32 * u + li;
-        const float l_tot = l_run[u] + __shfl_xor(l_run[u], 32, 64);
-        const float inv = 1.0f / fmaxf(l_tot, 1e-10f);
+        const float inv = 1.0f / fmaxf(lacc[u][0], 1e-10f);
         if (qi < S) {
             uint16_t* Og = p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
 #pragma unroll
@@ -661,16 +658,16 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
     }
 }
 
-template <int D, int QT, int NW, int NSTG>
+template <int D, int QT, int NW, int NSTG, int KT>
 static int launch_fa16_cfg(grl_ctx* c, const Fa16Args& f, bool rope_q) {
     const int qb = 32 * QT * NW;
     dim3 grid((unsigned)((f.S + qb - 1) / qb), (unsigned)f.H, (unsigned)f.B), block(NW * 64);
     if (f.mask) {
-        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, true>), grid, block, 0, c->stream, f);
-        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, true>), grid, block, 0, c->stream, f);
+        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, true, KT>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, true, KT>), grid, block, 0, c->stream, f);
     } else {
-        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, false>), grid, block, 0, c->stream, f);
-        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, false>), grid, block, 0, c->stream, f);
+        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, false, KT>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, false, KT>), grid, block, 0, c->stream, f);
     }
     GRL_CHECK_LAUNCH();
     return GRL_OK;
@@ -684,13 +681,14 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, bool rope_q) {
     f.B = a.B; f.S = a.S; f.H = a.H; f.scale = a.scale; f.causal = a.causal;
     f.q_stride = a.q_stride; f.k_stride = a.k_stride; f.v_stride = a.v_stride; f.o_stride = a.o_stride;
     // GRL_FA_CFG forces a configuration, for tuning runs:
-    //   1: 8 waves x 32 queries, deep ring   3: 4 waves x 32 queries, 4 stages
+    //   1: 8 waves, 64-key tiles, deep ring   2: 8 waves, 128-key tiles   3: 4 waves, 64-key tiles, 4 stages
     static const int forced = [] { const char* e = getenv("GRL_FA_CFG"); return e ? atoi(e) : 0; }();
-    int cfg = forced == 1 || forced == 3 ? forced : (a.S > 128 ? 1 : 3);
+    int cfg = forced >= 1 && forced <= 3 ? forced : (a.S > 128 ? 2 : 3);
     constexpr int DEEP = D == 128 ? 4 : 8;        // 128 KiB of K/V tiles: D=128 -> 4 x 32 KiB, else 8 x 16 (8) KiB
     switch (cfg) {
-        case 1: return launch_fa16_cfg<D, 1, 8, DEEP>(c, f, rope_q);
-        default: return launch_fa16_cfg<D, 1, 4, 4>(c, f, rope_q);
+        case 1: return launch_fa16_cfg<D, 1, 8, DEEP, 64>(c, f, rope_q);
+        case 2: return launch_fa16_cfg<D, 1, 8, DEEP / 2, 128>(c, f, rope_q);
+        default: return launch_fa16_cfg<D, 1, 4, 4, 64>(c, f, rope_q);
     }
 }
 
