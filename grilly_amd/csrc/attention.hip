@@ -425,11 +425,11 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
     auto make_rsrc = [&](const uint16_t* base, int64_t stride) {
         int64_t bytes = (int64_t)(S - 1) * stride * 2 + RB;
         uint32_t nrec = bytes > 0xffffffffLL ? 0xffffffffu : (uint32_t)bytes;
-        return __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)b * S * stride + h * D), 0, (int)nrec, 0x00020000);
+        return make_rsrc_words(base + (int64_t)b * S * stride + h * D, nrec);
     };
-    const __amdgpu_buffer_rsrc_t rsK = make_rsrc(p.K, p.k_stride);
-    const __amdgpu_buffer_rsrc_t rsV = make_rsrc(p.V, p.v_stride);
-    const __amdgpu_buffer_rsrc_t rsM = __builtin_amdgcn_make_buffer_rsrc((void*)(p.mask ? p.mask + (int64_t)b * S : (const float*)p.Q), 0, HAS_MASK ? S * 4 : 0, 0x00020000);
+    const rsrc_words rsK = make_rsrc(p.K, p.k_stride);
+    const rsrc_words rsV = make_rsrc(p.V, p.v_stride);
+    const rsrc_words rsM = make_rsrc_words(p.mask ? (const void*)(p.mask + (int64_t)b * S) : (const void*)p.Q, HAS_MASK ? (uint32_t)S * 4u : 0u);
     const int kstride_b = (int)p.k_stride * 2, vstride_b = (int)p.v_stride * 2;
     // lane -> (row, slot) inside one 1 KiB transfer; the slot holds chunk slot ^ swizzle(row)
     const int t_row = lane / NCH, t_slot = lane % NCH;
@@ -444,19 +444,14 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
             const int row = inst * RPI + t_row;
             const int chunk = NCH >= 8 ? (t_slot ^ (row & 7)) : (t_slot ^ ((row >> 1) & 3));
             const int rowg = k0 + row;
-            if (isv)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsV, (__attribute__((address_space(3))) void*)(lds + OFF_V + st * TILE + inst * 1024), 16,
-                                                         rowg * vstride_b + chunk * 16, 0, 0, 0);
-            else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsK, (__attribute__((address_space(3))) void*)(lds + st * TILE + inst * 1024), 16,
-                                                         rowg * kstride_b + chunk * 16, 0, 0, 0);
+            if (isv) dma16(rsV, lds + OFF_V + st * TILE + inst * 1024, rowg * vstride_b + chunk * 16);
+            else dma16(rsK, lds + st * TILE + inst * 1024, rowg * kstride_b + chunk * 16);
         }
         // raw mask values of the tile's 64 keys (256 B; the transfer unit is 1 KiB per wave, lanes
         // past the tile read further mask entries or out of range, which nobody uses).  Every wave
         // issues it so that all waves count the same number of transfers per tile.
         if (HAS_MASK)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsM, (__attribute__((address_space(3))) void*)(lds + OFF_M + st * 1024), 16,
-                                                     (k0 + lane * 4) * 4, 0, 0, 0);
+            dma16(rsM, lds + OFF_M + st * 1024, (k0 + lane * 4) * 4);
     };
 
     // lacc: row sums of P, accumulated by the matrix core against an all-ones operand (every

@@ -93,6 +93,25 @@ __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uin
 __device__ __forceinline__ float bf16lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
 __device__ __forceinline__ float bf16hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 
+// ---- global -> LDS transfer the compiler does not see (buffer_load_dwordx4 ... lds).
+// The wave writes 64 x 16 B to LDS at lds_dst (wave-uniform) + lane*16; each lane fetches from
+// resource base + voff; lanes whose voff is out of range transfer zeros.  Issued through inline
+// asm so that the compiler's wait-count insertion does not treat it as a pending LDS write that
+// later LDS accesses (notably the transposing reads) must fully wait for; the caller places the
+// s_waitcnt vmcnt(N) itself.
+typedef __attribute__((ext_vector_type(4))) int rsrc_words;
+__device__ __forceinline__ rsrc_words make_rsrc_words(const void* base, uint32_t num_bytes) {
+    const uint64_t a = (uint64_t)base;
+    // wave-uniform by construction; readfirstlane tells the compiler so (the words must sit in SGPRs)
+    rsrc_words r = {(int)__builtin_amdgcn_readfirstlane((uint32_t)a), (int)__builtin_amdgcn_readfirstlane((uint32_t)((a >> 32) & 0xffffu)),
+                    (int)__builtin_amdgcn_readfirstlane(num_bytes), 0x00020000};
+    return r;
+}
+__device__ __forceinline__ void dma16(rsrc_words rs, const void* lds_dst_wave_uniform, int voff) {
+    const uint32_t la = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)lds_dst_wave_uniform);
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(la), "v"(voff), "s"(rs) : "memory");
+}
+
 template <typename T> struct elem;
 template <> struct elem<float> {
     static __device__ __forceinline__ float ld(const float* p) { return *p; }
