@@ -409,9 +409,16 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lg = lane >> 5;
-    const int b = blockIdx.z, h = blockIdx.y;
-    const int qb = p.causal ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
-    const int q0 = qb * QB, S = p.S;
+    // 1-D grid.  Dense: query blocks of one (batch, head) are adjacent so that they share its K/V in L2.
+    // Causal: all (batch, head) pairs of the heaviest query block first, then the next lighter one ...
+    // (longest work first keeps the CUs evenly loaded whatever the dispatch order does).
+    const int S = p.S;
+    const int nqb = (S + QB - 1) / QB, nbh = p.B * p.H;
+    int qb, bh;
+    if (p.causal) { qb = nqb - 1 - (int)blockIdx.x / nbh; bh = (int)blockIdx.x % nbh; }
+    else { qb = (int)blockIdx.x % nqb; bh = (int)blockIdx.x / nqb; }
+    const int b = bh / p.H, h = bh % p.H;
+    const int q0 = qb * QB;
     const int qw0 = q0 + wave * QW;               // first query of this wave
     const uint16_t* Qg = p.Q + (int64_t)b * S * p.q_stride + h * D;
 
@@ -656,7 +663,7 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
 template <int D, int QT, int NW, int NSTG, int KT>
 static int launch_fa16_cfg(grl_ctx* c, const Fa16Args& f, bool rope_q) {
     const int qb = 32 * QT * NW;
-    dim3 grid((unsigned)((f.S + qb - 1) / qb), (unsigned)f.H, (unsigned)f.B), block(NW * 64);
+    dim3 grid((unsigned)(((f.S + qb - 1) / qb) * f.H * f.B)), block(NW * 64);
     if (f.mask) {
         if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, true, KT>), grid, block, 0, c->stream, f);
         else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, true, KT>), grid, block, 0, c->stream, f);
