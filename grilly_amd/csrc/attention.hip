@@ -24,6 +24,8 @@
 #include <cstdlib>
 
 int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling);
+int grl_rope_apply_table(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                         void* y, const float* table);
 int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
                      const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling);
 
@@ -752,7 +754,7 @@ static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t
             // every K row is rotated exactly once here; the kernel rotates Q rows as it loads them
             own2 = grl_malloc(c, (size_t)B * S * H * D * 2);
             if (!own2) { grl_free(c, own); return GRL_ERR_OOM; }
-            rc = grl_rope_strided(c, dtype, B, S, H, D, K, k_stride, nullptr, own2, GRL_ROPE_INTERLEAVED, rope_base, rope_scaling);
+            rc = grl_rope_apply_table(c, dtype, B, S, H, D, K, k_stride, own2, (const float*)own);
             a.K = own2; a.k_stride = hd;
         }
     }

@@ -376,6 +376,54 @@ int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float
     return GRL_OK;
 }
 
+// Interleaved RoPE from a precomputed (S, D/2) {cos, sin} table: one 16-byte chunk per thread,
+// every row read once and written once (the K pre-rotation of the fused-RoPE attention path).
+template <typename T>
+__global__ __launch_bounds__(256) void rope_table_apply_kernel(const T* __restrict__ x, int64_t x_stride, T* __restrict__ y,
+                                                              const float2* __restrict__ tab, int64_t nchunks, int S, int H, int D) {
+    constexpr int EPC = 16 / (int)sizeof(T), PPC = EPC / 2;
+    const int cpr = D / EPC;                       // chunks per (position, head) row
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nchunks; i += stride) {
+        const int c = (int)(i % cpr);
+        const int64_t vec = i / cpr;               // (b,s,h) flat
+        const int64_t bs = vec / H;
+        const int h = (int)(vec - bs * H), s = (int)(bs % S);
+        u32x4 v = *(const u32x4*)(x + bs * x_stride + (int64_t)h * D + c * EPC);
+        const float2* t = tab + (int64_t)s * (D / 2) + c * PPC;
+        u32x4 o;
+        if (sizeof(T) == 2) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float2 cs = t[j];
+                const float x0 = bf16lo(v[j]), x1 = bf16hi(v[j]);
+                o[j] = pack_bf16x2(x0 * cs.x - x1 * cs.y, x0 * cs.y + x1 * cs.x);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const float2 cs = t[j];
+                const float x0 = u2f(v[2 * j]), x1 = u2f(v[2 * j + 1]);
+                o[2 * j] = f2u(x0 * cs.x - x1 * cs.y);
+                o[2 * j + 1] = f2u(x0 * cs.y + x1 * cs.x);
+            }
+        }
+        *(u32x4*)(y + vec * D + c * EPC) = o;
+    }
+}
+
+int grl_rope_apply_table(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                         void* y, const float* table) {
+    const int64_t epc = dtype == GRL_BF16 ? 8 : 4;
+    const int64_t nchunks = B * S * H * (D / epc);
+    if (nchunks == 0) return GRL_OK;
+    dim3 g(ew_grid(nchunks)), b(256);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(rope_table_apply_kernel<float>, g, b, 0, c->stream, (const float*)x, x_stride, (float*)y, (const float2*)table, nchunks, (int)S, (int)H, (int)D);
+    else hipLaunchKernelGGL(rope_table_apply_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, x_stride, (uint16_t*)y, (const float2*)table, nchunks, (int)S, (int)H, (int)D);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
 // ------------------------------------------------------------------ embedding gather
 template <typename T>
 __global__ __launch_bounds__(256) void embed_kernel(const int32_t* __restrict__ ids, const float* __restrict__ tok,
