@@ -390,7 +390,7 @@ template <int IPT, int MAXT> __device__ __forceinline__ void wait_tiles_outstand
 }
 
 template <int D, bool ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK, int KT>
-__global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16Args p) {
     // QT = 32-query MFMA tiles per wave (every K / V fragment read from LDS feeds QT MFMAs),
     // NW waves per workgroup, NSTG-deep ring of 64-key K/V tiles in LDS (NSTG-1 tiles in flight).
     constexpr int RB = D * 2, NCH = RB / 16, NS = D / 16;
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(NW * 64) void fa2_bf16_kernel(Fa16Args p) {
     constexpr int RPI = 1024 / RB;                // tile rows per transfer
     constexpr int QW = 32 * QT, QB = NW * QW;     // queries per wave / per workgroup
     static_assert((2 * TPO) % NW == 0 && 2 * TPO >= NW, "transfers must divide over the waves");
-    static_assert(IPT * (NSTG - 1) < 64, "vmcnt is a 6-bit counter");
+    static_assert(NSTG >= 2 && IPT * (NSTG - 1) < 64, "ring of at least two stages; vmcnt is a 6-bit counter");
     // ONE LDS array with manual offsets: with several __shared__ objects the compiler tracks the
     // LDS-DMA transfers per object and puts a full vmcnt(0) in front of every LDS read of a ring
     // that has a transfer in flight, which would serialise the prefetch.
@@ -686,12 +686,16 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, bool rope_q) {
     f.q_stride = a.q_stride; f.k_stride = a.k_stride; f.v_stride = a.v_stride; f.o_stride = a.o_stride;
     // GRL_FA_CFG forces a configuration, for tuning runs:
     //   1: 8 waves, 64-key tiles, deep ring   2: 8 waves, 128-key tiles   3: 4 waves, 64-key tiles, 4 stages
+    //   4: 4 waves, 128-key tiles, half-size ring (two workgroups per CU)
     static const int forced = [] { const char* e = getenv("GRL_FA_CFG"); return e ? atoi(e) : 0; }();
-    int cfg = forced >= 1 && forced <= 3 ? forced : (a.S > 128 ? 2 : 3);
+    // short sequences: two small workgroups per CU hide each other's start-up and store tails;
+    // long ones: one 8-wave workgroup with the full ring
+    int cfg = forced >= 1 && forced <= 4 ? forced : (a.S > 1024 ? 2 : (a.S > 128 ? 4 : 3));
     constexpr int DEEP = D == 128 ? 4 : 8;        // 128 KiB of K/V tiles: D=128 -> 4 x 32 KiB, else 8 x 16 (8) KiB
     switch (cfg) {
         case 1: return launch_fa16_cfg<D, 1, 8, DEEP, 64>(c, f, rope_q);
         case 2: return launch_fa16_cfg<D, 1, 8, DEEP / 2, 128>(c, f, rope_q);
+        case 4: return launch_fa16_cfg<D, 1, 4, 2, (D == 128 ? 64 : 128)>(c, f, rope_q);
         default: return launch_fa16_cfg<D, 1, 4, 4, 64>(c, f, rope_q);
     }
 }
