@@ -28,6 +28,12 @@ PEAK_BF16 = 2.5e15      # MI355X dense bf16 MFMA, FLOP/s
 PEAK_FP32 = 157.3e12
 PEAK_HBM = 8.0e12       # B/s
 
+# HBM bytes per launch of the plain bf16 GEMM kernel, mean over its three layer shapes at batch 128 x seq 512:
+# rocprofv3 --pmc FETCH_SIZE (x2, the factor a 1 GiB copy kernel calibrates) + --pmc WRITE_SIZE (x1) on
+# `bench.py --mode gemm`; summary in profiles/gemm_bf16_bert_shapes_hbm_traffic.md.  A profiler reading, not
+# something this script can measure itself, so it is reported only for exactly that workload.
+GEMM_TRAFFIC_BYTES = {("bf16", 128, 512): 622.6e6}
+
 
 def time_launches(core, fn, reps, warm=3):
     """average milliseconds of one call of fn() (which only enqueues), HIP events on the context stream"""
@@ -84,6 +90,56 @@ def kernel_table(backend, enc, B, S, reps, only=None):
     return out
 
 
+def fill_normal(core, nbytes_elems, rng, std, code):
+    """device buffer of `nbytes_elems` elements ~N(0,std), tiled from a 4 Mi-element random block"""
+    from grilly_amd import _lib as L
+    es = 2 if code == L.GRL_BF16 else 4
+    blk = (rng.standard_normal(1 << 22) * std).astype(np.float32)
+    src = core.upload(blk, code)
+    dst = core.alloc(nbytes_elems * es)
+    off = 0
+    while off < nbytes_elems * es:
+        m = min(blk.size * es, nbytes_elems * es - off)
+        L.check(core.lib.grl_d2d(core.ctx, dst.ptr + off, src.ptr, m))
+        off += m
+    core.sync()
+    src.free()
+    return dst
+
+
+def side_workload(backend, mode, seed, reps):
+    """the two single-operator configurations: long causal attention with RoPE, and the SwiGLU MLP"""
+    from grilly_amd import _lib as L
+    c, lib, code = backend.core, backend.core.lib, L.GRL_BF16
+    rng = np.random.default_rng(seed)
+    if mode == "fa2_long":
+        B, H, S, D = 4, 32, 8192, 128
+        n = B * S * H * D
+        q, k, v = (fill_normal(c, n, rng, 1.0, code) for _ in range(3))
+        o = c.alloc(n * 2)
+        fn = lambda: L.check(lib.grl_fa2_fwd(c.ctx, code, B, S, H, D, q.ptr, k.ptr, v.ptr, None, o.ptr,
+                                             1.0 / np.sqrt(D), 1, L.ROPE_INTERLEAVED, 1e4, 1.0, None))
+        ms = time_launches(c, fn, reps)
+        flops = 4.0 * B * H * S * S * D * 0.5    # causal: half of the score matrix
+        return {"mode": mode, "workload": "BASELINE configs[4]: causal FA2 forward with RoPE, (B,S,H,D)=(4,8192,32,128), bf16",
+                "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_mfma": round(flops / (ms * 1e-3) / PEAK_BF16, 4),
+                "flops": flops, "includes": "cos/sin table kernel + K pre-rotation kernel + attention kernel (buffers from the caching pool)", "launches": reps + 3}
+    M, Kd, F = 16384, 4096, 11008
+    x = fill_normal(c, M * Kd, rng, 1.0, code)
+    wg, wu = fill_normal(c, F * Kd, rng, 0.02, code), fill_normal(c, F * Kd, rng, 0.02, code)
+    wd = fill_normal(c, Kd * F, rng, 0.02, code)
+    h, y = c.alloc(M * F * 2), c.alloc(M * Kd * 2)
+    f1 = lambda: L.check(lib.grl_swiglu_nt(c.ctx, code, code, M, F, Kd, x.ptr, wg.ptr, wu.ptr, None, None, h.ptr, None, None))
+    f2 = lambda: L.check(lib.grl_gemm_nt(c.ctx, code, code, M, Kd, F, h.ptr, wd.ptr, None, y.ptr, 0))
+    ms1, ms2 = time_launches(c, f1, reps), time_launches(c, f2, reps)
+    fl1, fl2 = 4.0 * M * F * Kd, 2.0 * M * F * Kd
+    return {"mode": mode, "workload": "BASELINE configs[3]: X[16384,4096] . (W_g,W_u)[11008,4096]^T -> silu(up)*gate -> . W_d[4096,11008]^T, bf16",
+            "gate_up_swiglu": {"ms": round(ms1, 4), "tflops": round(fl1 / ms1 / 1e9, 1), "frac_mfma": round(fl1 / (ms1 * 1e-3) / PEAK_BF16, 4)},
+            "down": {"ms": round(ms2, 4), "tflops": round(fl2 / ms2 / 1e9, 1), "frac_mfma": round(fl2 / (ms2 * 1e-3) / PEAK_BF16, 4)},
+            "total_ms": round(ms1 + ms2, 4), "tflops": round((fl1 + fl2) / (ms1 + ms2) / 1e9, 1),
+            "frac_mfma": round((fl1 + fl2) / ((ms1 + ms2) * 1e-3) / PEAK_BF16, 4), "launches_each": reps + 3}
+
+
 def cpu_baseline(cfg, weights, seed, nseq):
     """C restatement of the reference shaders on the host cores: `nseq` sequences of the workload
     (S=512 each) through embeddings + all layers.  tokens/s = nseq*512 / elapsed."""
@@ -115,9 +171,11 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
-    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "copy"],
+    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "copy", "fa2_long", "swiglu_mlp"],
                     help="forward: the benchmark; gemm / copy: only launch the dominant GEMM kernel at its three "
-                         "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs)")
+                         "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs); fa2_long: "
+                         "causal attention with RoPE at batch 4, 32 heads, seq 8192, head dim 128, bf16; swiglu_mlp: "
+                         "X[16384,4096] through gate/up [11008,4096] + silu*up + down [4096,11008], bf16")
     ap.add_argument("--cpu-sequences", type=int, default=12)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -139,6 +197,10 @@ def main():
         ms = time_launches(c, lambda: c.lib.grl_d2d(c.ctx, dst.ptr, src.ptr, nbytes), a.kernel_reps)
         print(json.dumps({"mode": "copy", "kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes,
                           "ms": round(ms, 4), "gbps": round(2 * nbytes / ms / 1e6, 1), "launches": a.kernel_reps + 3}))
+        backend.cleanup()
+        return
+    if a.mode in ("fa2_long", "swiglu_mlp"):
+        print(json.dumps(side_workload(backend, a.mode, seed, a.kernel_reps)))
         backend.cleanup()
         return
     weights = random_bert_weights(cfg, seed=seed)
@@ -191,7 +253,9 @@ def main():
         ach = avg_flops / (avg_ms * 1e-3) / 1e12
         out["roofline"] = {"kernel": "gemm_nt_dma_kernel<bf16,bf16,256,256,2,4,EPI_NONE>" if a.dtype == "bf16" else "gemm_nt_dma_kernel<f32,f32,256,256,2,4,EPI_NONE>",
                            "bound": "mfma", "achieved": round(ach, 1), "peak": peak / 1e12, "unit": "TFLOP/s",
-                           "frac": round(ach * 1e12 / peak, 4), "traffic": None,
+                           "frac": round(ach * 1e12 / peak, 4),
+                           "traffic": GEMM_TRAFFIC_BYTES.get((a.dtype, B, S)),
+                           "algorithmic_bytes": sum(r["bytes"] for r in g) / 3,
                            "avg_launch_ms": round(avg_ms, 4), "flops_per_launch": avg_flops,
                            "launches_per_step": 3 * cfg.layers}
     if not a.no_cpu_baseline:
