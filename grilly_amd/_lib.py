@@ -10,7 +10,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libgrilly_hip.so")
+# GRILLY_HIP_LIB points at another build of the same library (comparing two builds on one machine)
+LIB_PATH = os.environ.get("GRILLY_HIP_LIB") or os.path.join(_HERE, "lib", "libgrilly_hip.so")
 
 GRL_F32, GRL_BF16 = 0, 1
 EPI_NONE, EPI_GELU, EPI_SILU = 0, 1, 2

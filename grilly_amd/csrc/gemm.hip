@@ -493,7 +493,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                     const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
                     const int n = n0 + cc * EPCO;
                     if (m < p.M && n < p.N)
-                        *(u32x4*)(C + (int64_t)m * p.N + n) = *(const u32x4*)(reg + r * CROWB + ((cc ^ (r & (CPR - 1))) << 4));
+                        // written once, read by another kernel: keep it from displacing the operand panels in L2
+                        __builtin_nontemporal_store(*(const u32x4*)(reg + r * CROWB + ((cc ^ (r & (CPR - 1))) << 4)), (u32x4*)(C + (int64_t)m * p.N + n));
                 }
                 if (NREG == 1) __syncthreads();
             });

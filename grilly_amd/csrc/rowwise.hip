@@ -12,6 +12,9 @@ template <> struct vec4<float> {
     f32x4 v;
     __device__ __forceinline__ void load(const float* p) { v = *(const f32x4*)p; }
     __device__ __forceinline__ void store(float* p) const { *(f32x4*)p = v; }
+    // streaming variants: data that is touched once should not displace what other kernels keep in L2
+    __device__ __forceinline__ void load_stream(const float* p) { v = __builtin_nontemporal_load((const f32x4*)p); }
+    __device__ __forceinline__ void store_stream(float* p) const { __builtin_nontemporal_store(v, (f32x4*)p); }
     __device__ __forceinline__ float get(int i) const { return v[i]; }
     __device__ __forceinline__ void set(int i, float f) { v[i] = f; }
 };
@@ -19,6 +22,8 @@ template <> struct vec4<uint16_t> {
     u32x2 w;
     __device__ __forceinline__ void load(const uint16_t* p) { w = *(const u32x2*)p; }
     __device__ __forceinline__ void store(uint16_t* p) const { *(u32x2*)p = w; }
+    __device__ __forceinline__ void load_stream(const uint16_t* p) { w = __builtin_nontemporal_load((const u32x2*)p); }
+    __device__ __forceinline__ void store_stream(uint16_t* p) const { __builtin_nontemporal_store(w, (u32x2*)p); }
     __device__ __forceinline__ float get(int i) const {
         uint32_t x = w[i >> 1];
         return (i & 1) ? bf16hi(x) : bf16lo(x);
@@ -57,9 +62,9 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     for (int c = 0; c < MAXC; ++c) {
         int ch = lane + c * 64;
         if (ch < nch) {
-            vec4<T> a; a.load(xr + ch * 4);
+            vec4<T> a; a.load_stream(xr + ch * 4);
             if (HAS_RES) {
-                vec4<T> b; b.load(rr + ch * 4);
+                vec4<T> b; b.load_stream(rr + ch * 4);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) t[c][i] = a.get(i) + b.get(i);
             } else {
@@ -94,7 +99,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
             vec4<T> o;
 #pragma unroll
             for (int i = 0; i < 4; ++i) o.set(i, g[i] * ((t[c][i] - mean) / sd) + b[i]);
-            o.store(yr + ch * 4);
+            o.store_stream(yr + ch * 4);
         }
     }
 }
