@@ -322,7 +322,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     constexpr int RG = WGM * 32 * CROWB;                    // one staging region
     constexpr int NREG = 2 * RG <= STAGE ? 2 : 1;
     static_assert(RG <= STAGE && (CPR & (CPR - 1)) == 0, "output staging must fit in LDS stage 1");
-    __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
+    constexpr int BIASB = BN * 4;                           // one tile's bias slice(s), fp32
+    __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + 2 * BIASB];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -373,6 +374,20 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                                                      lane_off + (b_row0_glb + j * 8) * (int)rowbytes, sbyte, 0, 0);
     };
 
+    // The bias slice of a tile travels to LDS with the tile's first slab (two buffers, alternating per
+    // tile), so the epilogue reads it with LDS latency instead of one global round trip per column group.
+    // Wave 0 fetches bias[n0 .. n0+BNO), the first wave of the upper half bias2 (columns past N read zero).
+    auto issue_bias = [&](int n0t, int buf) {
+        const bool w1 = wave == 0 && p.bias, w2 = DUAL && wave == NW / 2 && p.bias2;
+        if ((w1 || w2) && lane < BNO / 4) {
+            const float* src = (w2 ? p.bias2 : p.bias) + n0t;
+            int left = (p.N - n0t) * 4;
+            __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, left > 0 ? left : 0, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + 2 * STAGE + buf * BIASB + (w2 ? BNO * 4 : 0)),
+                                                     16, lane * 16, 0, 0, 0);
+        }
+    };
+
     int rowX[TM], rowW[TN];
 #pragma unroll
     for (int a = 0; a < TM; ++a) rowX[a] = wm * WM + a * 32 + li;
@@ -393,6 +408,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     __amdgpu_buffer_rsrc_t rsA = make_rsrc(p.A, m0, p.M);
     __amdgpu_buffer_rsrc_t rsW = make_rsrc(Wsrc, n0, p.N);
     issue(rsA, rsW, 0);
+    int bbuf = 0;
+    issue_bias(n0, bbuf);
 
     for (;;) {
         f32x16 acc[TM][TN];
@@ -436,73 +453,79 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             rsAn = make_rsrc(p.A, m0n, p.M);
             rsWn = make_rsrc(Wsrc, n0n, p.N);
             issue(rsAn, rsWn, 0);
+            issue_bias(n0n, bbuf ^ 1);
         }
 
         if (staged) {
             // ---- LDS-staged epilogue in stage 1, one 32-row band of every wave-row per pass
             constexpr int EPCO = 16 / OES;
             char* stg = lds + STAGE;
+            const char* bias_lds = lds + 2 * STAGE + bbuf * BIASB;
+            // bias of this lane's 4-column groups, once per tile (columns past N hold zero)
+            f32x4 bv1[TNO][4], bv2[TNO][4];
+#pragma unroll
+            for (int b = 0; b < TNO; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
+                    bv1[b][q] = p.bias ? *(const f32x4*)(bias_lds + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                    if (DUAL) bv2[b][q] = p.bias2 ? *(const f32x4*)(bias_lds + BNO * 4 + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                }
             static_for<TM>([&](auto ia) {
                 constexpr int a = decltype(ia)::value;
                 char* reg = stg + (NREG == 2 ? (a & 1) * RG : 0);
                 const int r_w = wm * 32 + li;
                 char* crow = reg + r_w * CROWB;
+                // columns past N carry zero accumulators (their weight rows read as zero); they are
+                // converted like the rest and dropped at the global store
                 static_for<TNO>([&](auto ib) {
                     constexpr int b = decltype(ib)::value;
                     static_for<4>([&](auto iq) {
                         constexpr int q = decltype(iq)::value;
                         const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
-                        const int n = n0 + nl;
                         float v[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e];
-                        if (n < p.N) {     // N % 4 == 0 here, so the 4 columns are in or out together
-                            if (p.bias) {
-                                f32x4 bv = *(const f32x4*)(p.bias + n);
+                        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] + bv1[b][q][e];
+                        if (DUAL) {
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) v[e] += bv[e];
-                            }
-                            if (DUAL) {
-                                float u[4];
+                            for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(acc[a][DUAL ? b + TNO : b][4 * q + e] + bv2[b][q][e]);
+                        } else {
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) u[e] = acc[a][DUAL ? b + TNO : b][4 * q + e];
-                                if (p.bias2) {
-                                    f32x4 bv = *(const f32x4*)(p.bias2 + n);
-#pragma unroll
-                                    for (int e = 0; e < 4; ++e) u[e] += bv[e];
-                                }
-#pragma unroll
-                                for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(u[e]);
-                            } else {
-#pragma unroll
-                                for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
-                            }
+                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
                         }
                         const int byte = nl * OES;
                         const int chunk = (byte >> 4) ^ (r_w & (CPR - 1));
                         store4<OutT>((OutT*)(crow + (chunk << 4) + (byte & 15)), v[0], v[1], v[2], v[3]);
                     });
                 });
-                __syncthreads();
+                // LDS-only barrier: a fence here would also wait for the global stores of the pass before
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
                 constexpr int TOTAL = WGM * 32 * CPR;
                 static_assert(TOTAL % NT == 0, "staged chunks divide over the threads");
+                constexpr int PER = TOTAL / NT;
+                u32x4 val[PER];
 #pragma unroll
-                for (int i = 0; i < TOTAL / NT; ++i) {
+                for (int i = 0; i < PER; ++i) {
+                    const int id = tid + i * NT;
+                    const int r = id / CPR, cc = id % CPR;
+                    val[i] = *(const u32x4*)(reg + r * CROWB + ((cc ^ (r & (CPR - 1))) << 4));
+                }
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
                     const int id = tid + i * NT;
                     const int r = id / CPR, cc = id % CPR;
                     const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
                     const int n = n0 + cc * EPCO;
-                    if (m < p.M && n < p.N)
-                        // written once, read by another kernel: keep it from displacing the operand panels in L2
-                        __builtin_nontemporal_store(*(const u32x4*)(reg + r * CROWB + ((cc ^ (r & (CPR - 1))) << 4)), (u32x4*)(C + (int64_t)m * p.N + n));
+                    // written once, read by another kernel: keep it from displacing the operand panels in L2
+                    if (m < p.M && n < p.N) __builtin_nontemporal_store(val[i], (u32x4*)(C + (int64_t)m * p.N + n));
                 }
-                if (NREG == 1) __syncthreads();
+                if (NREG == 1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             });
         } else {
             epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
         }
         if (!has_next) break;
-        pid = npid; m0 = m0n; n0 = n0n; rsA = rsAn; rsW = rsWn;
+        pid = npid; m0 = m0n; n0 = n0n; rsA = rsAn; rsW = rsWn; bbuf ^= 1;
     }
 }
 
