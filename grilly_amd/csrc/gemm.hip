@@ -420,6 +420,17 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
+        // where the next tile is: index arithmetic done here hides under the wait for the first slab
+        const int npid = pid + (int)gridDim.x;
+        const bool has_next = npid < ntiles;
+        int m0n = 0, n0n = 0;
+        __amdgpu_buffer_rsrc_t rsAn = rsA, rsWn = rsW;
+        if (has_next) {
+            tile_of(npid, m0n, n0n);
+            rsAn = make_rsrc(p.A, m0n, p.M);
+            rsWn = make_rsrc(Wsrc, n0n, p.N);
+        }
+
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's transfers (and earlier stores) are done
         __syncthreads();                         // ... and everybody else's; all staging reads of the last tile too
         for (int kt = 0; kt < KT; ++kt) {
@@ -444,14 +455,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
         }
 
         // both LDS stages are free now: request the next tile's first slab into stage 0
-        const int npid = pid + (int)gridDim.x;
-        const bool has_next = npid < ntiles;
-        int m0n = 0, n0n = 0;
-        __amdgpu_buffer_rsrc_t rsAn = rsA, rsWn = rsW;
         if (has_next) {
-            tile_of(npid, m0n, n0n);
-            rsAn = make_rsrc(p.A, m0n, p.M);
-            rsWn = make_rsrc(Wsrc, n0n, p.N);
             issue(rsAn, rsWn, 0);
             issue_bias(n0n, bbuf ^ 1);
         }
@@ -471,13 +475,16 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                     bv1[b][q] = p.bias ? *(const f32x4*)(bias_lds + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
                     if (DUAL) bv2[b][q] = p.bias2 ? *(const f32x4*)(bias_lds + BNO * 4 + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
                 }
-            static_for<TM>([&](auto ia) {
+            constexpr int TOTAL = WGM * 32 * CPR;
+            static_assert(TOTAL % NT == 0, "staged chunks divide over the threads");
+            constexpr int PER = TOTAL / NT;
+            const int r_w = wm * 32 + li;
+            // bias/activation/convert band `a` of every wave-row into its staging region.  Columns past N
+            // carry zero accumulators (their weight rows read as zero); they are converted like the rest
+            // and dropped at the global store.
+            auto stage_band = [&](auto ia) {
                 constexpr int a = decltype(ia)::value;
-                char* reg = stg + (NREG == 2 ? (a & 1) * RG : 0);
-                const int r_w = wm * 32 + li;
-                char* crow = reg + r_w * CROWB;
-                // columns past N carry zero accumulators (their weight rows read as zero); they are
-                // converted like the rest and dropped at the global store
+                char* crow = stg + (NREG == 2 ? (a & 1) * RG : 0) + r_w * CROWB;
                 static_for<TNO>([&](auto ib) {
                     constexpr int b = decltype(ib)::value;
                     static_for<4>([&](auto iq) {
@@ -498,18 +505,19 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                         store4<OutT>((OutT*)(crow + (chunk << 4) + (byte & 15)), v[0], v[1], v[2], v[3]);
                     });
                 });
-                // LDS-only barrier: a fence here would also wait for the global stores of the pass before
-                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                constexpr int TOTAL = WGM * 32 * CPR;
-                static_assert(TOTAL % NT == 0, "staged chunks divide over the threads");
-                constexpr int PER = TOTAL / NT;
-                u32x4 val[PER];
+            };
+            auto fetch_band = [&](auto ia, u32x4 (&val)[PER]) {
+                constexpr int a = decltype(ia)::value;
+                const char* reg = stg + (NREG == 2 ? (a & 1) * RG : 0);
 #pragma unroll
                 for (int i = 0; i < PER; ++i) {
                     const int id = tid + i * NT;
                     const int r = id / CPR, cc = id % CPR;
                     val[i] = *(const u32x4*)(reg + r * CROWB + ((cc ^ (r & (CPR - 1))) << 4));
                 }
+            };
+            auto store_band = [&](auto ia, const u32x4 (&val)[PER]) {
+                constexpr int a = decltype(ia)::value;
 #pragma unroll
                 for (int i = 0; i < PER; ++i) {
                     const int id = tid + i * NT;
@@ -519,8 +527,30 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                     // written once, read by another kernel: keep it from displacing the operand panels in L2
                     if (m < p.M && n < p.N) __builtin_nontemporal_store(val[i], (u32x4*)(C + (int64_t)m * p.N + n));
                 }
-                if (NREG == 1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            });
+            };
+            // Barriers here are LDS-only (a fence would also wait for the global stores of earlier bands).
+            if constexpr (NREG == 2) {
+                // two regions: band a+1 is converted and written while band a's staged rows are on their
+                // way back from LDS, one barrier per band
+                stage_band(std::integral_constant<int, 0>{});
+                static_for<TM>([&](auto ia) {
+                    constexpr int a = decltype(ia)::value;
+                    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    u32x4 val[PER];
+                    fetch_band(ia, val);
+                    if constexpr (a + 1 < TM) stage_band(std::integral_constant<int, a + 1>{});
+                    store_band(ia, val);
+                });
+            } else {
+                static_for<TM>([&](auto ia) {
+                    stage_band(ia);
+                    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    u32x4 val[PER];
+                    fetch_band(ia, val);
+                    store_band(ia, val);
+                    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                });
+            }
         } else {
             epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
         }
