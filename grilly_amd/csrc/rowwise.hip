@@ -462,10 +462,45 @@ extern "C" int grl_embed(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F,
 }
 
 // ------------------------------------------------------------------ masked mean pool (+ L2 normalise)
-// grid (ceil(F/256), B): thread f sums its feature over the sequence (coalesced across f).
+// grid (ceil(F/256), B).  F % 4 == 0: a lane owns 4 adjacent features (8- or 16-byte loads), the 4 waves
+// of a workgroup take every 4th position of the sequence and their partial sums meet in LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void mean_pool_kernel(const T* __restrict__ x, const float* __restrict__ mask,
                                                        float* __restrict__ out, int S, int F) {
+    __shared__ float part[4][256];
+    __shared__ float cpart[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int f0 = blockIdx.x * 256 + lane * 4;
+    const int64_t b = blockIdx.y;
+    float a[4] = {0.f, 0.f, 0.f, 0.f}, cnt = 0.f;
+    const T* xb = x + b * S * (int64_t)F + f0;
+    const bool live = f0 < F;
+#pragma unroll 8
+    for (int s = wave; s < S; s += 4) {
+        const float m = mask ? mask[b * S + s] : 1.0f;
+        cnt += m;
+        if (live) {
+            vec4<T> v; v.load_stream(xb + (int64_t)s * F);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] += m * v.get(i);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][lane * 4 + i] = a[i];
+    if (lane == 0) cpart[wave] = cnt;
+    __syncthreads();
+    const int f = blockIdx.x * 256 + threadIdx.x;
+    if (f < F) {
+        const float tot = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+        const float c = (cpart[0] + cpart[1]) + (cpart[2] + cpart[3]);
+        out[b * F + f] = tot / fmaxf(c, 1e-9f);
+    }
+}
+
+// any F: thread f sums its feature over the sequence (coalesced across f)
+template <typename T>
+__global__ __launch_bounds__(256) void mean_pool_generic_kernel(const T* __restrict__ x, const float* __restrict__ mask,
+                                                               float* __restrict__ out, int S, int F) {
     const int f = blockIdx.x * 256 + threadIdx.x;
     const int64_t b = blockIdx.y;
     if (f >= F) return;
@@ -497,8 +532,14 @@ extern "C" int grl_mean_pool(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_
     GRL_REQUIRE(B >= 0 && B < 65536 && S > 0 && F > 0 && S < (1LL << 31) && F < (1LL << 31), GRL_ERR_SHAPE, "grl_mean_pool: bad shape");
     if (B == 0) return GRL_OK;
     dim3 g((unsigned)((F + 255) / 256), (unsigned)B), b(256);
-    if (dtype == GRL_F32) hipLaunchKernelGGL(mean_pool_kernel<float>, g, b, 0, c->stream, (const float*)x, mask, out, (int)S, (int)F);
-    else hipLaunchKernelGGL(mean_pool_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, mask, out, (int)S, (int)F);
+    const bool vec = F % 4 == 0 && aligned16(x);
+    if (dtype == GRL_F32) {
+        if (vec) hipLaunchKernelGGL(mean_pool_kernel<float>, g, b, 0, c->stream, (const float*)x, mask, out, (int)S, (int)F);
+        else hipLaunchKernelGGL(mean_pool_generic_kernel<float>, g, b, 0, c->stream, (const float*)x, mask, out, (int)S, (int)F);
+    } else {
+        if (vec) hipLaunchKernelGGL(mean_pool_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, mask, out, (int)S, (int)F);
+        else hipLaunchKernelGGL(mean_pool_generic_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, mask, out, (int)S, (int)F);
+    }
     GRL_CHECK_LAUNCH();
     if (l2_normalize) {
         hipLaunchKernelGGL(l2_normalize_kernel, dim3((unsigned)B), dim3(256), 0, c->stream, out, (int)F);

@@ -132,6 +132,25 @@ def test_embed_and_mean_pool(backend):
         t.free()
 
 
+@pytest.mark.parametrize("dtype,F", [("f32", 390), ("f32", 301), ("bf16", 768), ("bf16", 250), ("bf16", 37)])
+def test_mean_pool_shapes(backend, dtype, F):
+    """vector path (F % 4 == 0, also with a ragged last 256-feature block) and the any-F path"""
+    rng = np.random.default_rng(F)
+    B, S = 5, 77
+    code = L.GRL_BF16 if dtype == "bf16" else L.GRL_F32
+    x = rng.standard_normal((B, S, F)).astype(np.float32)
+    if dtype == "bf16":
+        x = O.bf16_round(x)
+    m = (np.arange(S)[None] < np.array([77, 1, 40, 76, 3])[:, None]).astype(np.float32)
+    c = backend.core
+    dx, dm, do = c.upload(x, code), c.upload(m), c.alloc(B * F * 4)
+    for l2 in (0, 1):
+        L.check(c.lib.grl_mean_pool(c.ctx, code, B, S, F, dx.ptr, dm.ptr, do.ptr, l2))
+        assert O.max_rel(c.download(do, (B, F)), O.truth_mean_pool(x, m, l2=bool(l2))) < 1e-5
+    for t in (dx, dm, do):
+        t.free()
+
+
 def test_c_abi_argument_errors(backend):
     c = backend.core
     lib = c.lib
