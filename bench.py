@@ -35,7 +35,10 @@ PEAK_HBM = 8.0e12       # B/s
 GEMM_TRAFFIC_BYTES = {("bf16", 128, 512): 608.2e6}
 
 
-def time_launches(core, fn, reps, warm=3):
+WARM = 5
+
+
+def time_launches(core, fn, reps, warm=WARM):
     """average milliseconds of one call of fn() (which only enqueues), HIP events on the context stream"""
     for _ in range(warm):
         fn()
@@ -123,7 +126,7 @@ def side_workload(backend, mode, seed, reps):
         flops = 4.0 * B * H * S * S * D * 0.5    # causal: half of the score matrix
         return {"mode": mode, "workload": "BASELINE configs[4]: causal FA2 forward with RoPE, (B,S,H,D)=(4,8192,32,128), bf16",
                 "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_mfma": round(flops / (ms * 1e-3) / PEAK_BF16, 4),
-                "flops": flops, "includes": "cos/sin table kernel + K pre-rotation kernel + attention kernel (buffers from the caching pool)", "launches": reps + 3}
+                "flops": flops, "includes": "cos/sin table kernel + K pre-rotation kernel + attention kernel (buffers from the caching pool)", "launches": reps + WARM}
     M, Kd, F = 16384, 4096, 11008
     x = fill_normal(c, M * Kd, rng, 1.0, code)
     wg, wu = fill_normal(c, F * Kd, rng, 0.02, code), fill_normal(c, F * Kd, rng, 0.02, code)
@@ -137,7 +140,7 @@ def side_workload(backend, mode, seed, reps):
             "gate_up_swiglu": {"ms": round(ms1, 4), "tflops": round(fl1 / ms1 / 1e9, 1), "frac_mfma": round(fl1 / (ms1 * 1e-3) / PEAK_BF16, 4)},
             "down": {"ms": round(ms2, 4), "tflops": round(fl2 / ms2 / 1e9, 1), "frac_mfma": round(fl2 / (ms2 * 1e-3) / PEAK_BF16, 4)},
             "total_ms": round(ms1 + ms2, 4), "tflops": round((fl1 + fl2) / (ms1 + ms2) / 1e9, 1),
-            "frac_mfma": round((fl1 + fl2) / ((ms1 + ms2) * 1e-3) / PEAK_BF16, 4), "launches_each": reps + 3}
+            "frac_mfma": round((fl1 + fl2) / ((ms1 + ms2) * 1e-3) / PEAK_BF16, 4), "launches_each": reps + WARM}
 
 
 def cpu_baseline(cfg, weights, seed, nseq):
@@ -171,9 +174,10 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
-    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "copy", "fa2_long", "swiglu_mlp"],
+    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "kernels", "copy", "fa2_long", "swiglu_mlp"],
                     help="forward: the benchmark; gemm / copy: only launch the dominant GEMM kernel at its three "
-                         "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs); fa2_long: "
+                         "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs); kernels: every kernel of "
+                         "the layer at its layer shape, nothing else (counter runs); fa2_long: "
                          "causal attention with RoPE at batch 4, 32 heads, seq 8192, head dim 128, bf16; swiglu_mlp: "
                          "X[16384,4096] through gate/up [11008,4096] + silu*up + down [4096,11008], bf16")
     ap.add_argument("--cpu-sequences", type=int, default=12)
@@ -196,7 +200,7 @@ def main():
         c.lib.grl_memset(c.ctx, src.ptr, 1, nbytes)
         ms = time_launches(c, lambda: c.lib.grl_d2d(c.ctx, dst.ptr, src.ptr, nbytes), a.kernel_reps)
         print(json.dumps({"mode": "copy", "kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes,
-                          "ms": round(ms, 4), "gbps": round(2 * nbytes / ms / 1e6, 1), "launches": a.kernel_reps + 3}))
+                          "ms": round(ms, 4), "gbps": round(2 * nbytes / ms / 1e6, 1), "launches": a.kernel_reps + WARM}))
         backend.cleanup()
         return
     if a.mode in ("fa2_long", "swiglu_mlp"):
@@ -210,9 +214,10 @@ def main():
     ids = rng.integers(0, cfg.vocab, (B, S))
     enc.set_inputs(ids, None)                 # no padding in this configuration
 
-    if a.mode == "gemm":
-        kt = kernel_table(backend, enc, B, S, a.kernel_reps, only=("gemm_qkv", "gemm_out", "gemm_ffn2"))
-        print(json.dumps({"mode": "gemm", "kernels": kt, "launches_each": a.kernel_reps + 3}))
+    if a.mode in ("gemm", "kernels"):
+        only = ("gemm_qkv", "gemm_out", "gemm_ffn2") if a.mode == "gemm" else None
+        kt = kernel_table(backend, enc, B, S, a.kernel_reps, only=only)
+        print(json.dumps({"mode": a.mode, "kernels": kt, "launches_each": a.kernel_reps + WARM}))
         backend.cleanup()
         return
 

@@ -193,7 +193,7 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
             u32x4 v = kreg[i];
             if (ROPE) v = rope_chunk<T>(v, kcs[i]);
             if (k0 + key >= S) v = zero;
-            const int slot = NCH >= 8 ? (c ^ (key & 7)) : (c ^ ((key >> 1) & 3));
+            const int slot = c ^ lds_swz<NCH>(key);
             *(u32x4*)(Kb + key * RB + slot * 16) = v;
         }
         if (BF) {
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 const int c = 2 * s + lg;
-                const int slot = NCH >= 8 ? (c ^ (key & 7)) : (c ^ ((key >> 1) & 3));
+                const int slot = c ^ lds_swz<NCH>(key);
                 u32x4 kf = *(const u32x4*)(Kb + key * RB + slot * 16);
                 Slab<T>::run(kf, qf[s], sacc[t]);
             }
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
             const bool isv = g >= TPO;
             const int inst = isv ? g - TPO : g;
             const int row = inst * RPI + t_row;
-            const int chunk = NCH >= 8 ? (t_slot ^ (row & 7)) : (t_slot ^ ((row >> 1) & 3));
+            const int chunk = t_slot ^ (isv ? lds_swz_v<NCH>(row) : lds_swz<NCH>(row));
             const int rowg = k0 + row;
             if (isv) dma16(rsV, lds + OFF_V + st * TILE + inst * 1024, rowg * vstride_b + chunk * 16);
             else dma16(rsK, lds + st * TILE + inst * 1024, rowg * kstride_b + chunk * 16);
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 const int c = 2 * s + lg;
-                const int slot = NCH >= 8 ? (c ^ (key & 7)) : (c ^ ((key >> 1) & 3));
+                const int slot = c ^ lds_swz<NCH>(key);
                 u32x4 kf = *(const u32x4*)(Kb + key * RB + slot * 16);
                 sfor<QT>([&](auto iu) { Slab<uint16_t>::run(kf, qf[decltype(iu)::value][s], sacc[decltype(iu)::value][t]); });
             }
@@ -632,7 +632,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
                     const int dcol = 32 * dt + 16 * (grp & 1) + 4 * (j16 & 3);     // first of 4 dims this lane points at
                     const int ch = dcol >> 3, sub = (dcol & 7) * 2;
                     auto addr = [&](int key) {
-                        const int slot = NCH >= 8 ? (ch ^ (key & 7)) : (ch ^ ((key >> 1) & 3));
+                        const int slot = ch ^ lds_swz_v<NCH>(key);
                         return (__attribute__((address_space(3))) s16x4_t*)(Vb + key * RB + slot * 16 + sub);
                     };
                     s16x4_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16(addr(kA));

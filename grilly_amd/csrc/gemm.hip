@@ -17,8 +17,8 @@
 // output row: stores are 8 B (bf16) / 16 B (fp32) wide and bias is a 4-vector per lane.
 //
 // LDS bank behaviour: a tile row is 128 B = 8 chunks of 16 B; chunk c of row r lives at
-// slot c ^ (r & 7).  Eight consecutive lanes (eight consecutive rows, same logical chunk)
-// therefore hit eight different slots = all 32 banks once, for the reads as for the writes.
+// slot c ^ lds_swz<8>(r), which makes 16 consecutive rows of one logical chunk (what 16 lanes of a
+// ds_read_b128 fragment read touch) cover all 64 banks exactly once.
 #include "common.hpp"
 #include <type_traits>
 #include <cstdlib>
@@ -208,7 +208,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
     const __amdgpu_buffer_rsrc_t rsW2 = make_rsrc(DUAL ? p.W2 : p.W, n0, p.N);
     const int voff = row_t * (int)rowbytes + c_t * 16;
     const int pass_stride = RPP * (int)rowbytes;
-    const int soff_t = row_t * 128 + ((c_t ^ (row_t & 7)) << 4);
+    static_assert(RPP % 16 == 0, "the swizzle repeats every 16 rows");
+    const int soff_t = row_t * 128 + ((c_t ^ lds_swz<8>(row_t)) << 4);
 
     u32x4 ra[CA], rb[CB];
     auto load_slab = [&](int kt) {
@@ -266,9 +267,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
             const int ch = 2 * sl + lg;
             u32x4 xf[TM], wf[TN];
 #pragma unroll
-            for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ (rowX[a] & 7)) << 4));
+            for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ lds_swz<8>(rowX[a])) << 4));
 #pragma unroll
-            for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ (rowW[b] & 7)) << 4));
+            for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ lds_swz<8>(rowW[b])) << 4));
             static_for<TM>([&](auto ia) {
                 static_for<TN>([&](auto ib) {
                     MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
@@ -355,8 +356,10 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     const bool second = DUAL && (wave >= NW / 2);
     const void* Wsrc = second ? p.W2 : p.W;
     const int lr = lane >> 3, ls = lane & 7;
-    // lane -> (row lr of the group, chunk ls ^ lr): LDS slot ls of row r holds chunk ls ^ (r & 7)
-    const int lane_off = lr * (int)rowbytes + ((ls ^ lr) << 4);
+    // lane -> (row lr of an 8-row group, slot ls): LDS slot ls of row r holds chunk ls ^ lds_swz<8>(r).
+    // The swizzle depends on bits 1-3 of r, i.e. on lr and on whether the group is an even or odd one.
+    static_assert(GA % 2 == 0 && GB % 2 == 0, "group parity is the transfer index parity");
+    const int lane_off_p[2] = {lr * (int)rowbytes + ((ls ^ lds_swz<8>(lr)) << 4), lr * (int)rowbytes + ((ls ^ lds_swz<8>(8 + lr)) << 4)};
     const int a_row0 = wave * GA * 8;                                    // first A tile row of this wave
     const int b_row0_lds = wave * GB * 8;                                // LDS row in the weight region
     const int b_row0_glb = second ? b_row0_lds - BNO : b_row0_lds;       // row relative to n0 in its matrix
@@ -367,11 +370,11 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
 #pragma unroll
         for (int j = 0; j < GA; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (__attribute__((address_space(3))) void*)(st + (a_row0 + j * 8) * 128), 16,
-                                                     lane_off + (a_row0 + j * 8) * (int)rowbytes, sbyte, 0, 0);
+                                                     lane_off_p[j & 1] + (a_row0 + j * 8) * (int)rowbytes, sbyte, 0, 0);
 #pragma unroll
         for (int j = 0; j < GB; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (__attribute__((address_space(3))) void*)(st + BM * 128 + (b_row0_lds + j * 8) * 128), 16,
-                                                     lane_off + (b_row0_glb + j * 8) * (int)rowbytes, sbyte, 0, 0);
+                                                     lane_off_p[j & 1] + (b_row0_glb + j * 8) * (int)rowbytes, sbyte, 0, 0);
     };
 
     // The bias slice of a tile travels to LDS with the tile's first slab (two buffers, alternating per
@@ -441,9 +444,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                 const int ch = 2 * sl + lg;
                 u32x4 xf[TM], wf[TN];
 #pragma unroll
-                for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ (rowX[a] & 7)) << 4));
+                for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ lds_swz<8>(rowX[a])) << 4));
 #pragma unroll
-                for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ (rowW[b] & 7)) << 4));
+                for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ lds_swz<8>(rowW[b])) << 4));
                 static_for<TM>([&](auto ia) {
                     static_for<TN>([&](auto ib) {
                         MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
