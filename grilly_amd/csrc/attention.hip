@@ -372,6 +372,7 @@ struct Fa16Args {
     int B, S, H;
     float scale;
     int causal;
+    int order;            // workgroup -> (head, query block) map, see fa2_bf16_kernel
     int64_t q_stride, k_stride, v_stride, o_stride;
 };
 
@@ -411,14 +412,20 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lg = lane >> 5;
-    // 1-D grid.  Dense: query blocks of one (batch, head) are adjacent so that they share its K/V in L2.
-    // Causal: all (batch, head) pairs of the heaviest query block first, then the next lighter one ...
-    // (longest work first keeps the CUs evenly loaded whatever the dispatch order does).
+    // 1-D grid; p.order picks the workgroup -> (batch*head, query block) map: bit 0 renumbers the ids per XCD,
+    // bit 1 puts the heaviest query blocks of all heads first (causal), else heads are walked one by one
+    // (causal: each head's heavy blocks first) so that neighbours share that head's K/V in L2.
     const int S = p.S;
     const int nqb = (S + QB - 1) / QB, nbh = p.B * p.H;
+    // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2: `lin` renumbers them so
+    // that every XCD walks one contiguous run, and workgroups that run side by side on an XCD are
+    // neighbours in `lin`.
+    const int nwg = (int)gridDim.x, per = nwg >> 3, rem = nwg & 7, xcd = (int)blockIdx.x & 7, loc = (int)blockIdx.x >> 3;
+    const int lin = (p.order & 1) ? xcd * per + (xcd < rem ? xcd : rem) + loc : (int)blockIdx.x;
     int qb, bh;
-    if (p.causal) { qb = nqb - 1 - (int)blockIdx.x / nbh; bh = (int)blockIdx.x % nbh; }
-    else { qb = (int)blockIdx.x % nqb; bh = (int)blockIdx.x / nqb; }
+    if (p.order & 2) { qb = nqb - 1 - lin / nbh; bh = lin % nbh; }            // heaviest query blocks of all heads first
+    else if (p.causal) { bh = lin / nqb; qb = nqb - 1 - lin % nqb; }          // head by head, heavy blocks first
+    else { qb = lin % nqb; bh = lin / nqb; }                                  // head by head
     const int b = bh / p.H, h = bh % p.H;
     const int q0 = qb * QB;
     const int qw0 = q0 + wave * QW;               // first query of this wave
@@ -683,6 +690,10 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, bool rope_q) {
     f.Q = (const uint16_t*)a.Q; f.K = (const uint16_t*)a.K; f.V = (const uint16_t*)a.V;
     f.mask = a.mask; f.O = (uint16_t*)a.O; f.rope = a.rope;
     f.B = a.B; f.S = a.S; f.H = a.H; f.scale = a.scale; f.causal = a.causal;
+    static const int order_env = [] { const char* e = getenv("GRL_FA_ORDER"); return e ? atoi(e) : -1; }();
+    // measured: causal and short sequences do best head by head on XCD-contiguous runs; long dense sequences with
+    // the plain id order (32 CUs of an XCD streaming the same K/V tiles in lockstep miss L2 together)
+    f.order = order_env >= 0 ? order_env : ((a.causal || a.S <= 1024) ? 1 : 0);
     f.q_stride = a.q_stride; f.k_stride = a.k_stride; f.v_stride = a.v_stride; f.o_stride = a.o_stride;
     // GRL_FA_CFG forces a configuration, for tuning runs:
     //   1: 8 waves, 64-key tiles, deep ring   2: 8 waves, 128-key tiles   3: 4 waves, 64-key tiles, 4 stages
