@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("GRILLY_HIP_LIB") or os.path.join(_HERE, "lib", "libgrilly_hip.so")
 
 GRL_F32, GRL_BF16 = 0, 1
-EPI_NONE, EPI_GELU, EPI_SILU = 0, 1, 2
+EPI_NONE, EPI_GELU, EPI_SILU, EPI_RELU, EPI_GCU, EPI_ROSWISH = 0, 1, 2, 3, 4, 5
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALF = 0, 1, 2
 ERR_ARG, ERR_SHAPE, ERR_HIP, ERR_OOM = -1, -2, -3, -4
 
@@ -58,6 +58,8 @@ SIGNATURES = {
     "grl_gemm_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
     "grl_gemm_nn": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "grl_swiglu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 8),
+    "grl_glu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 8 + [c_int]),
+    "grl_gemm_nt_act": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 4 + [c_int, c_float, c_float]),
     "grl_fa2_fwd": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64] + [c_void_p] * 5 + [c_float, c_int, c_int, c_float, c_float, c_void_p]),
     "grl_fa2_fwd_strided": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64] + [c_void_p] * 5 + [c_i64] * 4 + [c_float, c_int, c_int, c_float, c_float]),
     "grl_rope": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float]),

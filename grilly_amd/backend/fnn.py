@@ -42,7 +42,7 @@ class HipFNN:
         return self.core.pool_stats()
 
     # ------------------------------------------------------------------ GEMM family
-    def _linear_impl(self, x, weights, bias, epi, dtype):
+    def _linear_impl(self, x, weights, bias, epi, dtype, alpha=1.0, beta=1.0):
         code = dtype_code(dtype)
         W = np.asarray(weights)
         if W.ndim != 2:
@@ -57,7 +57,8 @@ class HipFNN:
         db = c.upload(np.asarray(bias).reshape(-1)) if bias is not None else None
         dy = c.alloc(M * N * (2 if code == L.GRL_BF16 else 4))
         try:
-            L.check(c.lib.grl_gemm_nt(c.ctx, code, code, M, N, K, dx.ptr, dw.ptr, db.ptr if db else None, dy.ptr, epi), "gemm_nt")
+            L.check(c.lib.grl_gemm_nt_act(c.ctx, code, code, M, N, K, dx.ptr, dw.ptr, db.ptr if db else None, dy.ptr, epi,
+                                          float(alpha), float(beta)), "gemm_nt")
             return c.download(dy, (M, N), code)
         finally:
             for b in (dx, dw, db, dy):
@@ -91,6 +92,53 @@ class HipFNN:
         """SiLU(x.W^T + b) in one kernel (reference backend/fnn.py:2214-2303)."""
         x = np.asarray(x)
         return self._fused_shape(x, self._linear_impl(x, weights, bias, L.EPI_SILU, dtype))
+
+    def fused_linear_relu(self, x, weights, bias=None, dtype="fp32"):
+        """ReLU(x.W^T + b) in one kernel (reference backend/fnn.py:2125-2212)."""
+        x = np.asarray(x)
+        return self._fused_shape(x, self._linear_impl(x, weights, bias, L.EPI_RELU, dtype))
+
+    def fused_linear_gcu(self, x, weights, bias=None, dtype="fp32"):
+        """GCU(s) = s*cos(s) on s = x.W^T + b in one kernel (reference backend/fnn.py:2307-2383)."""
+        x = np.asarray(x)
+        return self._fused_shape(x, self._linear_impl(x, weights, bias, L.EPI_GCU, dtype))
+
+    def fused_linear_roswish(self, x, weights, bias=None, alpha=1.0, beta=1.0, dtype="fp32"):
+        """RoSwish(s) = (s+alpha)*sigmoid(beta*s) - alpha/2 on s = x.W^T + b in one kernel
+        (reference backend/fnn.py:2385-2470)."""
+        x = np.asarray(x)
+        return self._fused_shape(x, self._linear_impl(x, weights, bias, L.EPI_ROSWISH, dtype, alpha, beta))
+
+    def fused_layernorm_linear(self, x, gamma, beta, weights, bias=None, eps=1e-5, dtype="fp32"):
+        """Linear(LayerNorm(x)) (reference shaders/fused-layernorm-linear.glsl:67-128; the reference has no host
+        wrapper for it): the row-normalising kernel and the GEMM run back to back on the device, the
+        normalised rows never leave it (on the bf16 path they are rounded to bf16 between the two)."""
+        code = dtype_code(dtype)
+        W = np.asarray(weights)
+        if W.ndim != 2:
+            raise ValueError("weights must be (out_features, in_features)")
+        N, K = W.shape
+        x = np.asarray(x)
+        x2 = _as2d(x, K)
+        M = x2.shape[0]
+        g, bt = np.asarray(gamma, np.float32).reshape(-1), np.asarray(beta, np.float32).reshape(-1)
+        if g.size != K or bt.size != K:
+            raise ValueError("gamma/beta must have `in_features` elements")
+        if bias is not None and np.asarray(bias).size != N:
+            raise ValueError(f"bias has {np.asarray(bias).size} elements, expected {N}")
+        c = self.core
+        es = 2 if code == L.GRL_BF16 else 4
+        dx, dw, dg, dbt = c.upload(x2, code), c.upload(W, code), c.upload(g), c.upload(bt)
+        db = c.upload(np.asarray(bias).reshape(-1)) if bias is not None else None
+        dn, dy = c.alloc(max(M * K, 1) * es), c.alloc(max(M * N, 1) * es)
+        try:
+            L.check(c.lib.grl_layernorm(c.ctx, code, M, K, dx.ptr, None, dg.ptr, dbt.ptr, float(eps), dn.ptr), "layernorm")
+            L.check(c.lib.grl_gemm_nt(c.ctx, code, code, M, N, K, dn.ptr, dw.ptr, db.ptr if db else None, dy.ptr, L.EPI_NONE), "gemm_nt")
+            return self._fused_shape(x, c.download(dy, (M, N), code))
+        finally:
+            for t in (dx, dw, dg, dbt, db, dn, dy):
+                if t is not None:
+                    t.free()
 
     def fused_qkv_projection(self, x, W_qkv, b_qkv=None, num_heads=None, head_dim=None, dtype="fp32"):
         """QKV = x.[Wq;Wk;Wv]^T + [bq;bk;bv] -> (..., 3*H*D); Q is columns [0,H*D), K the next
@@ -131,6 +179,17 @@ class HipFNN:
         """(x.Wg^T + bg) * SiLU(x.Wu^T + bu), output always 2-D (M, hidden)
         (reference backend/_glu_append.py:8-129; SiLU is on the UP projection,
         shaders/fused-swiglu.glsl:76-78; biases only when both are given, :68)."""
+        return self._glu_impl(x, W_gate, W_up, b_gate, b_up, return_cache, dtype, L.EPI_SILU)
+
+    def fused_reglu(self, x, W_gate, W_up, b_gate=None, b_up=None, return_cache=False, dtype="fp32"):
+        """(x.Wg^T + bg) * ReLU(x.Wu^T + bu) (reference backend/_glu_append.py:131-222, shaders/fused-reglu.glsl:42-75)."""
+        return self._glu_impl(x, W_gate, W_up, b_gate, b_up, return_cache, dtype, L.EPI_RELU)
+
+    def fused_geglu(self, x, W_gate, W_up, b_gate=None, b_up=None, return_cache=False, dtype="fp32"):
+        """(x.Wg^T + bg) * GELU_tanh(x.Wu^T + bu) (reference backend/_glu_append.py:224-315, shaders/fused-geglu.glsl:43-82)."""
+        return self._glu_impl(x, W_gate, W_up, b_gate, b_up, return_cache, dtype, L.EPI_GELU)
+
+    def _glu_impl(self, x, W_gate, W_up, b_gate, b_up, return_cache, dtype, act):
         code = dtype_code(dtype)
         Wg, Wu = np.asarray(W_gate), np.asarray(W_up)
         if Wg.shape != Wu.shape or Wg.ndim != 2:
@@ -148,9 +207,9 @@ class HipFNN:
         cg = c.alloc(M * N * 4) if return_cache else None
         cu = c.alloc(M * N * 4) if return_cache else None
         try:
-            L.check(c.lib.grl_swiglu_nt(c.ctx, code, code, M, N, K, dx.ptr, dg.ptr, du.ptr,
-                                        dbg.ptr if dbg else None, dbu.ptr if dbu else None, dy.ptr,
-                                        cg.ptr if cg else None, cu.ptr if cu else None), "swiglu_nt")
+            L.check(c.lib.grl_glu_nt(c.ctx, code, code, M, N, K, dx.ptr, dg.ptr, du.ptr,
+                                     dbg.ptr if dbg else None, dbu.ptr if dbu else None, dy.ptr,
+                                     cg.ptr if cg else None, cu.ptr if cu else None, act), "glu_nt")
             out = c.download(dy, (M, N), code)
             if return_cache:
                 return out, c.download(cg, (M, N)), c.download(cu, (M, N))

@@ -38,14 +38,36 @@ struct GemmArgs {
     int M, N, K;
     int tiles_m, tiles_n;
     int group;           // tile-rows per band of the tile walk
+    int act;             // run-time activation code of the EPI_RT / dual epilogues (a GRL_EPI_* value)
+    float alpha, beta;   // RoSwish parameters
 };
 
-enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
+// Epilogue template codes.  NONE / GELU / SILU are compiled in (the encoder's hot shapes); EPI_RT picks
+// ReLU / GCU / RoSwish from GemmArgs::act at run time (one more instantiation instead of three), and the
+// dual-weight epilogue EPI_GLU picks the gate activation (SiLU / ReLU / GELU) the same way.
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_RT = 3, EPI_GLU = 4 };
 
-template <int EPI> __device__ __forceinline__ float epi_apply(float v) {
+// shaders/fused-linear-relu.glsl:63, fused-linear-gcu.glsl:44-46 (x*cos(x)), fused-linear-roswish.glsl:46-58
+// ((x+alpha)*sigmoid(beta*x) - alpha/2; the shader's sign-split sigmoid equals 1/(1+exp(-beta*x)) with the
+// exponential saturating to 0 / +inf)
+__device__ __forceinline__ float act_runtime(float v, const GemmArgs& p) {
+    if (p.act == GRL_EPI_RELU) return fmaxf(v, 0.0f);
+    if (p.act == GRL_EPI_GCU) return v * cosf(v);
+    const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * (p.beta * v)));
+    return (v + p.alpha) * sg - 0.5f * p.alpha;
+}
+template <int EPI> __device__ __forceinline__ float epi_apply(float v, const GemmArgs& p) {
     if (EPI == EPI_GELU) return gelu_fast(v);
     if (EPI == EPI_SILU) return silu_clamped(v);
+    if (EPI == EPI_RT) return act_runtime(v, p);
     return v;
+}
+// gate * act(up): shaders/fused-swiglu.glsl:44-79 (x/(1+exp(-x))), fused-reglu.glsl:74 (max(0,up)),
+// fused-geglu.glsl:44-49,80 (tanh GELU without the clamp rule)
+__device__ __forceinline__ float glu_apply(float gate, float up, const GemmArgs& p) {
+    if (p.act == GRL_EPI_RELU) return gate * fmaxf(up, 0.0f);
+    if (p.act == GRL_EPI_GELU) return gate * gelu_fast(up);
+    return gate * silu_plain(up);
 }
 
 // ---- one 128-byte-per-row K slab on the matrix cores --------------------------------------
@@ -121,10 +143,10 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
                             if (p.cache1) store4<float>(p.cache1 + o, v[0], v[1], v[2], v[3]);
                             if (p.cache2) store4<float>(p.cache2 + o, u[0], u[1], u[2], u[3]);
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(u[e]);
+                            for (int e = 0; e < 4; ++e) v[e] = glu_apply(v[e], u[e], p);
                         } else {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
+                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
                         }
                         store4<OutT>(C + o, v[0], v[1], v[2], v[3]);
                     } else {
@@ -136,9 +158,9 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
                                     float y = u[e] + (p.bias2 ? p.bias2[n + e] : 0.f);
                                     if (p.cache1) p.cache1[o + e] = x;
                                     if (p.cache2) p.cache2[o + e] = y;
-                                    x = x * silu_plain(y);
+                                    x = glu_apply(x, y, p);
                                 } else {
-                                    x = epi_apply<EPI>(x);
+                                    x = epi_apply<EPI>(x, p);
                                 }
                                 elem<OutT>::st(C + o + e, x);
                             }
@@ -498,10 +520,10 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                         for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] + bv1[b][q][e];
                         if (DUAL) {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = v[e] * silu_plain(acc[a][DUAL ? b + TNO : b][4 * q + e] + bv2[b][q][e]);
+                            for (int e = 0; e < 4; ++e) v[e] = glu_apply(v[e], acc[a][DUAL ? b + TNO : b][4 * q + e] + bv2[b][q][e], p);
                         } else {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e]);
+                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
                         }
                         const int byte = nl * OES;
                         const int chunk = (byte >> 4) ^ (r_w & (CPR - 1));
@@ -581,9 +603,9 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmArgs p) {
         if (p.bias2) u += p.bias2[n];
         if (p.cache1) p.cache1[idx] = s;
         if (p.cache2) p.cache2[idx] = u;
-        s = s * silu_plain(u);
+        s = glu_apply(s, u, p);
     } else {
-        s = epi_apply<EPI>(s);
+        s = epi_apply<EPI>(s, p);
     }
     elem<OutT>::st((OutT*)p.C + idx, s);
 }
@@ -646,7 +668,8 @@ static int dispatch_epi(grl_ctx* c, GemmArgs& a, int epi) {
         case EPI_NONE: return launch_gemm<T, OutT, EPI_NONE, false>(c, a);
         case EPI_GELU: return launch_gemm<T, OutT, EPI_GELU, false>(c, a);
         case EPI_SILU: return launch_gemm<T, OutT, EPI_SILU, false>(c, a);
-        case EPI_SWIGLU: return launch_gemm<T, OutT, EPI_SWIGLU, true>(c, a);
+        case EPI_RT: return launch_gemm<T, OutT, EPI_RT, false>(c, a);
+        case EPI_GLU: return launch_gemm<T, OutT, EPI_GLU, true>(c, a);
     }
     grl_set_error("gemm: bad epilogue %d", epi);
     return GRL_ERR_ARG;
@@ -669,53 +692,70 @@ static int check_dims(const char* who, int64_t M, int64_t N, int64_t K) {
 
 // K == 0: the sum is empty, C = epi(bias)
 template <typename OutT>
-__global__ __launch_bounds__(256) void bias_fill_kernel(OutT* C, const float* bias, int64_t total, int N, int epi) {
+__global__ __launch_bounds__(256) void bias_fill_kernel(OutT* C, const float* bias, int64_t total, int N, int epi, GemmArgs p) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     float v = bias ? bias[i % N] : 0.f;
-    v = epi == EPI_GELU ? epi_apply<EPI_GELU>(v) : epi == EPI_SILU ? epi_apply<EPI_SILU>(v) : v;
+    v = epi == EPI_GELU ? epi_apply<EPI_GELU>(v, p) : epi == EPI_SILU ? epi_apply<EPI_SILU>(v, p) : epi == EPI_RT ? epi_apply<EPI_RT>(v, p) : v;
     elem<OutT>::st(C + i, v);
 }
 
-extern "C" int grl_gemm_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
-                           const void* A, const void* W, const float* bias, void* C, int epilogue) {
+extern "C" int grl_gemm_nt_act(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                               const void* A, const void* W, const float* bias, void* C, int epilogue,
+                               float alpha, float beta) {
     GRL_REQUIRE(c, GRL_ERR_ARG, "grl_gemm_nt: null context");
     GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_gemm_nt: bad dtype");
-    GRL_REQUIRE(epilogue >= GRL_EPI_NONE && epilogue <= GRL_EPI_SILU, GRL_ERR_ARG, "grl_gemm_nt: bad epilogue %d", epilogue);
+    GRL_REQUIRE(epilogue >= GRL_EPI_NONE && epilogue <= GRL_EPI_ROSWISH, GRL_ERR_ARG, "grl_gemm_nt: bad epilogue %d", epilogue);
     int rc = check_dims("grl_gemm_nt", M, N, K);
     if (rc) return rc;
     if (M == 0 || N == 0) return GRL_OK;
     GRL_REQUIRE(C && (K == 0 || (A && W)), GRL_ERR_ARG, "grl_gemm_nt: null argument");
-    if (K == 0) {
-        int64_t total = M * N;
-        GRL_REQUIRE((total + 255) / 256 < (1LL << 31), GRL_ERR_SHAPE, "grl_gemm_nt: output too large");
-        if (out_dtype == GRL_F32) hipLaunchKernelGGL(bias_fill_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, (float*)C, bias, total, (int)N, epilogue);
-        else hipLaunchKernelGGL(bias_fill_kernel<uint16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, (uint16_t*)C, bias, total, (int)N, epilogue);
-        GRL_CHECK_LAUNCH();
-        return GRL_OK;
-    }
     GemmArgs a{};
     a.A = A; a.W = W; a.bias = bias; a.C = C;
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
-    return dispatch_types(c, a, in_dtype, out_dtype, epilogue);
+    a.act = epilogue; a.alpha = alpha; a.beta = beta;
+    const int epi = epilogue <= GRL_EPI_SILU ? epilogue : EPI_RT;
+    if (K == 0) {
+        int64_t total = M * N;
+        GRL_REQUIRE((total + 255) / 256 < (1LL << 31), GRL_ERR_SHAPE, "grl_gemm_nt: output too large");
+        if (out_dtype == GRL_F32) hipLaunchKernelGGL(bias_fill_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, (float*)C, bias, total, (int)N, epi, a);
+        else hipLaunchKernelGGL(bias_fill_kernel<uint16_t>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, (uint16_t*)C, bias, total, (int)N, epi, a);
+        GRL_CHECK_LAUNCH();
+        return GRL_OK;
+    }
+    return dispatch_types(c, a, in_dtype, out_dtype, epi);
 }
 
-extern "C" int grl_swiglu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
-                             const void* x, const void* W_gate, const void* W_up, const float* b_gate,
-                             const float* b_up, void* out, float* gate_cache, float* up_cache) {
-    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_swiglu_nt: null context");
-    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_swiglu_nt: bad dtype");
-    int rc = check_dims("grl_swiglu_nt", M, N, K);
+extern "C" int grl_gemm_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                           const void* A, const void* W, const float* bias, void* C, int epilogue) {
+    return grl_gemm_nt_act(c, in_dtype, out_dtype, M, N, K, A, W, bias, C, epilogue, 1.0f, 1.0f);
+}
+
+extern "C" int grl_glu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                          const void* x, const void* W_gate, const void* W_up, const float* b_gate,
+                          const float* b_up, void* out, float* gate_cache, float* up_cache, int activation) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_glu_nt: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_glu_nt: bad dtype");
+    GRL_REQUIRE(activation == GRL_EPI_SILU || activation == GRL_EPI_RELU || activation == GRL_EPI_GELU, GRL_ERR_ARG,
+                "grl_glu_nt: activation must be GRL_EPI_SILU, GRL_EPI_RELU or GRL_EPI_GELU (got %d)", activation);
+    int rc = check_dims("grl_glu_nt", M, N, K);
     if (rc) return rc;
     if (M == 0 || N == 0) return GRL_OK;
-    GRL_REQUIRE(out && K > 0 && x && W_gate && W_up, GRL_ERR_ARG, "grl_swiglu_nt: null argument or K == 0");
+    GRL_REQUIRE(out && K > 0 && x && W_gate && W_up, GRL_ERR_ARG, "grl_glu_nt: null argument or K == 0");
     GemmArgs a{};
     a.A = x; a.W = W_gate; a.W2 = W_up; a.C = out;
     // the reference applies biases only when both are present (backend/_glu_append.py:68)
     if (b_gate && b_up) { a.bias = b_gate; a.bias2 = b_up; }
     a.cache1 = gate_cache; a.cache2 = up_cache;
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
-    return dispatch_types(c, a, in_dtype, out_dtype, EPI_SWIGLU);
+    a.act = activation;
+    return dispatch_types(c, a, in_dtype, out_dtype, EPI_GLU);
+}
+
+extern "C" int grl_swiglu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                             const void* x, const void* W_gate, const void* W_up, const float* b_gate,
+                             const float* b_up, void* out, float* gate_cache, float* up_cache) {
+    return grl_glu_nt(c, in_dtype, out_dtype, M, N, K, x, W_gate, W_up, b_gate, b_up, out, gate_cache, up_cache, GRL_EPI_SILU);
 }
 
 extern "C" int grl_gemm_nn(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,

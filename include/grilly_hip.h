@@ -45,7 +45,10 @@ typedef enum grl_dtype { GRL_F32 = 0, GRL_BF16 = 1 } grl_dtype;
 typedef enum grl_epilogue {
     GRL_EPI_NONE = 0,
     GRL_EPI_GELU = 1,   /* tanh GELU with the +-50 clamp rule of shaders/fused-linear-gelu.glsl:45-63 */
-    GRL_EPI_SILU = 2    /* s/(1+exp(-clamp(s,-88,88))), shaders/fused-linear-silu.glsl:43-48 */
+    GRL_EPI_SILU = 2,   /* s/(1+exp(-clamp(s,-88,88))), shaders/fused-linear-silu.glsl:43-48 */
+    GRL_EPI_RELU = 3,   /* max(0,s), shaders/fused-linear-relu.glsl:63 */
+    GRL_EPI_GCU = 4,    /* s*cos(s), shaders/fused-linear-gcu.glsl:44-46 */
+    GRL_EPI_ROSWISH = 5 /* (s+alpha)*sigmoid(beta*s) - alpha/2, shaders/fused-linear-roswish.glsl:46-58 */
 } grl_epilogue;
 
 typedef enum grl_rope_style { GRL_ROPE_NONE = 0, GRL_ROPE_INTERLEAVED = 1, GRL_ROPE_HALF = 2 } grl_rope_style;
@@ -119,6 +122,24 @@ int grl_gemm_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N,
  * kernel transposes B once); pass NULL to let the context allocate it from its pool. */
 int grl_gemm_nn(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
                 const void* A, const void* B, void* C, void* workspace);
+
+/* grl_gemm_nt with every epilogue of the reference's fused-linear family: additionally
+ * GRL_EPI_RELU (VulkanFNN.fused_linear_relu, backend/fnn.py:2125-2212, shaders/fused-linear-relu.glsl:40-68),
+ * GRL_EPI_GCU (fused_linear_gcu, backend/fnn.py:2307-2383, shaders/fused-linear-gcu.glsl:43-75) and
+ * GRL_EPI_ROSWISH (fused_linear_roswish, backend/fnn.py:2385-2470, shaders/fused-linear-roswish.glsl:44-90)
+ * with its two parameters; alpha and beta are ignored by the other epilogues. */
+int grl_gemm_nt_act(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                    const void* A, const void* W, const float* bias, void* C, int epilogue,
+                    float alpha, float beta);
+
+/* out[m,n] = (x.Wg^T + bg)[m,n] * act((x.Wu^T + bu)[m,n]) with act = GRL_EPI_SILU (SwiGLU, below),
+ * GRL_EPI_RELU (fused_reglu, backend/_glu_append.py:131-222, shaders/fused-reglu.glsl:42-75) or
+ * GRL_EPI_GELU (fused_geglu, backend/_glu_append.py:224-315, shaders/fused-geglu.glsl:43-82: tanh GELU
+ * without the clamp rule).  Biases and caches as for grl_swiglu_nt. */
+int grl_glu_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+               const void* x, const void* W_gate, const void* W_up,
+               const float* b_gate, const float* b_up, void* out,
+               float* gate_cache, float* up_cache, int activation);
 
 /* out[m,n] = (x.Wg^T + bg)[m,n] * silu((x.Wu^T + bu)[m,n]),  silu(u) = u/(1+exp(-u)).
  * Replaces fused_swiglu (backend/_glu_append.py:8-129, shaders/fused-swiglu.glsl:43-79).

@@ -32,6 +32,9 @@
 #define EPI_NONE 0
 #define EPI_GELU 1
 #define EPI_SILU 2
+#define EPI_RELU 3
+#define EPI_GCU 4
+#define EPI_ROSWISH 5
 
 /* shaders/fused-linear-gelu.glsl:45-63 (same body as shaders/activation-gelu.glsl:33-50) */
 static inline float gelu_shader(float x) {
@@ -62,7 +65,20 @@ static inline float sigmoid_split(float v) {
 /* y[m,n] = epi(sum_k x[m,k]*W[n,k] + b[n]):  shaders/fnn-linear.glsl:33-58,
  * shaders/fused-linear-gelu.glsl:65-93, shaders/fused-linear-silu.glsl:50-78;
  * with N = 3*H*D and packed weights also shaders/fused-qkv-projection.glsl:48-74. */
-void orc_linear(const float* x, const float* W, const float* b, float* y, int64_t M, int64_t K, int64_t N, int epi) {
+/* shaders/fused-linear-roswish.glsl:46-58 */
+static inline float roswish_shader(float x, float alpha, float beta) {
+    return (x + alpha) * sigmoid_split(beta * x) - 0.5f * alpha;
+}
+
+/* shaders/fused-geglu.glsl:44-49: tanh GELU without the +-50 clamp rule */
+static inline float gelu_plain(float x) {
+    return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+
+/* epi 0..2 as above; 3 = shaders/fused-linear-relu.glsl:40-68 (max(0,s)); 4 = shaders/fused-linear-gcu.glsl:43-75
+ * (s*cos(s)); 5 = shaders/fused-linear-roswish.glsl:60-90 */
+void orc_linear_act(const float* x, const float* W, const float* b, float* y, int64_t M, int64_t K, int64_t N, int epi,
+                    float alpha, float beta) {
 #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; ++m) {
         for (int64_t n = 0; n < N; ++n) {
@@ -71,9 +87,16 @@ void orc_linear(const float* x, const float* W, const float* b, float* y, int64_
             if (b) sum += b[n];
             if (epi == EPI_GELU) sum = gelu_shader(sum);
             else if (epi == EPI_SILU) sum = silu_clamped(sum);
+            else if (epi == EPI_RELU) sum = sum > 0.0f ? sum : 0.0f;
+            else if (epi == EPI_GCU) sum = sum * cosf(sum);
+            else if (epi == EPI_ROSWISH) sum = roswish_shader(sum, alpha, beta);
             y[m * N + n] = sum;
         }
     }
+}
+
+void orc_linear(const float* x, const float* W, const float* b, float* y, int64_t M, int64_t K, int64_t N, int epi) {
+    orc_linear_act(x, W, b, y, M, K, N, epi, 1.0f, 1.0f);
 }
 
 /* C = A.B, B (K,N): shaders/gemm_mnk.glsl:35-88 (ascending k over 16-wide tiles = ascending k) */
@@ -90,8 +113,18 @@ void orc_gemm_nn(const float* A, const float* B, float* C, int64_t M, int64_t K,
 /* shaders/fused-swiglu.glsl:48-79: gate*silu(up); biases only when both given
  * (backend/_glu_append.py:68).  gate_c/up_c (optional) receive the pre-activations
  * (backend/_glu_append.py:120-127). */
+void orc_fused_glu(const float* x, const float* Wg, const float* Wu, const float* bg, const float* bu,
+                   float* out, float* gate_c, float* up_c, int64_t M, int64_t K, int64_t N, int act);
+
 void orc_fused_swiglu(const float* x, const float* Wg, const float* Wu, const float* bg, const float* bu,
                       float* out, float* gate_c, float* up_c, int64_t M, int64_t K, int64_t N) {
+    orc_fused_glu(x, Wg, Wu, bg, bu, out, gate_c, up_c, M, K, N, EPI_SILU);
+}
+
+/* act 2: the SwiGLU above; act 3: shaders/fused-reglu.glsl:42-75 (gate*max(0,up), backend/_glu_append.py:131-222);
+ * act 1: shaders/fused-geglu.glsl:43-82 (gate*gelu(up), backend/_glu_append.py:224-315) */
+void orc_fused_glu(const float* x, const float* Wg, const float* Wu, const float* bg, const float* bu,
+                   float* out, float* gate_c, float* up_c, int64_t M, int64_t K, int64_t N, int act) {
     int has_bias = bg && bu;
 #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; ++m)
@@ -103,7 +136,7 @@ void orc_fused_swiglu(const float* x, const float* Wg, const float* Wu, const fl
             if (has_bias) up += bu[n];
             if (gate_c) gate_c[m * N + n] = gate;
             if (up_c) up_c[m * N + n] = up;
-            out[m * N + n] = gate * silu_plain(up);
+            out[m * N + n] = act == EPI_RELU ? gate * (up > 0.0f ? up : 0.0f) : act == EPI_GELU ? gate * gelu_plain(up) : gate * silu_plain(up);
         }
 }
 

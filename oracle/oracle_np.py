@@ -64,7 +64,7 @@ def truth_silu(x):
         return x / (1.0 + np.exp(-x))
 
 
-def truth_linear(x, W, b=None, epi="none"):
+def truth_linear(x, W, b=None, epi="none", alpha=1.0, beta=1.0):
     """x.W^T + b: shaders/fnn-linear.glsl:42-57; W is (out,in) (backend/fnn.py:1394-1419)."""
     y = np.asarray(x, np.float64) @ np.asarray(W, np.float64).T
     if b is not None:
@@ -73,7 +73,40 @@ def truth_linear(x, W, b=None, epi="none"):
         y = truth_gelu(y)
     elif epi == "silu":
         y = truth_silu_clamped(y)
+    elif epi == "relu":          # shaders/fused-linear-relu.glsl:63
+        y = np.maximum(y, 0.0)
+    elif epi == "gcu":           # shaders/fused-linear-gcu.glsl:44-46
+        y = y * np.cos(y)
+    elif epi == "roswish":       # shaders/fused-linear-roswish.glsl:46-58
+        y = truth_roswish(y, alpha, beta)
+    elif epi != "none":
+        raise ValueError(epi)
     return y
+
+
+def truth_roswish(x, alpha=1.0, beta=1.0):
+    """(x+alpha)*sigmoid(beta*x) - alpha/2: shaders/fused-linear-roswish.glsl:46-58"""
+    x = np.asarray(x, np.float64)
+    with np.errstate(over="ignore"):
+        return (x + alpha) / (1.0 + np.exp(-beta * x)) - 0.5 * alpha
+
+
+def truth_gelu_plain(x):
+    """tanh GELU without the clamp rule: shaders/fused-geglu.glsl:44-49"""
+    x = np.asarray(x, np.float64)
+    return 0.5 * x * (1.0 + np.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
+
+
+def truth_fused_glu(x, Wg, Wu, bg=None, bu=None, act="silu"):
+    """gate*act(up) for act silu / relu / gelu: shaders/fused-swiglu.glsl:54-78, fused-reglu.glsl:42-75,
+    fused-geglu.glsl:43-82; biases only if both given (backend/_glu_append.py:68).  Returns (out, gate, up)."""
+    g = np.asarray(x, np.float64) @ np.asarray(Wg, np.float64).T
+    u = np.asarray(x, np.float64) @ np.asarray(Wu, np.float64).T
+    if bg is not None and bu is not None:
+        g = g + np.asarray(bg, np.float64)
+        u = u + np.asarray(bu, np.float64)
+    a = {"silu": truth_silu, "relu": lambda t: np.maximum(t, 0.0), "gelu": truth_gelu_plain}[act](u)
+    return g * a, g, u
 
 
 def truth_gemm(A, B):
@@ -251,6 +284,8 @@ class COracle:
         self.lib = ctypes.CDLL(_LIB_PATH)
         L, i64, f, ci = self.lib, ctypes.c_int64, ctypes.c_float, ctypes.c_int
         L.orc_linear.argtypes = [_F, _F, _F, _F, i64, i64, i64, ci]
+        L.orc_linear_act.argtypes = [_F, _F, _F, _F, i64, i64, i64, ci, f, f]
+        L.orc_fused_glu.argtypes = [_F, _F, _F, _F, _F, _F, _F, _F, i64, i64, i64, ci]
         L.orc_gemm_nn.argtypes = [_F, _F, _F, i64, i64, i64]
         L.orc_fused_swiglu.argtypes = [_F, _F, _F, _F, _F, _F, _F, _F, i64, i64, i64]
         L.orc_layernorm.argtypes = [_F, _F, _F, _F, _F, i64, i64, f]
@@ -264,19 +299,28 @@ class COracle:
         L.orc_mean_pool.argtypes = [_F, _F, _F, i64, i64, i64, ci]
         L.orc_bert_layer.argtypes = [_F, _F, i64, i64, i64, i64, i64] + [_F] * 12 + [f, _F]
         L.orc_num_threads.restype = ci
-        for n in ("orc_linear", "orc_gemm_nn", "orc_fused_swiglu", "orc_layernorm", "orc_residual", "orc_gelu",
+        for n in ("orc_linear", "orc_linear_act", "orc_fused_glu", "orc_gemm_nn", "orc_fused_swiglu", "orc_layernorm", "orc_residual", "orc_gelu",
                   "orc_silu", "orc_swiglu_act", "orc_rope", "orc_attention", "orc_embed", "orc_mean_pool", "orc_bert_layer"):
             getattr(L, n).restype = None
 
     def num_threads(self):
         return int(self.lib.orc_num_threads())
 
-    def linear(self, x, W, b=None, epi="none"):
+    def linear(self, x, W, b=None, epi="none", alpha=1.0, beta=1.0):
         x, W, b = _f32(x), _f32(W), _f32(b)
         M, K = x.shape; N = W.shape[0]
         y = np.empty((M, N), np.float32)
-        self.lib.orc_linear(_fp(x), _fp(W), _fp(b), _fp(y), M, K, N, {"none": 0, "gelu": 1, "silu": 2}[epi])
+        code = {"none": 0, "gelu": 1, "silu": 2, "relu": 3, "gcu": 4, "roswish": 5}[epi]
+        self.lib.orc_linear_act(_fp(x), _fp(W), _fp(b), _fp(y), M, K, N, code, alpha, beta)
         return y
+
+    def fused_glu(self, x, Wg, Wu, bg=None, bu=None, act="silu"):
+        x, Wg, Wu, bg, bu = _f32(x), _f32(Wg), _f32(Wu), _f32(bg), _f32(bu)
+        M, K = x.shape; N = Wg.shape[0]
+        out, g, u = (np.empty((M, N), np.float32) for _ in range(3))
+        self.lib.orc_fused_glu(_fp(x), _fp(Wg), _fp(Wu), _fp(bg), _fp(bu), _fp(out), _fp(g), _fp(u), M, K, N,
+                               {"silu": 2, "relu": 3, "gelu": 1}[act])
+        return out, g, u
 
     def gemm(self, A, B):
         A, B = _f32(A), _f32(B)

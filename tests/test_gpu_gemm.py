@@ -6,6 +6,7 @@ import pytest
 
 from conftest import TOL_F32, TOL_BF16, rng_for
 from oracle import oracle_np as O
+from grilly_amd import _lib as L
 
 pytestmark = pytest.mark.gpu
 
@@ -105,6 +106,73 @@ def test_fused_swiglu_parity(backend, dtype, M, K, N, bias):
     # a single bias is ignored, as in the reference
     np.testing.assert_array_equal(backend.fnn.fused_swiglu(x, Wg, Wu, bg, None, dtype=dtype),
                                   backend.fnn.fused_swiglu(x, Wg, Wu, dtype=dtype))
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("epi", ["relu", "gcu", "roswish"])
+@pytest.mark.parametrize("M,K,N", [(5, 24, 7), (129, 136, 260), (1024, 768, 1536)])
+def test_further_fused_linear_parity(backend, dtype, epi, M, K, N):
+    rng = np.random.default_rng(17 + M + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    W = (rng.standard_normal((N, K)) * 0.1).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    x, W = prep(dtype, x, W)
+    if epi == "relu":
+        y = backend.fnn.fused_linear_relu(x, W, b, dtype=dtype)
+    elif epi == "gcu":
+        y = backend.fnn.fused_linear_gcu(x, W, b, dtype=dtype)
+    else:
+        y = backend.fnn.fused_linear_roswish(x, W, b, alpha=0.7, beta=1.3, dtype=dtype)
+    assert y.shape == (M, N)
+    assert O.max_rel(y, O.truth_linear(x, W, b, epi, 0.7, 1.3)) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("act", ["relu", "gelu"])
+@pytest.mark.parametrize("M,K,N,bias", [(6, 20, 10, True), (513, 264, 130, False), (1024, 512, 1408, True)])
+def test_reglu_geglu_parity(backend, dtype, act, M, K, N, bias):
+    rng = np.random.default_rng(M + N + 3)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    Wg = (rng.standard_normal((N, K)) * 0.1).astype(np.float32)
+    Wu = (rng.standard_normal((N, K)) * 0.1).astype(np.float32)
+    bg = rng.standard_normal(N).astype(np.float32) if bias else None
+    bu = rng.standard_normal(N).astype(np.float32) if bias else None
+    x, Wg, Wu = prep(dtype, x, Wg, Wu)
+    t_out, t_g, t_u = O.truth_fused_glu(x, Wg, Wu, bg, bu, act)
+    fn = backend.fnn.fused_reglu if act == "relu" else backend.fnn.fused_geglu
+    out, g, u = fn(x, Wg, Wu, bg, bu, return_cache=True, dtype=dtype)
+    assert out.shape == (M, N)
+    assert O.max_rel(out, t_out) < tol(dtype)
+    assert O.max_rel(g, t_g) < 1e-4 and O.max_rel(u, t_u) < 1e-4
+    assert O.max_rel(fn(x, Wg, Wu, bg, bu, dtype=dtype), t_out) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_fused_layernorm_linear(backend, dtype):
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal((3, 50, 768)).astype(np.float32)
+    W = (rng.standard_normal((300, 768)) * 0.05).astype(np.float32)
+    b = rng.standard_normal(300).astype(np.float32)
+    g, bt = rng.standard_normal(768).astype(np.float32), rng.standard_normal(768).astype(np.float32)
+    x, W = prep(dtype, x, W)
+    y = backend.fnn.fused_layernorm_linear(x, g, bt, W, b, eps=1e-5, dtype=dtype)
+    assert y.shape == (3, 50, 300)
+    ref = O.truth_linear(O.truth_layernorm(x, g, bt, 1e-5), W, b)
+    assert O.max_rel(y, ref) < tol(dtype)
+
+
+def test_further_epilogue_edges(backend):
+    s = np.array([0.0, np.pi, -np.pi, 2.0, -3.0, 60.0, -60.0, 200.0, -200.0], np.float32)
+    x = np.zeros((len(s), 8), np.float32); x[:, 0] = s
+    W = np.zeros((4, 8), np.float32); W[:, 0] = 1
+    np.testing.assert_array_equal(backend.fnn.fused_linear_relu(x, W)[:, 0], np.maximum(s, 0))
+    np.testing.assert_allclose(backend.fnn.fused_linear_gcu(x, W)[:, 0], O.truth_linear(x, W, None, "gcu")[:, 0], rtol=1e-5, atol=1e-5)
+    ro = backend.fnn.fused_linear_roswish(x, W, alpha=0.8, beta=1.5)[:, 0]
+    np.testing.assert_allclose(ro, O.truth_roswish(s, 0.8, 1.5), rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        L.check(backend.core.lib.grl_gemm_nt(backend.core.ctx, 0, 0, 1, 1, 1, None, None, None, None, 6))
+    with pytest.raises(ValueError):
+        L.check(backend.core.lib.grl_glu_nt(backend.core.ctx, 0, 0, 1, 1, 1, None, None, None, None, None, None, None, None, 4))
 
 
 def test_fused_swiglu_always_2d_and_config4_convention(backend):

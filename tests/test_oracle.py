@@ -128,6 +128,46 @@ def test_fused_swiglu_conventions(corc):
     np.testing.assert_array_equal(o1, o0)
 
 
+def test_further_epilogues_known_answers_and_composition(corc):
+    """ReLU / GCU / RoSwish fused linears and ReGLU / GeGLU (shaders/fused-linear-relu.glsl:63,
+    fused-linear-gcu.glsl:44-46, fused-linear-roswish.glsl:46-58, fused-reglu.glsl:74, fused-geglu.glsl:44-49,80).
+    The reference holds no numeric test for them; pinned by values the formulas fix and by composition."""
+    # drive chosen pre-activations through a 1-wide linear
+    s = np.array([0.0, np.pi, -np.pi, np.pi / 2, 2.0, -3.0, 40.0, -40.0], np.float32)
+    x = np.zeros((len(s), 3), np.float32); x[:, 0] = s
+    W = np.zeros((2, 3), np.float32); W[:, 0] = 1
+    relu = corc.linear(x, W, None, "relu")[:, 0]
+    np.testing.assert_array_equal(relu, np.maximum(s, 0))
+    gcu = corc.linear(x, W, None, "gcu")[:, 0]
+    # x*cos(x): 0 at 0, -pi at pi, +pi at -pi, ~0 at pi/2
+    np.testing.assert_allclose(gcu[:4], [0.0, -np.pi, np.pi, 0.0], atol=1e-6)
+    # RoSwish: alpha = 0, beta = 1 is x*sigmoid(x) = SiLU; value at 0 is 0 for every alpha; large beta*x -> x + alpha/2, 0 - alpha/2
+    ro0 = corc.linear(x, W, None, "roswish", 0.0, 1.0)[:, 0]
+    np.testing.assert_allclose(ro0, O.truth_silu(s), rtol=1e-6, atol=1e-7)
+    ro = corc.linear(x, W, None, "roswish", 0.8, 1.5)[:, 0]
+    assert abs(ro[0]) < 1e-7
+    np.testing.assert_allclose(ro[6:], [40.0 + 0.4, -0.4], rtol=1e-6)
+    rng = np.random.default_rng(5)
+    xx = rng.standard_normal((9, 12)).astype(np.float32)
+    Wg, Wu = (rng.standard_normal((6, 12)).astype(np.float32) for _ in range(2))
+    bg, bu = (rng.standard_normal(6).astype(np.float32) for _ in range(2))
+    for epi, a, b in (("relu", 1, 1), ("gcu", 1, 1), ("roswish", 0.3, 2.0)):
+        assert rel(corc.linear(xx, Wg, bg, epi, a, b), O.truth_linear(xx, Wg, bg, epi, a, b)) < 1e-6
+    # GLU family = gate * act(up) with the separately pinned pieces; biases only when both are given
+    for act, f in (("relu", lambda t: np.maximum(t, 0)), ("gelu", O.truth_gelu), ("silu", O.truth_silu)):
+        out, g, u = corc.fused_glu(xx, Wg, Wu, bg, bu, act)
+        np.testing.assert_allclose(g, corc.linear(xx, Wg, bg), rtol=1e-6, atol=1e-6)
+        np.testing.assert_allclose(u, corc.linear(xx, Wu, bu), rtol=1e-6, atol=1e-6)
+        assert rel(out, g.astype(np.float64) * f(u.astype(np.float64))) < 1e-6     # |up| < 50 here: clamp rule idle
+        one, _, _ = corc.fused_glu(xx, Wg, Wu, bg, None, act)
+        none, _, _ = corc.fused_glu(xx, Wg, Wu, None, None, act)
+        np.testing.assert_array_equal(one, none)
+    # fused LayerNorm + linear (shaders/fused-layernorm-linear.glsl:67-128) is the composition of the two pinned pieces
+    gam, bet = rng.standard_normal(12).astype(np.float32), rng.standard_normal(12).astype(np.float32)
+    ln = corc.layernorm(xx, gam, bet, 1e-5)
+    assert rel(corc.linear(ln, Wg, bg), O.truth_linear(O.truth_layernorm(xx, gam, bet, 1e-5), Wg, bg)) < 1e-5
+
+
 def test_qkv_is_concat_of_three_linears(corc):
     rng = np.random.default_rng(5)
     x = rng.standard_normal((4, 12)).astype(np.float32)
