@@ -6,7 +6,8 @@
     o = backend.attention.flash_attention2(q, k, v, num_heads, head_dim)
 
 Same numpy-in / numpy-out methods as the reference's `grilly.Compute()` for this path; the
-work is done by hand-written HIP kernels in grilly_amd/lib/libgrilly_hip.so.
+work is done by hand-written HIP kernels in grilly_amd/lib/libgrilly_hip.so.  `grilly_amd.nn`
+holds forward-only Module adapters (Linear, LayerNorm, FlashAttention2, TransformerEncoderLayer ...).
 """
 from .backend.compute import HipCompute, Compute
 from .encoder import BertEncoder, EncoderConfig, random_bert_weights

@@ -67,6 +67,7 @@ SIGNATURES = {
     "grl_add": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p, c_void_p]),
     "grl_gelu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),
     "grl_silu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),
+    "grl_relu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),
     "grl_swiglu_act": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_void_p]),
     "grl_embed": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "grl_mean_pool": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_int]),

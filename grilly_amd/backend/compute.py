@@ -35,10 +35,14 @@ class HipCompute:
     def residual(self, *a, **k): return self.fnn.residual(*a, **k)
     def activation_gelu(self, *a, **k): return self.fnn.activation_gelu(*a, **k)
     def activation_silu(self, *a, **k): return self.fnn.activation_silu(*a, **k)
+    def activation_relu(self, *a, **k): return self.fnn.activation_relu(*a, **k)
     def activation_swiglu(self, *a, **k): return self.fnn.activation_swiglu(*a, **k)
     def fused_linear_gelu(self, *a, **k): return self.fnn.fused_linear_gelu(*a, **k)
     def fused_linear_silu(self, *a, **k): return self.fnn.fused_linear_silu(*a, **k)
     def fused_swiglu(self, *a, **k): return self.fnn.fused_swiglu(*a, **k)
+    def fused_linear_relu(self, *a, **k): return self.fnn.fused_linear_relu(*a, **k)
+    def fused_reglu(self, *a, **k): return self.fnn.fused_reglu(*a, **k)
+    def fused_geglu(self, *a, **k): return self.fnn.fused_geglu(*a, **k)
     def apply_rope(self, *a, **k): return self.attention.apply_rope(*a, **k)
 
     def __enter__(self):

@@ -277,6 +277,10 @@ class HipFNN:
         """Reference backend/fnn.py:344-391."""
         return self._unary(self.core.lib.grl_silu, x, dtype, "silu")
 
+    def activation_relu(self, x, dtype="fp32"):
+        """Reference backend/fnn.py:232-283."""
+        return self._unary(self.core.lib.grl_relu, x, dtype, "relu")
+
     def activation_swiglu(self, x, dtype="fp32"):
         """Last dim 2h -> h: x1 * silu(x2) (reference backend/fnn.py:499-572); any rank >= 1."""
         code = dtype_code(dtype)

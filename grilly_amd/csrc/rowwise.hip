@@ -170,7 +170,7 @@ extern "C" int grl_layernorm(grl_ctx* c, int dtype, int64_t rows, int64_t F, con
 }
 
 // ------------------------------------------------------------------ elementwise
-enum { OP_ADD = 0, OP_GELU = 1, OP_SILU = 2 };
+enum { OP_ADD = 0, OP_GELU = 1, OP_SILU = 2, OP_RELU = 3 };
 
 // shaders/activation-swiglu.glsl:40-49: sign-split stable sigmoid
 __device__ __forceinline__ float sigmoid_stable(float v) {
@@ -182,6 +182,7 @@ __device__ __forceinline__ float sigmoid_stable(float v) {
 template <int OP> __device__ __forceinline__ float ew_apply(float a, float b) {
     if (OP == OP_ADD) return a + b;
     if (OP == OP_GELU) return gelu_ref(a);
+    if (OP == OP_RELU) return fmaxf(a, 0.0f);   // shaders/activation-relu.glsl (backend/fnn.py:232-283)
     return a * sigmoid_stable(a);   // backend/fnn.py:344-391 (activation_silu): x*sigmoid(x)
 }
 
@@ -235,6 +236,7 @@ static int launch_ew(grl_ctx* c, int64_t n, const void* a, const void* b, void* 
 extern "C" int grl_add(grl_ctx* c, int dtype, int64_t n, const void* a, const void* b, void* out) { EW_ENTRY("grl_add", OP_ADD, true) }
 extern "C" int grl_gelu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_gelu", OP_GELU, false) }
 extern "C" int grl_silu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_silu", OP_SILU, false) }
+extern "C" int grl_relu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_relu", OP_RELU, false) }
 
 // x (rows, 2h) -> y (rows, h)
 template <typename T>

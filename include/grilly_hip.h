@@ -197,6 +197,8 @@ int grl_add(grl_ctx* ctx, int dtype, int64_t n, const void* a, const void* b, vo
 int grl_gelu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
 /* Replaces VulkanFNN.activation_silu (backend/fnn.py:344-391): x*sigmoid(x). */
 int grl_silu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
+/* Replaces VulkanFNN.activation_relu (backend/fnn.py:232-283): max(0,x). */
+int grl_relu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
 /* x (rows, 2h) -> y (rows, h): x1*(x2*sigmoid(x2)), x1 first half.
  * Replaces VulkanFNN.activation_swiglu (backend/fnn.py:499-572, shaders/activation-swiglu.glsl:21-52). */
 int grl_swiglu_act(grl_ctx* ctx, int dtype, int64_t rows, int64_t h, const void* x, void* y);
