@@ -1,0 +1,137 @@
+"""Local checkpoint import (grilly_amd/checkpoint.py) on synthetic BERT- and DistilBERT-named files."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from grilly_amd.checkpoint import load_encoder_checkpoint
+from grilly_amd.encoder import EncoderConfig, random_bert_weights
+
+CFG = EncoderConfig(layers=2, d_model=64, heads=2, d_ff=128, vocab=100, max_pos=32)
+
+
+def bert_state(w, prefix="bert."):
+    sd = {prefix + "embeddings.word_embeddings.weight": w["tok_emb"], prefix + "embeddings.position_embeddings.weight": w["pos_emb"],
+          prefix + "embeddings.token_type_embeddings.weight": w["type_emb"],
+          prefix + "embeddings.LayerNorm.weight": w["emb_ln_g"], prefix + "embeddings.LayerNorm.bias": w["emb_ln_b"]}
+    d = CFG.d_model
+    for i, lw in enumerate(w["layers"]):
+        p = f"{prefix}encoder.layer.{i}."
+        for j, t in enumerate(("query", "key", "value")):
+            sd[p + f"attention.self.{t}.weight"] = lw["w_qkv"][j * d:(j + 1) * d]
+            sd[p + f"attention.self.{t}.bias"] = lw["b_qkv"][j * d:(j + 1) * d]
+        for name, (wk, bk) in {"attention.output.dense": ("w_o", "b_o"), "attention.output.LayerNorm": ("ln1_g", "ln1_b"),
+                               "intermediate.dense": ("w_ff1", "b_ff1"), "output.dense": ("w_ff2", "b_ff2"),
+                               "output.LayerNorm": ("ln2_g", "ln2_b")}.items():
+            sd[p + name + ".weight"], sd[p + name + ".bias"] = lw[wk], lw[bk]
+    return {k: np.ascontiguousarray(v) for k, v in sd.items()}
+
+
+def noisy_weights(seed):
+    w = random_bert_weights(CFG, seed=seed)
+    rng = np.random.default_rng(seed + 1)
+    for lw in w["layers"]:
+        for k in lw:
+            if lw[k].ndim == 1:
+                lw[k] = (lw[k] + 0.1 * rng.standard_normal(lw[k].shape)).astype(np.float32)
+    return w
+
+
+def same(a, b):
+    for k in ("tok_emb", "pos_emb", "type_emb", "emb_ln_g", "emb_ln_b"):
+        np.testing.assert_array_equal(a[k], b[k])
+    assert len(a["layers"]) == len(b["layers"])
+    for la, lb in zip(a["layers"], b["layers"]):
+        assert set(la) == set(lb)
+        for k in la:
+            np.testing.assert_array_equal(la[k], lb[k])
+
+
+def write_config(d, distil=False):
+    hf = ({"n_layers": 2, "dim": 64, "n_heads": 2, "hidden_dim": 128} if distil else
+          {"num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 2, "intermediate_size": 128, "hidden_act": "gelu"})
+    hf.update({"vocab_size": 100, "max_position_embeddings": 32})
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(hf, f)
+
+
+def test_bert_safetensors_roundtrip(tmp_path):
+    from safetensors.numpy import save_file
+    w = noisy_weights(1)
+    write_config(tmp_path)
+    save_file(bert_state(w), str(tmp_path / "model.safetensors"))
+    cfg, got = load_encoder_checkpoint(str(tmp_path))
+    assert cfg == CFG
+    same(got, w)
+
+
+def test_sentence_transformers_layout_and_torch_bin(tmp_path):
+    torch = pytest.importorskip("torch")
+    w = noisy_weights(2)
+    sub = tmp_path / "0_Transformer"
+    sub.mkdir()
+    write_config(sub)
+    torch.save({k: torch.from_numpy(v) for k, v in bert_state(w, prefix="").items()}, str(sub / "pytorch_model.bin"))
+    cfg, got = load_encoder_checkpoint(str(tmp_path))
+    assert cfg == CFG
+    same(got, w)
+
+
+def test_distilbert_names(tmp_path):
+    from safetensors.numpy import save_file
+    w = noisy_weights(3)
+    w["type_emb"] = np.zeros_like(w["type_emb"])
+    d = CFG.d_model
+    sd = {"distilbert.embeddings.word_embeddings.weight": w["tok_emb"], "distilbert.embeddings.position_embeddings.weight": w["pos_emb"],
+          "distilbert.embeddings.LayerNorm.weight": w["emb_ln_g"], "distilbert.embeddings.LayerNorm.bias": w["emb_ln_b"]}
+    for i, lw in enumerate(w["layers"]):
+        p = f"distilbert.transformer.layer.{i}."
+        for j, t in enumerate(("q_lin", "k_lin", "v_lin")):
+            sd[p + f"attention.{t}.weight"] = lw["w_qkv"][j * d:(j + 1) * d]
+            sd[p + f"attention.{t}.bias"] = lw["b_qkv"][j * d:(j + 1) * d]
+        for name, (wk, bk) in {"attention.out_lin": ("w_o", "b_o"), "sa_layer_norm": ("ln1_g", "ln1_b"), "ffn.lin1": ("w_ff1", "b_ff1"),
+                               "ffn.lin2": ("w_ff2", "b_ff2"), "output_layer_norm": ("ln2_g", "ln2_b")}.items():
+            sd[p + name + ".weight"], sd[p + name + ".bias"] = lw[wk], lw[bk]
+    write_config(tmp_path, distil=True)
+    save_file({k: np.ascontiguousarray(v) for k, v in sd.items()}, str(tmp_path / "model.safetensors"))
+    cfg, got = load_encoder_checkpoint(str(tmp_path))
+    assert cfg == CFG
+    same(got, w)
+
+
+def test_errors(tmp_path):
+    from safetensors.numpy import save_file
+    with pytest.raises(FileNotFoundError):
+        load_encoder_checkpoint(str(tmp_path))
+    write_config(tmp_path)
+    with pytest.raises(FileNotFoundError):
+        load_encoder_checkpoint(str(tmp_path))
+    sd = bert_state(noisy_weights(4))
+    del sd["bert.encoder.layer.1.output.dense.bias"]
+    save_file(sd, str(tmp_path / "model.safetensors"))
+    with pytest.raises(ValueError, match="output.dense.bias"):
+        load_encoder_checkpoint(str(tmp_path))
+    save_file({"x": np.zeros(3, np.float32)}, str(tmp_path / "model.safetensors"))
+    with pytest.raises(ValueError, match="word_embeddings"):
+        load_encoder_checkpoint(str(tmp_path))
+
+
+@pytest.mark.gpu
+def test_imported_checkpoint_runs_like_the_oracle(tmp_path, backend, corc):
+    from safetensors.numpy import save_file
+    from grilly_amd import BertEncoder
+    from oracle import oracle_np as O
+    w = noisy_weights(5)
+    write_config(tmp_path)
+    save_file(bert_state(w), str(tmp_path / "model.safetensors"))
+    cfg, got = load_encoder_checkpoint(str(tmp_path))
+    rng = np.random.default_rng(6)
+    ids = rng.integers(0, cfg.vocab, (3, 20))
+    mask = (np.arange(20)[None] < np.array([20, 9, 14])[:, None]).astype(np.float32)
+    enc = BertEncoder(backend, cfg, got, dtype="fp32")
+    pooled = enc.forward(ids, mask)
+    x = corc.layernorm(corc.embed(ids, w["tok_emb"], w["pos_emb"], w["type_emb"]), w["emb_ln_g"], w["emb_ln_b"], cfg.eps)
+    for lw in w["layers"]:
+        x = corc.bert_layer(x, lw, mask, cfg.heads, cfg.eps)
+    assert O.max_rel(pooled, corc.mean_pool(x, mask)) < 1e-4
