@@ -386,18 +386,29 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     const int b_row0_lds = wave * GB * 8;                                // LDS row in the weight region
     const int b_row0_glb = second ? b_row0_lds - BNO : b_row0_lds;       // row relative to n0 in its matrix
 
-    auto issue = [&](__amdgpu_buffer_rsrc_t rsA, __amdgpu_buffer_rsrc_t rsW, int kt) {
+    // the transfers of wave v's share of slab kt (v is wave-uniform; sec: v's weight rows come from W2)
+    auto issue_for = [&](__amdgpu_buffer_rsrc_t rsA, __amdgpu_buffer_rsrc_t rsWv, int kt, int v, bool sec) {
         char* st = lds + (kt & 1) * STAGE;
         const int sbyte = kt * 128;
+        const int ar = v * GA * 8, br = v * GB * 8, bg = sec ? br - BNO : br;
 #pragma unroll
         for (int j = 0; j < GA; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (__attribute__((address_space(3))) void*)(st + (a_row0 + j * 8) * 128), 16,
-                                                     lane_off_p[j & 1] + (a_row0 + j * 8) * (int)rowbytes, sbyte, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (__attribute__((address_space(3))) void*)(st + (ar + j * 8) * 128), 16,
+                                                     lane_off_p[j & 1] + (ar + j * 8) * (int)rowbytes, sbyte, 0, 0);
 #pragma unroll
         for (int j = 0; j < GB; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsW, (__attribute__((address_space(3))) void*)(st + BM * 128 + (b_row0_lds + j * 8) * 128), 16,
-                                                     lane_off_p[j & 1] + (b_row0_glb + j * 8) * (int)rowbytes, sbyte, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsWv, (__attribute__((address_space(3))) void*)(st + BM * 128 + (br + j * 8) * 128), 16,
+                                                     lane_off_p[j & 1] + (bg + j * 8) * (int)rowbytes, sbyte, 0, 0);
     };
+    auto issue = [&](__amdgpu_buffer_rsrc_t rsA, __amdgpu_buffer_rsrc_t rsW, int kt) { issue_for(rsA, rsW, kt, wave, second); };
+    // Inside the K loop of the 8-wave workgroup only one wave of each SIMD requests the next slab, for itself
+    // and for its SIMD partner (waves w and w^4 share a SIMD), and the two take turns slab by slab: the
+    // requesting wave sits in instruction issue while the address unit works through the queue (measured:
+    // that queue is full 60 % of the time), and its partner keeps the matrix core busy meanwhile.
+    constexpr bool PAIRED = NW == 8;
+    const int pw = wave ^ 4;
+    const bool second_p = DUAL && (pw >= NW / 2);
+    const void* Wsrc_p = second_p ? p.W2 : p.W;
 
     // The bias slice of a tile travels to LDS with the tile's first slab (two buffers, alternating per
     // tile), so the epilogue reads it with LDS latency instead of one global round trip per column group.
@@ -432,6 +443,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     tile_of(pid, m0, n0);
     __amdgpu_buffer_rsrc_t rsA = make_rsrc(p.A, m0, p.M);
     __amdgpu_buffer_rsrc_t rsW = make_rsrc(Wsrc, n0, p.N);
+    __amdgpu_buffer_rsrc_t rsWp = make_rsrc(Wsrc_p, n0, p.N);
     issue(rsA, rsW, 0);
     int bbuf = 0;
     issue_bias(n0, bbuf);
@@ -449,17 +461,24 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
         const int npid = pid + (int)gridDim.x;
         const bool has_next = npid < ntiles;
         int m0n = 0, n0n = 0;
-        __amdgpu_buffer_rsrc_t rsAn = rsA, rsWn = rsW;
+        __amdgpu_buffer_rsrc_t rsAn = rsA, rsWn = rsW, rsWpn = rsWp;
         if (has_next) {
             tile_of(npid, m0n, n0n);
             rsAn = make_rsrc(p.A, m0n, p.M);
             rsWn = make_rsrc(Wsrc, n0n, p.N);
+            rsWpn = make_rsrc(Wsrc_p, n0n, p.N);
         }
 
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's transfers (and earlier stores) are done
         __syncthreads();                         // ... and everybody else's; all staging reads of the last tile too
         for (int kt = 0; kt < KT; ++kt) {
-            if (kt + 1 < KT) issue(rsA, rsW, kt + 1);
+            if (kt + 1 < KT) {
+                if (!PAIRED) issue(rsA, rsW, kt + 1);
+                else if (((wave >> 2) & 1) == (kt & 1)) {
+                    issue_for(rsA, rsW, kt + 1, wave, second);
+                    issue_for(rsA, rsWp, kt + 1, pw, second_p);
+                }
+            }
             const char* s = lds + (kt & 1) * STAGE;
 #pragma unroll
             for (int sl = 0; sl < 4; ++sl) {
@@ -580,7 +599,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
         }
         if (!has_next) break;
-        pid = npid; m0 = m0n; n0 = n0n; rsA = rsAn; rsW = rsWn; bbuf ^= 1;
+        pid = npid; m0 = m0n; n0 = n0n; rsA = rsAn; rsW = rsWn; rsWp = rsWpn; bbuf ^= 1;
     }
 }
 
