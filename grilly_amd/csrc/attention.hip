@@ -511,34 +511,26 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
         }
     }
 
-    for (int t = 1; t < NSTG - 1 && t < nkt; ++t) issue(t);
-    wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1);
-
-    for (int kt = 0; kt < nkt; ++kt) {
-        const int st = kt % NSTG, k0 = kt * KT;
-        // tiles kt+1 .. kt+NSTG-2 may still be in flight; tile kt (this wave's part) must have landed
-        wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1 - kt);
-        // barrier without a memory fence (a fence would wait for every transfer in flight): LDS
-        // writes of this wave are drained by lgkmcnt(0), its tile transfers by the wait above
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        if (kt + NSTG - 1 < nkt) issue(kt + NSTG - 1);   // into the stage tile kt-1 has just left
-        char* Kb = lds + st * TILE;
-        char* Vb = lds + OFF_V + st * TILE;
-        const float* Mb = (const float*)(lds + OFF_M + st * 1024);
+    f32x16 sacc[QT][NKB];
+    // a wave whose queries all precede tile kt has nothing to add (causal): it only keeps the barriers
+    auto skip_tile = [&](int kt) { return p.causal && kt * KT > qw0 + QW - 1; };
+    // last, partial tile: rows >= S hold whatever the out-of-range transfer left; clear them (all threads)
+    auto zero_tail = [&](int kt) {
+        const int k0 = kt * KT;
         if (k0 + KT > S) {
-            // last, partial tile: rows >= S hold whatever the out-of-range transfer left; clear them
-            const int first = S - k0;
+            const int st = kt % NSTG, first = S - k0;
             for (int i = tid; i < (KT - first) * NCH; i += NT) {
                 const u32x4 zero = {0u, 0u, 0u, 0u};
-                *(u32x4*)(Kb + first * RB + i * 16) = zero;
-                *(u32x4*)(Vb + first * RB + i * 16) = zero;
+                *(u32x4*)(lds + st * TILE + first * RB + i * 16) = zero;
+                *(u32x4*)(lds + OFF_V + st * TILE + first * RB + i * 16) = zero;
             }
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
-        // a wave whose queries all precede this tile has nothing to add (causal): it only keeps the barriers
-        if (p.causal && k0 > qw0 + QW - 1) continue;
+    };
 
-        f32x16 sacc[QT][NKB];
+    // ---- score phase: S^T = K . Q^T for tile kt into sacc
+    auto phase_S = [&](int kt) {
+        const char* Kb = lds + (kt % NSTG) * TILE;
         sfor<NKB>([&](auto it) {
             constexpr int t = decltype(it)::value;
 #pragma unroll
@@ -555,7 +547,13 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
             }
         });
 
-        // ---- softmax in the base-2 domain: p = exp2(s*c2 + bias - m)
+    };
+
+    // ---- softmax in the base-2 domain, p = exp2(s*c2 + bias - m), and O^T += V^T . P^T for tile kt
+    auto phase_PV = [&](int kt) {
+        const int st = kt % NSTG, k0 = kt * KT;
+        const char* Vb = lds + OFF_V + st * TILE;
+        const float* Mb = (const float*)(lds + OFF_M + st * 1024);
         const bool diag = p.causal && (k0 + KT - 1 > qw0);
         const bool tail = k0 + KT > S;
         const bool biased = HAS_MASK || tail;
@@ -650,6 +648,24 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
                 });
             }
         });
+    };
+
+    // (A "ping-pong" schedule -- the two waves of a SIMD half a tile apart, one in the score phase while the
+    // other is in the softmax + PV phase, one barrier per half tile -- was built and measured: correct, 6-10 %
+    // slower; inside the PV phase the two waves already overlap each other's VALU and matrix work.)
+    for (int t = 1; t < NSTG - 1 && t < nkt; ++t) issue(t);
+    wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1);
+    for (int kt = 0; kt < nkt; ++kt) {
+        // tiles kt+1 .. kt+NSTG-2 may still be in flight; tile kt (this wave's part) must have landed
+        wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1 - kt);
+        // barrier without a memory fence (a fence would wait for every transfer in flight): LDS
+        // writes of this wave are drained by lgkmcnt(0), its tile transfers by the wait above
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (kt + NSTG - 1 < nkt) issue(kt + NSTG - 1);   // into the stage tile kt-1 has just left
+        zero_tail(kt);
+        if (skip_tile(kt)) continue;
+        phase_S(kt);
+        phase_PV(kt);
     }
 
 #pragma unroll
