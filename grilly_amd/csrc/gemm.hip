@@ -1,698 +1,12 @@
-// MFMA GEMM family for gfx950:  C[m,n] = epi( sum_k A[m,k]*W[n,k] + bias[n] )
-//
-// Both operands are K-contiguous, which is the layout MFMA wants: every lane feeds the
-// matrix core 16 contiguous bytes of one row (8 bf16 for v_mfma_f32_32x32x16_bf16, or
-// 4 fp32 that drive four v_mfma_f32_32x32x2_f32).  A workgroup owns a BM x BN tile of C
-// and walks K in slabs of 128 bytes per row (64 bf16 / 32 fp32):
-//
-//   HBM --128-bit loads--> VGPR --ds_write_b128--> LDS (2 stages, XOR-swizzled 16-B chunks)
-//       --ds_read_b128--> MFMA operands --> fp32 accumulators (registers, never spilled to LDS)
-//       --> bias / GELU / SiLU / SwiGLU epilogue in registers --> 8/16-byte stores
-//
-// The loads for slab t+1 are issued before the MFMAs of slab t and parked in registers, so
-// HBM/L2 latency hides behind the matrix work; one barrier per slab.
-//
-// MFMA operand roles are swapped (the weight rows are the "A" operand, the activation rows
-// the "B" operand) so that each lane ends up with 4 consecutive output columns of one
-// output row: stores are 8 B (bf16) / 16 B (fp32) wide and bias is a 4-vector per lane.
-//
-// LDS bank behaviour: a tile row is 128 B = 8 chunks of 16 B; chunk c of row r lives at
-// slot c ^ lds_swz<8>(r), which makes 16 consecutive rows of one logical chunk (what 16 lanes of a
-// ds_read_b128 fragment read touch) cover all 64 banks exactly once.
-#include "common.hpp"
-#include <type_traits>
-#include <cstdlib>
-#include <algorithm>
+// Host side of the GEMM family: argument checks and the C entry points.  The kernels live in
+// gemm_kernels.hpp; their instantiations are spread over gemm_inst_*.hip (one storage-type pair each)
+// so that they compile in parallel.
+#include "gemm_kernels.hpp"
 
-int grl_transpose2d(grl_ctx* c, int dtype, int64_t R, int64_t C, const void* in, void* out);
-
-struct GemmArgs {
-    const void* A;       // (M,K)
-    const void* W;       // (N,K)
-    const void* W2;      // (N,K) second weight (SwiGLU "up"), else null
-    const float* bias;   // (N) or null
-    const float* bias2;  // (N) or null
-    void* C;             // (M,N)
-    float* cache1;       // fp32 (M,N) pre-activation of W  (SwiGLU gate) or null
-    float* cache2;       // fp32 (M,N) pre-activation of W2 (SwiGLU up) or null
-    int M, N, K;
-    int tiles_m, tiles_n;
-    int group;           // tile-rows per band of the tile walk
-    int act;             // run-time activation code of the EPI_RT / dual epilogues (a GRL_EPI_* value)
-    float alpha, beta;   // RoSwish parameters
-};
-
-// Epilogue template codes.  NONE / GELU / SILU are compiled in (the encoder's hot shapes); EPI_RT picks
-// ReLU / GCU / RoSwish from GemmArgs::act at run time (one more instantiation instead of three), and the
-// dual-weight epilogue EPI_GLU picks the gate activation (SiLU / ReLU / GELU) the same way.
-enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_RT = 3, EPI_GLU = 4 };
-
-// shaders/fused-linear-relu.glsl:63, fused-linear-gcu.glsl:44-46 (x*cos(x)), fused-linear-roswish.glsl:46-58
-// ((x+alpha)*sigmoid(beta*x) - alpha/2; the shader's sign-split sigmoid equals 1/(1+exp(-beta*x)) with the
-// exponential saturating to 0 / +inf)
-__device__ __forceinline__ float act_runtime(float v, const GemmArgs& p) {
-    if (p.act == GRL_EPI_RELU) return fmaxf(v, 0.0f);
-    if (p.act == GRL_EPI_GCU) return v * cosf(v);
-    const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * (p.beta * v)));
-    return (v + p.alpha) * sg - 0.5f * p.alpha;
-}
-template <int EPI> __device__ __forceinline__ float epi_apply(float v, const GemmArgs& p) {
-    if (EPI == EPI_GELU) return gelu_fast(v);
-    if (EPI == EPI_SILU) return silu_clamped(v);
-    if (EPI == EPI_RT) return act_runtime(v, p);
-    return v;
-}
-// gate * act(up): shaders/fused-swiglu.glsl:44-79 (x/(1+exp(-x))), fused-reglu.glsl:74 (max(0,up)),
-// fused-geglu.glsl:44-49,80 (tanh GELU without the clamp rule)
-__device__ __forceinline__ float glu_apply(float gate, float up, const GemmArgs& p) {
-    if (p.act == GRL_EPI_RELU) return gate * fmaxf(up, 0.0f);
-    if (p.act == GRL_EPI_GELU) return gate * gelu_fast(up);
-    return gate * silu_plain(up);
-}
-
-// ---- one 128-byte-per-row K slab on the matrix cores --------------------------------------
-template <typename T> struct MfmaSlab;
-template <> struct MfmaSlab<uint16_t> {   // bf16: 16 B = 8 values, k = 8*(lane/32)+e
-    static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), acc, 0, 0, 0);
-    }
-};
-template <> struct MfmaSlab<float> {      // fp32: 16 B = 4 values, each feeds one 32x32x2 MFMA
-    static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u2f(w[e]), u2f(x[e]), acc, 0, 0, 0);
-    }
-};
-
-// compile-time loop: f(std::integral_constant<int, 0..N-1>)
-template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (N > 0) {
-        static_for<N - 1>(f);
-        f(std::integral_constant<int, N - 1>{});
-    }
-}
-
-template <typename OutT> __device__ __forceinline__ void store4(OutT* p, float a, float b, float c, float d);
-template <> __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
-    f32x4 v = {a, b, c, d};
-    *(f32x4*)p = v;
-}
-template <> __device__ __forceinline__ void store4<uint16_t>(uint16_t* p, float a, float b, float c, float d) {
-    u32x2 v = {pack_bf16x2(a, b), pack_bf16x2(c, d)};
-    *(u32x2*)p = v;
-}
-
-// ---- direct epilogue: lane (li, lg) holds, for output row m = .. + li, the columns
-// n = .. + 8*q + 4*lg + {0..3} in accumulator registers 4q..4q+3 and stores them itself
-// (8- or 16-byte stores).  Every index into the accumulators is a compile-time constant so
-// they stay in registers.  Used for ragged N, for the SwiGLU pre-activation outputs and by the
-// staged kernel.
-template <typename OutT, int TM, int TN, int TNO, int WM, int WNO, int EPI, bool DUAL>
-__device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const GemmArgs& p, int m0, int n0, int wm, int wn, int li, int lg) {
-    OutT* C = (OutT*)p.C;
-    const bool vec_ok = (p.N & 3) == 0;
-    static_for<TM>([&](auto ia) {
-        constexpr int a = decltype(ia)::value;
-        const int m = m0 + wm * WM + a * 32 + li;
-        static_for<TNO>([&](auto ib) {
-            constexpr int b = decltype(ib)::value;
-            static_for<4>([&](auto iq) {
-                constexpr int q = decltype(iq)::value;
-                const int n = n0 + wn * WNO + b * 32 + 8 * q + 4 * lg;
-                if (m < p.M && n < p.N) {
-                    float v[4], u[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        v[e] = acc[a][b][4 * q + e];
-                        u[e] = DUAL ? acc[a][DUAL ? b + TNO : b][4 * q + e] : 0.f;
-                    }
-                    const int64_t o = (int64_t)m * p.N + n;
-                    if (vec_ok) {
-                        if (p.bias) {
-                            f32x4 bv = *(const f32x4*)(p.bias + n);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] += bv[e];
-                        }
-                        if (DUAL) {
-                            if (p.bias2) {
-                                f32x4 bv = *(const f32x4*)(p.bias2 + n);
-#pragma unroll
-                                for (int e = 0; e < 4; ++e) u[e] += bv[e];
-                            }
-                            if (p.cache1) store4<float>(p.cache1 + o, v[0], v[1], v[2], v[3]);
-                            if (p.cache2) store4<float>(p.cache2 + o, u[0], u[1], u[2], u[3]);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = glu_apply(v[e], u[e], p);
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
-                        }
-                        store4<OutT>(C + o, v[0], v[1], v[2], v[3]);
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            if (n + e < p.N) {
-                                float x = v[e] + (p.bias ? p.bias[n + e] : 0.f);
-                                if (DUAL) {
-                                    float y = u[e] + (p.bias2 ? p.bias2[n + e] : 0.f);
-                                    if (p.cache1) p.cache1[o + e] = x;
-                                    if (p.cache2) p.cache2[o + e] = y;
-                                    x = glu_apply(x, y, p);
-                                } else {
-                                    x = epi_apply<EPI>(x, p);
-                                }
-                                elem<OutT>::st(C + o + e, x);
-                            }
-                        }
-                    }
-                }
-            });
-        });
-    });
-}
-
-// BN counts LDS rows of the weight tile; with DUAL it is 2x the output-column count of the
-// tile (first half gate rows, second half up rows).
-template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL>
-__global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
-    constexpr int NT = WGM * WGN * 64;
-    constexpr int EPC = 16 / (int)sizeof(T);     // elements per 16-byte chunk
-    constexpr int BK = 8 * EPC;                  // elements per 128-byte slab row
-    constexpr int WM = BM / WGM, WN = BN / WGN;  // per-wave tile (WN in LDS rows)
-    constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int BNO = DUAL ? BN / 2 : BN;      // output columns per tile
-    constexpr int WNO = DUAL ? WN / 2 : WN;      // output columns per wave
-    constexpr int TNO = DUAL ? TN / 2 : TN;
-    constexpr int CA = BM * 8 / NT, CB = BN * 8 / NT;
-    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile rows must divide over the threads");
-    static_assert(!DUAL || (BN / 2) % (NT / 8) == 0, "a staging pass must not straddle the two weights");
-    static_assert(WM % 32 == 0 && WN % 32 == 0 && (!DUAL || TN % 2 == 0), "wave tile is made of 32x32 MFMA tiles");
-    constexpr int STAGE = (BM + BN) * 128;
-    __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN;
-    const int li = lane & 31, lg = lane >> 5;
-
-    // ---- workgroup -> tile: give each XCD (workgroups are dealt round-robin over the 8 XCDs)
-    // a contiguous run of tiles, and walk tiles in bands of 8 tile-rows so that the 32 CUs of
-    // an XCD share a small set of A and W row panels in their L2.
-    int tile_m, tile_n;
-    {
-        const int nb = gridDim.x, pid = blockIdx.x;
-        const int per = nb >> 3, rem = nb & 7, xcd = pid & 7, loc = pid >> 3;
-        const int npid = xcd * per + (xcd < rem ? xcd : rem) + loc;
-        constexpr int GROUP = 8;
-        const int width = GROUP * p.tiles_n;
-        const int first_m = (npid / width) * GROUP;
-        const int gsize = p.tiles_m - first_m < GROUP ? p.tiles_m - first_m : GROUP;
-        tile_m = first_m + (npid % width) % gsize;
-        tile_n = (npid % width) / gsize;
-    }
-    const int m0 = tile_m * BM, n0 = tile_n * BNO;
-
-    // ---- global -> register staging through buffer loads: the resource starts at the tile's
-    // first row and ends with the tensor, so rows past the edge read as zero in hardware; the
-    // slab offset travels in a scalar register.  Thread t owns chunk (t & 7) of row (t >> 3)
-    // of every 32-row pass; K chunks past the end are zeroed when the slab is written to LDS.
-    constexpr int RPP = NT / 8;                   // rows per pass
-    const int row_t = tid >> 3, c_t = tid & 7;
-    const int64_t rowbytes = (int64_t)p.K * (int64_t)sizeof(T);
-    auto make_rsrc = [&](const void* base, int first_row, int rows_total) {
-        int64_t left = (int64_t)(rows_total - first_row) * rowbytes;
-        if (left < 0) left = 0;
-        uint32_t nrec = left > 0xffffffffLL ? 0xffffffffu : (uint32_t)left;
-        return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base + (int64_t)first_row * rowbytes), 0, (int)nrec, 0x00020000);
-    };
-    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(p.A, m0, p.M);
-    const __amdgpu_buffer_rsrc_t rsW = make_rsrc(p.W, n0, p.N);
-    const __amdgpu_buffer_rsrc_t rsW2 = make_rsrc(DUAL ? p.W2 : p.W, n0, p.N);
-    const int voff = row_t * (int)rowbytes + c_t * 16;
-    const int pass_stride = RPP * (int)rowbytes;
-    static_assert(RPP % 16 == 0, "the swizzle repeats every 16 rows");
-    const int soff_t = row_t * 128 + ((c_t ^ lds_swz<8>(row_t)) << 4);
-
-    u32x4 ra[CA], rb[CB];
-    auto load_slab = [&](int kt) {
-        const int sbyte = kt * 128;
-#pragma unroll
-        for (int i = 0; i < CA; ++i)
-            ra[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsA, voff + i * pass_stride, sbyte, 0));
-#pragma unroll
-        for (int i = 0; i < CB; ++i) {
-            const bool second = DUAL && (i * RPP >= BNO);
-            const int vo = voff + (second ? i - BNO / RPP : i) * pass_stride;
-            rb[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(second ? rsW2 : rsW, vo, sbyte, 0));
-        }
-    };
-    // the K-tail select sits here, after the MFMAs of the previous slab, so that nothing
-    // between the load and this point waits on the data
-    auto stash_slab = [&](int kt) {
-        char* s = lds + (kt & 1) * STAGE + soff_t;
-        const bool live = kt * BK + c_t * EPC < p.K;
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int i = 0; i < CA; ++i) *(u32x4*)(s + i * RPP * 128) = live ? ra[i] : zero;
-#pragma unroll
-        for (int i = 0; i < CB; ++i) *(u32x4*)(s + BM * 128 + i * RPP * 128) = live ? rb[i] : zero;
-    };
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int a = 0; a < TM; ++a)
-#pragma unroll
-        for (int b = 0; b < TN; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-
-    // LDS row of this lane inside each 32-row operand tile
-    int rowX[TM], rowW[TN];
-#pragma unroll
-    for (int a = 0; a < TM; ++a) rowX[a] = wm * WM + a * 32 + li;
-#pragma unroll
-    for (int b = 0; b < TN; ++b) {
-        int base = DUAL ? ((b >= TNO ? BNO : 0) + wn * WNO + (b % TNO) * 32) : (wn * WN + b * 32);
-        rowW[b] = base + li;
-    }
-
-    const int KT = (p.K + BK - 1) / BK;
-    load_slab(0);
-    stash_slab(0);
-    __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const bool more = kt + 1 < KT;
-        if (more) load_slab(kt + 1);
-        const char* s = lds + (kt & 1) * STAGE;
-#pragma unroll
-        for (int sl = 0; sl < 4; ++sl) {
-            const int ch = 2 * sl + lg;
-            u32x4 xf[TM], wf[TN];
-#pragma unroll
-            for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ lds_swz<8>(rowX[a])) << 4));
-#pragma unroll
-            for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ lds_swz<8>(rowW[b])) << 4));
-            static_for<TM>([&](auto ia) {
-                static_for<TN>([&](auto ib) {
-                    MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
-                });
-            });
-        }
-        if (more) stash_slab(kt + 1);
-        __syncthreads();
-    }
-
-    epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
-}
-
-// =====================================================================================
-// Main kernel: persistent workgroups, global -> LDS without passing through registers.
-//
-//   buffer_load_dwordx4 ... lds   writes each wave's 64 x 16 B straight into 1 KiB of LDS
-//   (8 tile rows); the lane -> chunk assignment carries the XOR swizzle, so the LDS image is
-//   the same as in the staged kernel above and the MFMA fragment reads are unchanged.
-//   No staging VGPRs, no ds_write, no select: the slab t+1 transfer runs entirely under the
-//   MFMAs of slab t.  8 waves per 256x256 tile (2 per SIMD) so that one wave's LDS waits hide
-//   under the other's matrix work.
-//
-//   One workgroup per CU walks over its tiles.  When a tile's K loop ends, the first slab of
-//   the NEXT tile is already requested into LDS stage 0 before the epilogue starts, so its
-//   HBM/L2 latency hides under the epilogue, which stages the output through LDS stage 1.
-//
-//   Needs K to be a whole number of 128-byte slabs (the transfer cannot zero a K tail);
-//   M and N are free: rows past the edge are out of range for the buffer resource, read as
-//   zero, and feed only accumulators that are never stored.
-//
-//   Epilogue: accumulators -> bias/activation -> OutT -> LDS (row-major, 16-byte chunks XOR
-//   swizzled by row) -> 16-byte row-contiguous global stores, 32 output rows per wave-row
-//   per pass, two staging regions used alternately so a pass costs one barrier.
-// =====================================================================================
-template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL>
-__global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p) {
-    constexpr int NW = WGM * WGN, NT = NW * 64;
-    constexpr int WM = BM / WGM, WN = BN / WGN;
-    constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int BNO = DUAL ? BN / 2 : BN;
-    constexpr int WNO = DUAL ? WN / 2 : WN;
-    constexpr int TNO = DUAL ? TN / 2 : TN;
-    constexpr int GA = BM / 8 / NW, GB = BN / 8 / NW;      // 8-row groups per wave
-    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "row groups must divide over the waves");
-    static_assert(!DUAL || (NW % 2 == 0), "the two weights split the waves evenly");
-    constexpr int STAGE = (BM + BN) * 128;
-    constexpr int OES = (int)sizeof(OutT);
-    constexpr int CROWB = BNO * OES;                        // bytes per staged output row
-    constexpr int CPR = CROWB / 16;                         // 16-byte chunks per staged row
-    constexpr int RG = WGM * 32 * CROWB;                    // one staging region
-    constexpr int NREG = 2 * RG <= STAGE ? 2 : 1;
-    static_assert(RG <= STAGE && (CPR & (CPR - 1)) == 0, "output staging must fit in LDS stage 1");
-    constexpr int BIASB = BN * 4;                           // one tile's bias slice(s), fp32
-    __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + 2 * BIASB];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN;
-    const int li = lane & 31, lg = lane >> 5;
-    const int ntiles = p.tiles_m * p.tiles_n;
-
-    // workgroup id -> tile: give each XCD (workgroup ids are dealt round-robin over the 8 XCDs,
-    // and the persistent stride is a multiple of 8) a contiguous run of tiles, walked in bands
-    // of 8 tile-rows so that the 32 CUs of an XCD share few A and W row panels in their L2.
-    auto tile_of = [&](int pid, int& m0, int& n0) {
-        const int per = ntiles >> 3, rem = ntiles & 7, xcd = pid & 7, loc = pid >> 3;
-        const int npid = xcd * per + (xcd < rem ? xcd : rem) + loc;
-        const int GROUP = p.group;
-        const int width = GROUP * p.tiles_n;
-        const int first_m = (npid / width) * GROUP;
-        const int gsize = p.tiles_m - first_m < GROUP ? p.tiles_m - first_m : GROUP;
-        m0 = (first_m + (npid % width) % gsize) * BM;
-        n0 = ((npid % width) / gsize) * BNO;
-    };
-
-    const int64_t rowbytes = (int64_t)p.K * (int64_t)sizeof(T);
-    auto make_rsrc = [&](const void* base, int first_row, int rows_total) {
-        int64_t left = (int64_t)(rows_total - first_row) * rowbytes;
-        if (left < 0) left = 0;
-        uint32_t nrec = left > 0xffffffffLL ? 0xffffffffu : (uint32_t)left;
-        return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base + (int64_t)first_row * rowbytes), 0, (int)nrec, 0x00020000);
-    };
-    // with two weights the lower half of the waves fetches the gate rows, the upper half the up rows
-    const bool second = DUAL && (wave >= NW / 2);
-    const void* Wsrc = second ? p.W2 : p.W;
-    const int lr = lane >> 3, ls = lane & 7;
-    // lane -> (row lr of an 8-row group, slot ls): LDS slot ls of row r holds chunk ls ^ lds_swz<8>(r).
-    // The swizzle depends on bits 1-3 of r, i.e. on lr and on whether the group is an even or odd one.
-    static_assert(GA % 2 == 0 && GB % 2 == 0, "group parity is the transfer index parity");
-    const int lane_off_p[2] = {lr * (int)rowbytes + ((ls ^ lds_swz<8>(lr)) << 4), lr * (int)rowbytes + ((ls ^ lds_swz<8>(8 + lr)) << 4)};
-    const int a_row0 = wave * GA * 8;                                    // first A tile row of this wave
-    const int b_row0_lds = wave * GB * 8;                                // LDS row in the weight region
-    const int b_row0_glb = second ? b_row0_lds - BNO : b_row0_lds;       // row relative to n0 in its matrix
-
-    // the transfers of wave v's share of slab kt (v is wave-uniform; sec: v's weight rows come from W2)
-    auto issue_for = [&](__amdgpu_buffer_rsrc_t rsA, __amdgpu_buffer_rsrc_t rsWv, int kt, int v, bool sec) {
-        char* st = lds + (kt & 1) * STAGE;
-        const int sbyte = kt * 128;
-        const int ar = v * GA * 8, br = v * GB * 8, bg = sec ? br - BNO : br;
-#pragma unroll
-        for (int j = 0; j < GA; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (__attribute__((address_space(3))) void*)(st + (ar + j * 8) * 128), 16,
-                                                     lane_off_p[j & 1] + (ar + j * 8) * (int)rowbytes, sbyte, 0, 0);
-#pragma unroll
-        for (int j = 0; j < GB; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsWv, (__attribute__((address_space(3))) void*)(st + BM * 128 + (br + j * 8) * 128), 16,
-                                                     lane_off_p[j & 1] + (bg + j * 8) * (int)rowbytes, sbyte, 0, 0);
-    };
-    auto issue = [&](__amdgpu_buffer_rsrc_t rsA, __amdgpu_buffer_rsrc_t rsW, int kt) { issue_for(rsA, rsW, kt, wave, second); };
-    // Inside the K loop of the 8-wave workgroup only one wave of each SIMD requests the next slab, for itself
-    // and for its SIMD partner (waves w and w^4 share a SIMD), and the two take turns slab by slab: the
-    // requesting wave sits in instruction issue while the address unit works through the queue (measured:
-    // that queue is full 60 % of the time), and its partner keeps the matrix core busy meanwhile.
-    constexpr bool PAIRED = NW == 8;
-    const int pw = wave ^ 4;
-    const bool second_p = DUAL && (pw >= NW / 2);
-    const void* Wsrc_p = second_p ? p.W2 : p.W;
-
-    // The bias slice of a tile travels to LDS with the tile's first slab (two buffers, alternating per
-    // tile), so the epilogue reads it with LDS latency instead of one global round trip per column group.
-    // Wave 0 fetches bias[n0 .. n0+BNO), the first wave of the upper half bias2 (columns past N read zero).
-    auto issue_bias = [&](int n0t, int buf) {
-        const bool w1 = wave == 0 && p.bias, w2 = DUAL && wave == NW / 2 && p.bias2;
-        if ((w1 || w2) && lane < BNO / 4) {
-            const float* src = (w2 ? p.bias2 : p.bias) + n0t;
-            int left = (p.N - n0t) * 4;
-            __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, left > 0 ? left : 0, 0x00020000);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + 2 * STAGE + buf * BIASB + (w2 ? BNO * 4 : 0)),
-                                                     16, lane * 16, 0, 0, 0);
-        }
-    };
-
-    int rowX[TM], rowW[TN];
-#pragma unroll
-    for (int a = 0; a < TM; ++a) rowX[a] = wm * WM + a * 32 + li;
-#pragma unroll
-    for (int b = 0; b < TN; ++b) {
-        int base = DUAL ? ((b >= TNO ? BNO : 0) + wn * WNO + (b % TNO) * 32) : (wn * WN + b * 32);
-        rowW[b] = base + li;
-    }
-
-    constexpr int BKE = 128 / (int)sizeof(T);
-    const int KT = p.K / BKE;
-    OutT* C = (OutT*)p.C;
-    const bool staged = ((int64_t)p.N * OES) % 16 == 0 && !p.cache1 && !p.cache2;
-
-    int pid = blockIdx.x;
-    int m0, n0;
-    tile_of(pid, m0, n0);
-    __amdgpu_buffer_rsrc_t rsA = make_rsrc(p.A, m0, p.M);
-    __amdgpu_buffer_rsrc_t rsW = make_rsrc(Wsrc, n0, p.N);
-    __amdgpu_buffer_rsrc_t rsWp = make_rsrc(Wsrc_p, n0, p.N);
-    issue(rsA, rsW, 0);
-    int bbuf = 0;
-    issue_bias(n0, bbuf);
-
-    for (;;) {
-        f32x16 acc[TM][TN];
-#pragma unroll
-        for (int a = 0; a < TM; ++a)
-#pragma unroll
-            for (int b = 0; b < TN; ++b)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-
-        // where the next tile is: index arithmetic done here hides under the wait for the first slab
-        const int npid = pid + (int)gridDim.x;
-        const bool has_next = npid < ntiles;
-        int m0n = 0, n0n = 0;
-        __amdgpu_buffer_rsrc_t rsAn = rsA, rsWn = rsW, rsWpn = rsWp;
-        if (has_next) {
-            tile_of(npid, m0n, n0n);
-            rsAn = make_rsrc(p.A, m0n, p.M);
-            rsWn = make_rsrc(Wsrc, n0n, p.N);
-            rsWpn = make_rsrc(Wsrc_p, n0n, p.N);
-        }
-
-        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's transfers (and earlier stores) are done
-        __syncthreads();                         // ... and everybody else's; all staging reads of the last tile too
-        for (int kt = 0; kt < KT; ++kt) {
-            if (kt + 1 < KT) {
-                if (!PAIRED) issue(rsA, rsW, kt + 1);
-                else if (((wave >> 2) & 1) == (kt & 1)) {
-                    issue_for(rsA, rsW, kt + 1, wave, second);
-                    issue_for(rsA, rsWp, kt + 1, pw, second_p);
-                }
-            }
-            const char* s = lds + (kt & 1) * STAGE;
-#pragma unroll
-            for (int sl = 0; sl < 4; ++sl) {
-                const int ch = 2 * sl + lg;
-                u32x4 xf[TM], wf[TN];
-#pragma unroll
-                for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ lds_swz<8>(rowX[a])) << 4));
-#pragma unroll
-                for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ lds_swz<8>(rowW[b])) << 4));
-                static_for<TM>([&](auto ia) {
-                    static_for<TN>([&](auto ib) {
-                        MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
-                    });
-                });
-            }
-            __builtin_amdgcn_s_waitcnt(0x0f70);
-            __syncthreads();
-        }
-
-        // both LDS stages are free now: request the next tile's first slab into stage 0
-        if (has_next) {
-            issue(rsAn, rsWn, 0);
-            issue_bias(n0n, bbuf ^ 1);
-        }
-
-        if (staged) {
-            // ---- LDS-staged epilogue in stage 1, one 32-row band of every wave-row per pass
-            constexpr int EPCO = 16 / OES;
-            char* stg = lds + STAGE;
-            const char* bias_lds = lds + 2 * STAGE + bbuf * BIASB;
-            // bias of this lane's 4-column groups, once per tile (columns past N hold zero)
-            f32x4 bv1[TNO][4], bv2[TNO][4];
-#pragma unroll
-            for (int b = 0; b < TNO; ++b)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
-                    bv1[b][q] = p.bias ? *(const f32x4*)(bias_lds + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
-                    if (DUAL) bv2[b][q] = p.bias2 ? *(const f32x4*)(bias_lds + BNO * 4 + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
-                }
-            constexpr int TOTAL = WGM * 32 * CPR;
-            static_assert(TOTAL % NT == 0, "staged chunks divide over the threads");
-            constexpr int PER = TOTAL / NT;
-            const int r_w = wm * 32 + li;
-            // bias/activation/convert band `a` of every wave-row into its staging region.  Columns past N
-            // carry zero accumulators (their weight rows read as zero); they are converted like the rest
-            // and dropped at the global store.
-            auto stage_band = [&](auto ia) {
-                constexpr int a = decltype(ia)::value;
-                char* crow = stg + (NREG == 2 ? (a & 1) * RG : 0) + r_w * CROWB;
-                static_for<TNO>([&](auto ib) {
-                    constexpr int b = decltype(ib)::value;
-                    static_for<4>([&](auto iq) {
-                        constexpr int q = decltype(iq)::value;
-                        const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
-                        float v[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] + bv1[b][q][e];
-                        if (DUAL) {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = glu_apply(v[e], acc[a][DUAL ? b + TNO : b][4 * q + e] + bv2[b][q][e], p);
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
-                        }
-                        const int byte = nl * OES;
-                        const int chunk = (byte >> 4) ^ (r_w & (CPR - 1));
-                        store4<OutT>((OutT*)(crow + (chunk << 4) + (byte & 15)), v[0], v[1], v[2], v[3]);
-                    });
-                });
-            };
-            auto fetch_band = [&](auto ia, u32x4 (&val)[PER]) {
-                constexpr int a = decltype(ia)::value;
-                const char* reg = stg + (NREG == 2 ? (a & 1) * RG : 0);
-#pragma unroll
-                for (int i = 0; i < PER; ++i) {
-                    const int id = tid + i * NT;
-                    const int r = id / CPR, cc = id % CPR;
-                    val[i] = *(const u32x4*)(reg + r * CROWB + ((cc ^ (r & (CPR - 1))) << 4));
-                }
-            };
-            auto store_band = [&](auto ia, const u32x4 (&val)[PER]) {
-                constexpr int a = decltype(ia)::value;
-#pragma unroll
-                for (int i = 0; i < PER; ++i) {
-                    const int id = tid + i * NT;
-                    const int r = id / CPR, cc = id % CPR;
-                    const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
-                    const int n = n0 + cc * EPCO;
-                    // written once, read by another kernel: keep it from displacing the operand panels in L2
-                    if (m < p.M && n < p.N) __builtin_nontemporal_store(val[i], (u32x4*)(C + (int64_t)m * p.N + n));
-                }
-            };
-            // Barriers here are LDS-only (a fence would also wait for the global stores of earlier bands).
-            if constexpr (NREG == 2) {
-                // two regions: band a+1 is converted and written while band a's staged rows are on their
-                // way back from LDS, one barrier per band
-                stage_band(std::integral_constant<int, 0>{});
-                static_for<TM>([&](auto ia) {
-                    constexpr int a = decltype(ia)::value;
-                    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                    u32x4 val[PER];
-                    fetch_band(ia, val);
-                    if constexpr (a + 1 < TM) stage_band(std::integral_constant<int, a + 1>{});
-                    store_band(ia, val);
-                });
-            } else {
-                static_for<TM>([&](auto ia) {
-                    stage_band(ia);
-                    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                    u32x4 val[PER];
-                    fetch_band(ia, val);
-                    store_band(ia, val);
-                    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                });
-            }
-        } else {
-            epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
-        }
-        if (!has_next) break;
-        pid = npid; m0 = m0n; n0 = n0n; rsA = rsAn; rsW = rsWn; rsWp = rsWpn; bbuf ^= 1;
-    }
-}
-
-// ---- any shape / any alignment: one thread per output, ascending-k fp32 sum (the summation
-// order of shaders/fnn-linear.glsl:45-49).  Used only when rows are not 16-byte aligned.
-template <typename T, typename OutT, int EPI, bool DUAL>
-__global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmArgs p) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (int64_t)p.M * p.N) return;
-    const int m = (int)(idx / p.N), n = (int)(idx % p.N);
-    const T* a = (const T*)p.A + (int64_t)m * p.K;
-    const T* w = (const T*)p.W + (int64_t)n * p.K;
-    float s = 0.f;
-    for (int k = 0; k < p.K; ++k) s += elem<T>::ld(a + k) * elem<T>::ld(w + k);
-    if (p.bias) s += p.bias[n];
-    if (DUAL) {
-        const T* w2 = (const T*)p.W2 + (int64_t)n * p.K;
-        float u = 0.f;
-        for (int k = 0; k < p.K; ++k) u += elem<T>::ld(a + k) * elem<T>::ld(w2 + k);
-        if (p.bias2) u += p.bias2[n];
-        if (p.cache1) p.cache1[idx] = s;
-        if (p.cache2) p.cache2[idx] = u;
-        s = glu_apply(s, u, p);
-    } else {
-        s = epi_apply<EPI>(s, p);
-    }
-    elem<OutT>::st((OutT*)p.C + idx, s);
-}
-
-// ------------------------------------------------------------------ host dispatch
-template <typename T, typename OutT, int EPI, bool DUAL>
-static int launch_gemm(grl_ctx* c, GemmArgs& a) {
-    const int64_t epc = 16 / (int64_t)sizeof(T);
-    const bool aligned = (a.K % epc == 0) && ((((uintptr_t)a.A) | ((uintptr_t)a.W) | ((uintptr_t)a.W2)) & 15u) == 0 &&
-                         ((((uintptr_t)a.C) | ((uintptr_t)a.bias) | ((uintptr_t)a.bias2) | ((uintptr_t)a.cache1) | ((uintptr_t)a.cache2)) & 15u) == 0;
-    if (!aligned) {
-        int64_t total = (int64_t)a.M * a.N;
-        GRL_REQUIRE((total + 255) / 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: unaligned problem too large for the scalar kernel");
-        hipLaunchKernelGGL((gemm_nt_scalar_kernel<T, OutT, EPI, DUAL>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, a);
-        GRL_CHECK_LAUNCH();
-        return GRL_OK;
-    }
-    // Tile choice.  The direct-to-LDS kernel needs whole 128-byte K slabs; the 256x256 tile is
-    // used once it yields enough workgroups to occupy most of the 256 CUs, else 128x128 tiles.
-    // GRL_GEMM_VARIANT (1..4) forces one variant, for tuning runs.
-    static const int forced = [] { const char* e = getenv("GRL_GEMM_VARIANT"); return e ? atoi(e) : 0; }();
-    // band height of the tile walk: rows of 8 KiB and more do better with narrow bands (measured)
-    static const int group = [] { const char* e = getenv("GRL_GEMM_GROUP"); return e ? atoi(e) : 0; }();
-    a.group = group > 0 ? group : (a.K * (int64_t)sizeof(T) >= 8192 ? 2 : 8);
-    const int64_t bke = 128 / (int64_t)sizeof(T);
-    const int64_t big_m = (a.M + 255) / 256, big_n = (a.N + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
-    const int64_t sm = (a.M + 127) / 128, sn = (a.N + (DUAL ? 63 : 127)) / (DUAL ? 64 : 128);
-    GRL_REQUIRE(sm * sn < (1LL << 31), GRL_ERR_SHAPE, "gemm: too many tiles");
-    GRL_REQUIRE(a.K * (int64_t)sizeof(T) * 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: K too large (256 rows must span < 2 GiB)");
-    const bool slabs = a.K % bke == 0;
-    const bool big = big_m * big_n >= 192;
-    const int64_t cus = c->prop.multiProcessorCount;     // one 128 KiB-LDS workgroup per CU, two of the 64 KiB ones
-    int variant = slabs ? (big ? 3 : 4) : (big ? 1 : 2);
-    if (forced >= 1 && forced <= 4 && (slabs || forced <= 2)) variant = forced;
-    switch (variant) {
-        case 1:
-            a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
-            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 256, 256, 2, 2, EPI, DUAL>), dim3((unsigned)(big_m * big_n)), dim3(256), 0, c->stream, a);
-            break;
-        case 2:
-            a.tiles_m = (int)sm; a.tiles_n = (int)sn;
-            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)(sm * sn)), dim3(256), 0, c->stream, a);
-            break;
-        case 3:
-            a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
-            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 256, 256, 2, 4, EPI, DUAL>), dim3((unsigned)std::min<int64_t>(big_m * big_n, cus)), dim3(512), 0, c->stream, a);
-            break;
-        default:
-            a.tiles_m = (int)sm; a.tiles_n = (int)sn;
-            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)std::min<int64_t>(sm * sn, 2 * cus)), dim3(256), 0, c->stream, a);
-            break;
-    }
-    GRL_CHECK_LAUNCH();
-    return GRL_OK;
-}
-
-template <typename T, typename OutT>
-static int dispatch_epi(grl_ctx* c, GemmArgs& a, int epi) {
-    switch (epi) {
-        case EPI_NONE: return launch_gemm<T, OutT, EPI_NONE, false>(c, a);
-        case EPI_GELU: return launch_gemm<T, OutT, EPI_GELU, false>(c, a);
-        case EPI_SILU: return launch_gemm<T, OutT, EPI_SILU, false>(c, a);
-        case EPI_RT: return launch_gemm<T, OutT, EPI_RT, false>(c, a);
-        case EPI_GLU: return launch_gemm<T, OutT, EPI_GLU, true>(c, a);
-    }
-    grl_set_error("gemm: bad epilogue %d", epi);
-    return GRL_ERR_ARG;
-}
+extern template int dispatch_epi<float, float>(grl_ctx*, GemmArgs&, int);
+extern template int dispatch_epi<uint16_t, uint16_t>(grl_ctx*, GemmArgs&, int);
+extern template int dispatch_epi<uint16_t, float>(grl_ctx*, GemmArgs&, int);
+extern template int dispatch_epi<float, uint16_t>(grl_ctx*, GemmArgs&, int);
 
 static int dispatch_types(grl_ctx* c, GemmArgs& a, int in_dtype, int out_dtype, int epi) {
     if (in_dtype == GRL_F32 && out_dtype == GRL_F32) return dispatch_epi<float, float>(c, a, epi);

@@ -1,0 +1,4 @@
+// GEMM kernel instantiations for operands stored as uint16_t and outputs stored as float.
+#include "gemm_kernels.hpp"
+
+template int dispatch_epi<uint16_t, float>(grl_ctx*, GemmArgs&, int);

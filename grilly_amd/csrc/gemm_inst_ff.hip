@@ -1,0 +1,4 @@
+// GEMM kernel instantiations for operands stored as float and outputs stored as float.
+#include "gemm_kernels.hpp"
+
+template int dispatch_epi<float, float>(grl_ctx*, GemmArgs&, int);
