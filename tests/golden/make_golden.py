@@ -59,6 +59,15 @@ def build():
     ml = (np.arange(24)[None] < np.array([24, 13])[:, None]).astype(np.float32)
     g.update({f"layer_{k_}": v_ for k_, v_ in w.items()})
     g.update(layer_x=xl, layer_mask=ml, layer_y=f32(O.truth_bert_layer(xl, w, ml, H)))
+
+    # further epilogues on the same inputs (appended last so that the arrays above keep their values)
+    g.update(lin_relu=f32(O.truth_linear(x, W, b, "relu")), lin_gcu=f32(O.truth_linear(x, W, b, "gcu")),
+             lin_roswish=f32(O.truth_linear(x, W, b, "roswish", 0.7, 1.3)),
+             glu_relu=f32(O.truth_fused_glu(x, Wg, Wu, bg, bu, "relu")[0]),
+             glu_gelu=f32(O.truth_fused_glu(x, Wg, Wu, bg, bu, "gelu")[0]),
+             ew_relu=f32(np.maximum(e, 0)))
+    Wl, bl = n(20, 384) * 0.1, n(20)
+    g.update(lnlin_W=Wl, lnlin_b=bl, lnlin_y=f32(O.truth_linear(O.truth_layernorm(xr, gam, bet), Wl, bl)))
     return g
 
 

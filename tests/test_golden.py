@@ -47,6 +47,12 @@ def test_c_oracle_matches_golden(corc):
     assert O.max_rel(corc.silu(G["ew_x"]), G["ew_silu"]) < 1e-5
     assert O.max_rel(corc.swiglu_act(G["ln_x"]), G["ew_swiglu"]) < 1e-5
     assert O.max_rel(corc.bert_layer(G["layer_x"], layer_weights(), G["layer_mask"], 2), G["layer_y"]) < 1e-5
+    assert O.max_rel(corc.linear(x, G["lin_W"], G["lin_b"], "relu"), G["lin_relu"]) < 1e-5
+    assert O.max_rel(corc.linear(x, G["lin_W"], G["lin_b"], "gcu"), G["lin_gcu"]) < 1e-5
+    assert O.max_rel(corc.linear(x, G["lin_W"], G["lin_b"], "roswish", 0.7, 1.3), G["lin_roswish"]) < 1e-5
+    assert O.max_rel(corc.fused_glu(x, G["sw_Wg"], G["sw_Wu"], G["sw_bg"], G["sw_bu"], "relu")[0], G["glu_relu"]) < 1e-5
+    assert O.max_rel(corc.fused_glu(x, G["sw_Wg"], G["sw_Wu"], G["sw_bg"], G["sw_bu"], "gelu")[0], G["glu_gelu"]) < 1e-5
+    assert O.max_rel(corc.linear(corc.layernorm(G["ln_x"], G["ln_g"], G["ln_b"]), G["lnlin_W"], G["lnlin_b"]), G["lnlin_y"]) < 1e-5
 
 
 @pytest.mark.gpu
@@ -71,6 +77,13 @@ def test_hip_path_matches_golden(backend):
     assert O.max_rel(f.activation_gelu(G["ew_x"]), G["ew_gelu"]) < TOL_F32
     assert O.max_rel(f.activation_silu(G["ew_x"]), G["ew_silu"]) < TOL_F32
     assert O.max_rel(f.activation_swiglu(G["ln_x"]), G["ew_swiglu"]) < TOL_F32
+    assert O.max_rel(f.fused_linear_relu(x, G["lin_W"], G["lin_b"]), G["lin_relu"]) < TOL_F32
+    assert O.max_rel(f.fused_linear_gcu(x, G["lin_W"], G["lin_b"]), G["lin_gcu"]) < TOL_F32
+    assert O.max_rel(f.fused_linear_roswish(x, G["lin_W"], G["lin_b"], alpha=0.7, beta=1.3), G["lin_roswish"]) < TOL_F32
+    assert O.max_rel(f.fused_reglu(x, G["sw_Wg"], G["sw_Wu"], G["sw_bg"], G["sw_bu"]), G["glu_relu"]) < TOL_F32
+    assert O.max_rel(f.fused_geglu(x, G["sw_Wg"], G["sw_Wu"], G["sw_bg"], G["sw_bu"]), G["glu_gelu"]) < TOL_F32
+    np.testing.assert_array_equal(f.activation_relu(G["ew_x"]), G["ew_relu"])
+    assert O.max_rel(f.fused_layernorm_linear(G["ln_x"], G["ln_g"], G["ln_b"], G["lnlin_W"], G["lnlin_b"]), G["lnlin_y"]) < TOL_F32
     # the encoder layer through the device-pointer entry point
     import ctypes
     from grilly_amd import _lib as L
