@@ -82,6 +82,20 @@ template <> __device__ __forceinline__ u32x4 rope_chunk<uint16_t>(u32x4 v, const
     }
     return o;
 }
+// 8 bf16 values times a scalar, optionally rotated first (one rounding at the end)
+template <bool ROT> __device__ __forceinline__ u32x4 scale_chunk_bf16(u32x4 v, const float2* cs, float scale) {
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float x0 = bf16lo(v[i]), x1 = bf16hi(v[i]);
+        if (ROT) {
+            const float r0 = x0 * cs[i].x - x1 * cs[i].y, r1 = x0 * cs[i].y + x1 * cs[i].x;
+            x0 = r0; x1 = r1;
+        }
+        o[i] = pack_bf16x2(x0 * scale, x1 * scale);
+    }
+    return o;
+}
 
 template <typename OutT> __device__ __forceinline__ void fa_store4(OutT* p, float a, float b, float c, float d);
 template <> __device__ __forceinline__ void fa_store4<float>(float* p, float a, float b, float c, float d) {
@@ -501,13 +515,13 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
         for (int s = 0; s < NS; ++s) {
             const int c = 2 * s + lg;
             u32x4 v = *(const u32x4*)(Qg + (int64_t)qc * p.q_stride + c * 8);
+            // queries carry scale*log2(e): the matrix core then delivers scores in the base-2 softmax domain
+            float2 cs[4];
             if (ROPE_Q) {
-                float2 cs[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) cs[i] = p.rope[(int64_t)qc * (D / 2) + c * 4 + i];
-                v = rope_chunk<uint16_t>(v, cs);
             }
-            qf[t][s] = v;
+            qf[t][s] = scale_chunk_bf16<ROPE_Q>(v, cs, c2);
         }
     }
 
@@ -528,15 +542,29 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
         }
     };
 
-    // ---- score phase: S^T = K . Q^T for tile kt into sacc
+    // A tile without mask, diagonal or ragged end, other than the first one, is a "lazy" tile: its score
+    // accumulators start at -m_run, so the matrix core hands back s - m_run and the exponentials need no
+    // further arithmetic; m_run is raised (with the usual rescale) only when a score exceeds it by more
+    // than 2^LAZY.  m_run is then a reference point at most LAZY below the true running maximum, which
+    // the softmax quotient does not depend on.
+    constexpr float LAZY = 6.0f;
+    auto is_lazy = [&](int kt) {
+        const int k0 = kt * KT;
+        return kt > 0 && !HAS_MASK && !(k0 + KT > S) && !(p.causal && (k0 + KT - 1 > qw0));
+    };
+
+    // ---- score phase: S^T = K . Q'^T for tile kt into sacc (Q' = Q * scale * log2 e)
     auto phase_S = [&](int kt) {
         const char* Kb = lds + (kt % NSTG) * TILE;
+        const bool lazy = is_lazy(kt);
         sfor<NKB>([&](auto it) {
             constexpr int t = decltype(it)::value;
 #pragma unroll
-            for (int u = 0; u < QT; ++u)
+            for (int u = 0; u < QT; ++u) {
+                const float init = lazy ? -m_run[u] : 0.f;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[u][t][r] = 0.f;
+                for (int r = 0; r < 16; ++r) sacc[u][t][r] = init;
+            }
             const int key = 32 * t + li;
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
@@ -557,7 +585,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
         const bool diag = p.causal && (k0 + KT - 1 > qw0);
         const bool tail = k0 + KT > S;
         const bool biased = HAS_MASK || tail;
-        float pmul[QT], pneg[QT];     // p = exp2(score * pmul + pneg), formed block by block below
+        const bool lazy = is_lazy(kt);
+        float pneg[QT];               // p = exp2(score + pneg); all zero on the fast path
+        bool fast = lazy;             // wave-uniform
         sfor<QT>([&](auto iu) {
             constexpr int u = decltype(iu)::value;
             const int qi = qw0 + 32 * u + li;
@@ -573,7 +603,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             // (mask-1)*1e9 as the shader forms it, then into the base-2 domain
-                            float sv = sacc[u][t][4 * qd + e] * c2;
+                            float sv = sacc[u][t][4 * qd + e];
                             if (HAS_MASK) sv += ((mk[e] - 1.0f) * 1e9f) * 1.4426950408889634f;
                             if ((diag && (k0 + kl + e > qi)) || (tail && (k0 + kl + e >= S))) sv = -__builtin_inff();
                             sacc[u][t][4 * qd + e] = sv;
@@ -581,37 +611,52 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
                         }
                     }
                 });
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                mx = fmaxf(m_run[u], mx);
-                pmul[u] = 1.0f;          // scores are already scaled and biased
             } else {
-                // plain tile: the max is taken on the raw products (c2 > 0) and the scale rides in the fma
                 sfor<NKB>([&](auto it) {
                     constexpr int t = decltype(it)::value;
 #pragma unroll
                     for (int r = 0; r < 16; r += 2) mx = __builtin_fmaxf(mx, __builtin_fmaxf(sacc[u][t][r], sacc[u][t][r + 1]));
                 });
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                mx = fmaxf(m_run[u], mx * c2);
-                pmul[u] = c2;
             }
-            pneg[u] = -mx;
-            const float alpha = __builtin_amdgcn_exp2f(m_run[u] - mx);
-            // rescale the running output and sum only when some row of the wave raised its maximum
-            if (__builtin_amdgcn_ballot_w64(mx != m_run[u]) != 0) {
-                lacc[u][0] *= alpha;
-                sfor<DT>([&](auto idt) {
-                    constexpr int dt = decltype(idt)::value;
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            if (!lazy) {
+                // absolute scores: the classic running maximum
+                mx = fmaxf(m_run[u], mx);
+                pneg[u] = -mx;
+                const float alpha = __builtin_amdgcn_exp2f(m_run[u] - mx);
+                // rescale the running output and sum only when some row of the wave raised its maximum
+                if (__builtin_amdgcn_ballot_w64(mx != m_run[u]) != 0) {
+                    lacc[u][0] *= alpha;
+                    sfor<DT>([&](auto idt) {
+                        constexpr int dt = decltype(idt)::value;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[u][dt][r] *= alpha;
-                });
+                        for (int r = 0; r < 16; ++r) oacc[u][dt][r] *= alpha;
+                    });
+                }
+                m_run[u] = mx;
+            } else {
+                // scores relative to m_run: move the reference only for rows that overshoot it by 2^LAZY
+                const float delta = mx > LAZY ? mx : 0.f;
+                pneg[u] = -delta;
+                if (__builtin_amdgcn_ballot_w64(delta != 0.f) != 0) {
+                    const float alpha = __builtin_amdgcn_exp2f(-delta);
+                    lacc[u][0] *= alpha;
+                    sfor<DT>([&](auto idt) {
+                        constexpr int dt = decltype(idt)::value;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) oacc[u][dt][r] *= alpha;
+                    });
+                    m_run[u] += delta;
+                    fast = false;
+                }
             }
-            m_run[u] = mx;
         });
 
         // ---- O^T += V^T . P^T; V operand through the transposing LDS read
         // source role of this lane inside its 16-lane group: key row j/4, 4 dims at 4*(j%4)
         const int j16 = lane & 15, grp = lane >> 4;
+        auto pv_loop = [&](auto ifast) {
+        constexpr bool FAST = decltype(ifast)::value;
         sfor<NKB>([&](auto it) {
             constexpr int t = decltype(it)::value;
 #pragma unroll
@@ -623,8 +668,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
                 for (int u = 0; u < QT; ++u)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][t][8 * hh + 2 * e], pmul[u], pneg[u]));
-                        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][t][8 * hh + 2 * e + 1], pmul[u], pneg[u]));
+                        const float p0 = __builtin_amdgcn_exp2f(FAST ? sacc[u][t][8 * hh + 2 * e] : sacc[u][t][8 * hh + 2 * e] + pneg[u]);
+                        const float p1 = __builtin_amdgcn_exp2f(FAST ? sacc[u][t][8 * hh + 2 * e + 1] : sacc[u][t][8 * hh + 2 * e + 1] + pneg[u]);
                         pf[u][e] = pack_bf16x2(p0, p1);
                     }
                 // row sums: P^T against an all-ones (bf16 1.0) operand
@@ -648,6 +693,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
                 });
             }
         });
+        };
+        if (fast) pv_loop(std::true_type{}); else pv_loop(std::false_type{});
     };
 
     // (A "ping-pong" schedule -- the two waves of a SIMD half a tile apart, one in the score phase while the
@@ -723,8 +770,9 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, bool rope_q) {
         case 1: return launch_fa16_cfg<D, 1, 8, DEEP, 64>(c, f, rope_q);
         case 2: return launch_fa16_cfg<D, 1, 8, DEEP / 2, 128>(c, f, rope_q);
         case 4: return launch_fa16_cfg<D, 1, 4, 2, (D == 128 ? 64 : 128)>(c, f, rope_q);
-        default: return launch_fa16_cfg<D, 1, 4, 4, 64>(c, f, rope_q);
+        default: break;
     }
+    return launch_fa16_cfg<D, 1, 4, 4, 64>(c, f, rope_q);
 }
 
 template <typename T, int D>
