@@ -404,8 +404,8 @@ template <int IPT, int MAXT> __device__ __forceinline__ void wait_tiles_outstand
     }
 }
 
-template <int D, bool ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK, int KT>
-__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16Args p) {
+template <int D, bool ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK, int KT, int OCC = (NW == 4 ? 2 : 1)>
+__global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     // QT = 32-query MFMA tiles per wave (every K / V fragment read from LDS feeds QT MFMAs),
     // NW waves per workgroup, NSTG-deep ring of 64-key K/V tiles in LDS (NSTG-1 tiles in flight).
     constexpr int RB = D * 2, NCH = RB / 16, NS = D / 16;
@@ -732,16 +732,16 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void fa2_bf16_kernel(Fa16
     }
 }
 
-template <int D, int QT, int NW, int NSTG, int KT>
+template <int D, int QT, int NW, int NSTG, int KT, int OCC = (NW == 4 ? 2 : 1)>
 static int launch_fa16_cfg(grl_ctx* c, const Fa16Args& f, bool rope_q) {
     const int qb = 32 * QT * NW;
     dim3 grid((unsigned)(((f.S + qb - 1) / qb) * f.H * f.B)), block(NW * 64);
     if (f.mask) {
-        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, true, KT>), grid, block, 0, c->stream, f);
-        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, true, KT>), grid, block, 0, c->stream, f);
+        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
     } else {
-        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, false, KT>), grid, block, 0, c->stream, f);
-        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, false, KT>), grid, block, 0, c->stream, f);
+        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
     }
     GRL_CHECK_LAUNCH();
     return GRL_OK;
@@ -761,15 +761,18 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, bool rope_q) {
     // GRL_FA_CFG forces a configuration, for tuning runs:
     //   1: 8 waves, 64-key tiles, deep ring   2: 8 waves, 128-key tiles   3: 4 waves, 64-key tiles, 4 stages
     //   4: 4 waves, 128-key tiles, half-size ring (two workgroups per CU)
+    //   5: 4 waves, 64-key tiles, two stages, three workgroups per CU (head dims up to 64)
     static const int forced = [] { const char* e = getenv("GRL_FA_CFG"); return e ? atoi(e) : 0; }();
-    // short sequences: two small workgroups per CU hide each other's start-up and store tails;
-    // long ones: one 8-wave workgroup with the full ring
-    int cfg = forced >= 1 && forced <= 4 ? forced : (a.S > 1024 ? 2 : (a.S > 128 ? 4 : 3));
+    // short sequences are bound by per-workgroup latency (first-tile wait, output stores): two or, where the
+    // registers allow it (head dims up to 64), three small workgroups per CU hide each other's; long ones: one
+    // 8-wave workgroup with the full ring
+    int cfg = forced >= 1 && forced <= 5 ? forced : (a.S > 1024 ? 2 : (D <= 64 ? 5 : (a.S > 128 ? 4 : 3)));
     constexpr int DEEP = D == 128 ? 4 : 8;        // 128 KiB of K/V tiles: D=128 -> 4 x 32 KiB, else 8 x 16 (8) KiB
     switch (cfg) {
         case 1: return launch_fa16_cfg<D, 1, 8, DEEP, 64>(c, f, rope_q);
         case 2: return launch_fa16_cfg<D, 1, 8, DEEP / 2, 128>(c, f, rope_q);
         case 4: return launch_fa16_cfg<D, 1, 4, 2, (D == 128 ? 64 : 128)>(c, f, rope_q);
+        case 5: if constexpr (D <= 64) return launch_fa16_cfg<D, 1, 4, 2, 64, 3>(c, f, rope_q); else break;
         default: break;
     }
     return launch_fa16_cfg<D, 1, 4, 4, 64>(c, f, rope_q);
