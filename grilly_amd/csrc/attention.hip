@@ -464,26 +464,38 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     // lane -> (row, slot) inside one 1 KiB transfer; the slot holds chunk slot ^ swizzle(row)
     const int t_row = lane / NCH, t_slot = lane % NCH;
 
-    auto issue = [&](int kt) {
-        const int st = kt % NSTG, k0 = kt * KT;
+    // Transfer addresses: the per-lane part (row inside the transfer x row stride + swizzled chunk) does not
+    // change from tile to tile and has KVAR variants for K (the swizzle looks at row bits the transfer index
+    // supplies) and one for V; the tile and transfer index are wave-uniform and travel in the scalar offset.
+    constexpr int TPW = 2 * TPO / NW;
+    constexpr int KVAR = NCH >= 16 ? 4 : (NCH == 8 ? 2 : 1);
+    static_assert(TPW % KVAR == 0 && TPO % KVAR == 0 && (RPI * KVAR) % 16 == 0, "swizzle period must divide the transfer split");
+    int voffK[KVAR];
 #pragma unroll
-        for (int j = 0; j < 2 * TPO / NW; ++j) {
-            const int g = wave * (2 * TPO / NW) + j;                 // transfer id within the tile: K first, then V
-            const bool isv = g >= TPO;
-            const int inst = isv ? g - TPO : g;
-            const int row = inst * RPI + t_row;
-            const int chunk = t_slot ^ (isv ? lds_swz_v<NCH>(row) : lds_swz<NCH>(row));
-            const int rowg = k0 + row;
-            if (isv) dma16(rsV, lds + OFF_V + st * TILE + inst * 1024, rowg * vstride_b + chunk * 16);
-            else dma16(rsK, lds + st * TILE + inst * 1024, rowg * kstride_b + chunk * 16);
+    for (int i = 0; i < KVAR; ++i) voffK[i] = t_row * kstride_b + ((t_slot ^ lds_swz<NCH>(i * RPI + t_row)) << 4);
+    const int voffV = t_row * vstride_b + ((t_slot ^ lds_swz_v<NCH>(t_row)) << 4);
+    // wave v's share of the K / V transfers of tile kt (v is wave-uniform)
+    auto issue_share = [&](int kt, int v) {
+        const int st = kt % NSTG, k0 = kt * KT;
+        const bool isv = v * TPW >= TPO;                             // K transfers first, then V: a share is all K or all V
+        static_assert(TPO % TPW == 0, "a wave's share does not straddle K and V");
+        const int inst0 = v * TPW - (isv ? TPO : 0);
+#pragma unroll
+        for (int j = 0; j < TPW; ++j) {
+            const int inst = inst0 + j;
+            const int rowg = k0 + inst * RPI;
+            if (isv) dma16s(rsV, lds + OFF_V + st * TILE + inst * 1024, voffV, rowg * vstride_b);
+            else dma16s(rsK, lds + st * TILE + inst * 1024, voffK[j % KVAR], rowg * kstride_b);
         }
-        // raw mask values of the tile's 64 keys (256 B; the transfer unit is 1 KiB per wave, lanes
-        // past the tile read further mask entries or out of range, which nobody uses).  Every wave
-        // issues it so that all waves count the same number of transfers per tile.
-        if (HAS_MASK)
-            dma16(rsM, lds + OFF_M + st * 1024, (k0 + lane * 4) * 4);
     };
-
+    // raw mask values of the tile's keys (the transfer unit is 1 KiB per wave, lanes past the tile read
+    // further mask entries or out of range, which nobody uses)
+    auto issue_mask = [&](int kt) {
+        if (HAS_MASK) dma16(rsM, lds + OFF_M + (kt % NSTG) * 1024, (kt * KT + lane * 4) * 4);
+    };
+    // every wave requests its own share (and a mask row, so that all waves count the same number of
+    // transfers per tile)
+    auto issue = [&](int kt) { issue_share(kt, wave); issue_mask(kt); };
     // lacc: row sums of P, accumulated by the matrix core against an all-ones operand (every
     // register of a lane then holds the full sum for that lane's query); only register 0 is kept exact
     f32x16 oacc[QT][DT], lacc[QT];
@@ -708,7 +720,9 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
         // barrier without a memory fence (a fence would wait for every transfer in flight): LDS
         // writes of this wave are drained by lgkmcnt(0), its tile transfers by the wait above
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        if (kt + NSTG - 1 < nkt) issue(kt + NSTG - 1);   // into the stage tile kt-1 has just left
+        // into the stage tile kt-1 has just left.  (Letting only one wave of each SIMD pair request the tile, as
+        // the GEMM does, was measured here too: no gain.)
+        if (kt + NSTG - 1 < nkt) issue(kt + NSTG - 1);
         zero_tail(kt);
         if (skip_tile(kt)) continue;
         phase_S(kt);

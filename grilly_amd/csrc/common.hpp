@@ -137,6 +137,13 @@ template <int NCH> __device__ __forceinline__ int lds_swz_v(int r) {
     else return (r & 3) << 2;
 }
 
+// the same with a wave-uniform byte offset in a scalar register (address = base + voff + soff)
+__device__ __forceinline__ void dma16s(rsrc_words rs, const void* lds_dst_wave_uniform, int voff, int soff) {
+    const uint32_t la = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)lds_dst_wave_uniform);
+    const int so = __builtin_amdgcn_readfirstlane(soff);
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(la), "v"(voff), "s"(rs), "s"(so) : "memory");
+}
+
 template <typename T> struct elem;
 template <> struct elem<float> {
     static __device__ __forceinline__ float ld(const float* p) { return *p; }
