@@ -115,6 +115,19 @@ def side_workload(backend, mode, seed, reps):
     from grilly_amd import _lib as L
     c, lib, code = backend.core, backend.core.lib, L.GRL_BF16
     rng = np.random.default_rng(seed)
+    if mode == "prenorm_forward":
+        from grilly_amd import PreNormEncoder, PreNormEncoderConfig, random_prenorm_weights
+        cfg = PreNormEncoderConfig()            # ModernBERT-base shape: 22 layers, d 768, 12 heads, GeGLU halves of 1152
+        B, S = 128, 512
+        enc = PreNormEncoder(backend, cfg, random_prenorm_weights(cfg, seed=seed), dtype="bf16")
+        enc.set_inputs(rng.integers(0, cfg.vocab, (B, S)), None)
+        ms = time_launches(c, enc.launch, max(reps // 4, 3), warm=2)
+        M, d, ff = B * S, cfg.d_model, cfg.d_ff
+        flops = cfg.layers * (2.0 * M * d * 3 * d + 2.0 * M * d * d + 3 * 2.0 * M * d * ff + 4.0 * B * cfg.heads * S * S * cfg.head_dim)
+        return {"mode": mode, "workload": "pre-norm / rotary / GeGLU encoder forward, ModernBERT-base shape (22 layers, d 768, 12x64 heads, "
+                "GeGLU 2x1152), batch 128 x seq 512, bf16, random weights, first-token pooling",
+                "ms": round(ms, 3), "tokens_per_s": round(M / ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 1),
+                "frac_mfma": round(flops / (ms * 1e-3) / PEAK_BF16, 4), "flops": flops}
     if mode == "fa2_long":
         B, H, S, D = 4, 32, 8192, 128
         n = B * S * H * D
@@ -174,12 +187,13 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
-    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "kernels", "copy", "fa2_long", "swiglu_mlp"],
+    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "kernels", "copy", "fa2_long", "swiglu_mlp", "prenorm_forward"],
                     help="forward: the benchmark; gemm / copy: only launch the dominant GEMM kernel at its three "
                          "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs); kernels: every kernel of "
                          "the layer at its layer shape, nothing else (counter runs); fa2_long: "
                          "causal attention with RoPE at batch 4, 32 heads, seq 8192, head dim 128, bf16; swiglu_mlp: "
-                         "X[16384,4096] through gate/up [11008,4096] + silu*up + down [4096,11008], bf16")
+                         "X[16384,4096] through gate/up [11008,4096] + silu*up + down [4096,11008], bf16; prenorm_forward: the "
+                         "pre-norm / rotary / GeGLU encoder at the ModernBERT-base shape, batch 128 x seq 512, bf16")
     ap.add_argument("--cpu-sequences", type=int, default=12)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -203,7 +217,7 @@ def main():
                           "ms": round(ms, 4), "gbps": round(2 * nbytes / ms / 1e6, 1), "launches": a.kernel_reps + WARM}))
         backend.cleanup()
         return
-    if a.mode in ("fa2_long", "swiglu_mlp"):
+    if a.mode in ("fa2_long", "swiglu_mlp", "prenorm_forward"):
         print(json.dumps(side_workload(backend, a.mode, seed, a.kernel_reps)))
         backend.cleanup()
         return

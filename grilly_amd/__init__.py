@@ -10,7 +10,9 @@ work is done by hand-written HIP kernels in grilly_amd/lib/libgrilly_hip.so.  `g
 holds forward-only Module adapters (Linear, LayerNorm, FlashAttention2, TransformerEncoderLayer ...).
 """
 from .backend.compute import HipCompute, Compute
-from .encoder import BertEncoder, EncoderConfig, random_bert_weights
+from .encoder import (BertEncoder, EncoderConfig, PreNormEncoder, PreNormEncoderConfig, random_bert_weights,
+                      random_prenorm_weights)
 
-__all__ = ["Compute", "HipCompute", "BertEncoder", "EncoderConfig", "random_bert_weights"]
+__all__ = ["Compute", "HipCompute", "BertEncoder", "EncoderConfig", "random_bert_weights",
+           "PreNormEncoder", "PreNormEncoderConfig", "random_prenorm_weights"]
 __version__ = "0.1.0"

@@ -1,5 +1,6 @@
-"""Weights of a BERT- or DistilBERT-style post-LN encoder from a local Hugging Face /
-sentence-transformers checkpoint directory, in the layout grilly_amd.BertEncoder takes.
+"""Weights of a BERT- or DistilBERT-style post-LN encoder (-> grilly_amd.BertEncoder) or of a
+ModernBERT-style pre-norm one (-> grilly_amd.PreNormEncoder) from a local Hugging Face /
+sentence-transformers checkpoint directory.
 
 The reference pulls the same tensors out of a live torch model
 (utils/vulkan_sentence_transformer.py:262-542 `_extract_layer_weights`, :563-708 embeddings); here
@@ -12,14 +13,17 @@ they are read straight from the files, offline, with loaders that execute nothin
 Names follow PyTorch's (out_features, in_features) weight layout, which is also the reference's and
 this library's, so nothing is transposed; the three attention projections are stacked into the packed
 [Wq;Wk;Wv] of the fused QKV projection.  The activation is the reference's tanh GELU whatever
-`hidden_act` says (its shaders have no erf GELU).
+`hidden_act` says (its shaders have no erf GELU).  A ModernBERT checkpoint (tok_embeddings, Wqkv, Wi / Wo)
+gives a PreNormEncoderConfig; as in the reference (:307-330, :426-452, :512-520) Wqkv stays packed as
+[Wq;Wk;Wv], the first half of Wi is the half that goes through GELU, absent biases become zeros, and the
+per-layer attn_norm is not used (the reference's forward skips it, :804-806).
 """
 import json
 import os
 
 import numpy as np
 
-from .encoder import EncoderConfig
+from .encoder import EncoderConfig, PreNormEncoderConfig
 
 
 def _find_dir(path):
@@ -53,6 +57,8 @@ def load_encoder_checkpoint(path):
     with open(os.path.join(d, "config.json")) as f:
         hf = json.load(f)
     T = _load_tensors(d)
+    if any(k.endswith("embeddings.tok_embeddings.weight") for k in T):
+        return _load_prenorm(hf, T)
     anchor = [k for k in T if k.endswith("embeddings.word_embeddings.weight")]
     if not anchor:
         raise ValueError("checkpoint has no embeddings.word_embeddings.weight: not a BERT / DistilBERT encoder")
@@ -103,6 +109,47 @@ def load_encoder_checkpoint(path):
               "w_ff2": get(names["ff2"] + ".weight"), "b_ff2": get(names["ff2"] + ".bias"),
               "ln2_g": get(names["ln2"] + ".weight"), "ln2_b": get(names["ln2"] + ".bias")}
         want = {"w_qkv": (3 * dm, dm), "w_o": (dm, dm), "w_ff1": (ff, dm), "w_ff2": (dm, ff)}
+        for k, shp in want.items():
+            if lw[k].shape != shp:
+                raise ValueError(f"layer {i}: {k} has shape {lw[k].shape}, config says {shp}")
+        w["layers"].append(lw)
+    return cfg, w
+
+
+def _load_prenorm(hf, T):
+    """ModernBERT names -> (PreNormEncoderConfig, weights for PreNormEncoder)."""
+    anchor = [k for k in T if k.endswith("embeddings.tok_embeddings.weight")][0]
+    prefix = anchor[: -len("embeddings.tok_embeddings.weight")]
+    dm, ff, L_ = hf["hidden_size"], hf["intermediate_size"], hf["num_hidden_layers"]
+
+    def get(name, zeros=None):
+        if prefix + name in T:
+            return _f32(T[prefix + name])
+        if zeros is not None:
+            return np.zeros(zeros, np.float32)
+        raise ValueError(f"checkpoint lacks {prefix}{name}")
+
+    rope_base = hf.get("local_rope_theta") or hf.get("rope_theta") or 10000.0      # reference :830-833
+    scaling = hf.get("rope_scaling")
+    cfg = PreNormEncoderConfig(layers=L_, d_model=dm, heads=hf["num_attention_heads"], d_ff=ff, vocab=hf["vocab_size"],
+                               emb_eps=hf.get("norm_eps", 1e-5), final_eps=hf.get("norm_eps", 1e-5),
+                               rope_base=float(rope_base),
+                               rope_scaling=float(scaling.get("factor", 1.0)) if isinstance(scaling, dict) else 1.0)
+    tok = get("embeddings.tok_embeddings.weight")
+    if tok.shape != (cfg.vocab, dm):
+        raise ValueError(f"embedding shape {tok.shape} does not match config ({cfg.vocab}, {dm})")
+    w = {"tok_emb": tok, "emb_ln_g": get("embeddings.norm.weight"), "emb_ln_b": get("embeddings.norm.bias", dm),
+         "final_ln_g": get("final_norm.weight") if prefix + "final_norm.weight" in T else None,
+         "final_ln_b": get("final_norm.bias", dm), "layers": []}
+    for i in range(L_):
+        p = f"layers.{i}."
+        wi, bi = get(p + "mlp.Wi.weight"), get(p + "mlp.Wi.bias", 2 * ff)
+        lw = {"w_qkv": get(p + "attn.Wqkv.weight"), "b_qkv": get(p + "attn.Wqkv.bias", 3 * dm),
+              "w_o": get(p + "attn.Wo.weight"), "b_o": get(p + "attn.Wo.bias", dm),
+              "ffn_ln_g": get(p + "mlp_norm.weight"), "ffn_ln_b": get(p + "mlp_norm.bias", dm),
+              "w_ff_in": _f32(wi[:ff]), "b_ff_in": _f32(bi[:ff]), "w_ff_gate": _f32(wi[ff:]), "b_ff_gate": _f32(bi[ff:]),
+              "w_ff2": get(p + "mlp.Wo.weight"), "b_ff2": get(p + "mlp.Wo.bias", dm)}
+        want = {"w_qkv": (3 * dm, dm), "w_o": (dm, dm), "w_ff_in": (ff, dm), "w_ff_gate": (ff, dm), "w_ff2": (dm, ff)}
         for k, shp in want.items():
             if lw[k].shape != shp:
                 raise ValueError(f"layer {i}: {k} has shape {lw[k].shape}, config says {shp}")

@@ -137,7 +137,9 @@ template <int NCH> __device__ __forceinline__ int lds_swz_v(int r) {
     else return (r & 3) << 2;
 }
 
-// the same with a wave-uniform byte offset in a scalar register (address = base + voff + soff)
+// the same with a wave-uniform byte offset in a scalar register (address = base + voff + soff).
+// For these raw resources the range check is made on voff + soff (a transfer whose scalar part alone
+// passes num_records returns zeros: checked on the hardware), so rows past the tensor are never touched.
 __device__ __forceinline__ void dma16s(rsrc_words rs, const void* lds_dst_wave_uniform, int voff, int soff) {
     const uint32_t la = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)lds_dst_wave_uniform);
     const int so = __builtin_amdgcn_readfirstlane(soff);

@@ -540,14 +540,19 @@ __global__ __launch_bounds__(256) void embed_kernel(const int32_t* __restrict__ 
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // the host validates; this only keeps loads in bounds
     const int s = (int)(row % S);
     const float* t = tok + (int64_t)id * F;
-    const float* p = pos + (int64_t)s * F;
     T* o = x + row * (int64_t)F;
-    for (int f = lane; f < F; f += 64) elem<T>::st(o + f, t[f] + typ[f] + p[f]);
+    if (pos && typ) {
+        const float* p = pos + (int64_t)s * F;
+        for (int f = lane; f < F; f += 64) elem<T>::st(o + f, t[f] + typ[f] + p[f]);
+    } else {                                            // tables a model does not have (wave-uniform branch)
+        const float* p = pos ? pos + (int64_t)s * F : nullptr;
+        for (int f = lane; f < F; f += 64) elem<T>::st(o + f, t[f] + (typ ? typ[f] : 0.f) + (p ? p[f] : 0.f));
+    }
 }
 
 extern "C" int grl_embed(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F, int64_t vocab, const int32_t* ids,
                          const float* tok_emb, const float* pos_emb, const float* type_emb, void* x) {
-    GRL_REQUIRE(c && ids && tok_emb && pos_emb && type_emb && x, GRL_ERR_ARG, "grl_embed: null argument");
+    GRL_REQUIRE(c && ids && tok_emb && x, GRL_ERR_ARG, "grl_embed: null argument");
     GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_embed: bad dtype %d", dtype);
     GRL_REQUIRE(B >= 0 && S > 0 && F > 0 && vocab > 0 && S < (1LL << 31) && F < (1LL << 31) && vocab < (1LL << 31),
                 GRL_ERR_SHAPE, "grl_embed: bad shape");

@@ -1,4 +1,5 @@
-"""Device-resident BERT-style (post-LN) encoder forward built from the hot-path kernels.
+"""Device-resident encoder forwards built from the hot-path kernels: the BERT-style post-LN encoder
+(BertEncoder) and the pre-norm / rotary / GeGLU one (PreNormEncoder, further down).
 
 Mirrors the forward recipe of the reference's VulkanSentenceTransformer
 (utils/vulkan_sentence_transformer.py): embeddings = token + token-type 0 + position, then
@@ -154,3 +155,169 @@ class BertEncoder:
         M, d, ff = B * S, cfg.d_model, cfg.d_ff
         per_layer = 2 * M * d * 3 * d + 2 * M * d * d + 2 * 2 * M * d * ff + 4 * B * cfg.heads * S * S * cfg.head_dim
         return cfg.layers * per_layer
+
+
+# ------------------------------------------------------------------------------------------------
+@dataclass
+class PreNormEncoderConfig:
+    """ModernBERT-shaped encoder: token embeddings only, rotary positions, GeGLU MLP."""
+    layers: int = 22
+    d_model: int = 768
+    heads: int = 12
+    d_ff: int = 1152           # width of each GeGLU half (Wi is (2*d_ff, d_model))
+    vocab: int = 50368
+    eps: float = 1e-5          # the reference hard-codes 1e-5 for the layer norm in front of the MLP (:901)
+    emb_eps: float = 1e-5
+    final_eps: float = 1e-5
+    rope_base: float = 10000.0
+    rope_scaling: float = 1.0
+
+    @property
+    def head_dim(self):
+        return self.d_model // self.heads
+
+
+def random_prenorm_weights(cfg, seed=0, std=0.02):
+    """Random-init weights, (out_features, in_features) matrices ~N(0,std), biases 0, norms 1 / 0."""
+    rng = np.random.default_rng(seed)
+    d, ff = cfg.d_model, cfg.d_ff
+    n = lambda *s: (rng.standard_normal(s) * std).astype(np.float32)
+    one, zero = (lambda k: np.ones(k, np.float32)), (lambda k: np.zeros(k, np.float32))
+    w = {"tok_emb": n(cfg.vocab, d), "emb_ln_g": one(d), "emb_ln_b": zero(d),
+         "final_ln_g": one(d), "final_ln_b": zero(d), "layers": []}
+    for _ in range(cfg.layers):
+        w["layers"].append({
+            "w_qkv": n(3 * d, d), "b_qkv": zero(3 * d), "w_o": n(d, d), "b_o": zero(d),
+            "ffn_ln_g": one(d), "ffn_ln_b": zero(d),
+            "w_ff_in": n(ff, d), "b_ff_in": zero(ff), "w_ff_gate": n(ff, d), "b_ff_gate": zero(ff),
+            "w_ff2": n(d, ff), "b_ff2": zero(d)})
+    return w
+
+
+class PreNormEncoder:
+    """Device-resident forward of the reference's pre-norm branch
+    (utils/vulkan_sentence_transformer.py:799-970 per layer; encode :1146-1183 around it):
+
+        x = LN(tok_emb[ids]; emb)                                              (:1153-1155, :749-785)
+        per layer:  x += Wo.Attn(rope(Wq x), rope(Wk x), Wv x; key mask)       (:806-893, no norm in front)
+                    x += W2.(gelu(Wi_in.LN(x)) * (Wi_gate.LN(x)))              (:901-945)
+        x = LN(x; final)   (only if final_ln_g is given, :1166-1175)
+        pooled = x[:, 0, :] (first token), L2-normalised                       (:1179-1183, :1194-1201)
+
+    Built from the same entry points as the post-LN encoder: the projection GEMMs, attention with the
+    rotate-half rotation fused, LayerNorm, the dual GEMM with the GELU gate and the elementwise add.
+    The packed Wqkv is read through three row blocks (no split copy).  The +-50 / +-1e6 clips the
+    reference puts around the gate (:924-930) are not applied: they only act beyond those magnitudes."""
+
+    _MATS = ("w_qkv", "w_o", "w_ff_in", "w_ff_gate", "w_ff2")
+    _VECS = ("b_qkv", "b_o", "ffn_ln_g", "ffn_ln_b", "b_ff_in", "b_ff_gate", "b_ff2")
+
+    def __init__(self, core, cfg, weights, dtype="fp32"):
+        self.core = core.core if hasattr(core, "core") else core
+        if not isinstance(self.core, HipCore):
+            raise TypeError("PreNormEncoder needs a Compute() backend or its HipCore")
+        if cfg.head_dim not in (32, 64, 128) or cfg.head_dim * cfg.heads != cfg.d_model:
+            raise ValueError("d_model must be heads*head_dim with head_dim 32, 64 or 128")
+        self.cfg, self.dtype, self.code = cfg, dtype, dtype_code(dtype)
+        c = self.core
+        self._keep = []
+        up = lambda a, code=L.GRL_F32: self._own(c.upload(a, code))
+        vec = lambda a: up(np.asarray(a, np.float32).reshape(-1))
+        self.tok = up(weights["tok_emb"])
+        self.emb_g, self.emb_b = vec(weights["emb_ln_g"]), vec(weights["emb_ln_b"])
+        self.final = None
+        if weights.get("final_ln_g") is not None:
+            self.final = (vec(weights["final_ln_g"]), vec(weights["final_ln_b"]))
+        self.layers = []
+        for lw in weights["layers"]:
+            entry = {k: up(lw[k], self.code) for k in self._MATS}
+            entry.update({k: vec(lw[k]) for k in self._VECS})
+            self.layers.append(entry)
+        self._shape = None
+
+    def _own(self, buf):
+        self._keep.append(buf)
+        return buf
+
+    def prepare(self, B, S):
+        if self._shape == (B, S):
+            return
+        self.release_activations()
+        cfg, c = self.cfg, self.core
+        es = 2 if self.code == L.GRL_BF16 else 4
+        act = B * S * cfg.d_model * es
+        self.x, self.q, self.k, self.v, self.att, self.t = (c.alloc(act) for _ in range(6))
+        self.h = c.alloc(B * S * cfg.d_ff * es)
+        self.ids = c.alloc(B * S * 4)
+        self.mask = c.alloc(B * S * 4)
+        first = np.zeros((B, S), np.float32)
+        first[:, 0] = 1.0                              # "mean" over the first token only = that token
+        self.first = c.upload_raw(first)
+        self.pooled = c.alloc(B * cfg.d_model * 4)
+        self._shape = (B, S)
+
+    def release_activations(self):
+        if self._shape is not None:
+            for b in (self.x, self.q, self.k, self.v, self.att, self.t, self.h, self.ids, self.mask, self.first, self.pooled):
+                b.free()
+            self._shape = None
+
+    def set_inputs(self, input_ids, attention_mask=None):
+        ids = np.ascontiguousarray(input_ids, dtype=np.int32)
+        if ids.ndim != 2 or ids.shape[1] == 0:
+            raise ValueError("input_ids must be (batch, seq_len) with seq_len > 0")
+        if ids.size and (ids.min() < 0 or ids.max() >= self.cfg.vocab):
+            raise IndexError("token id out of range")
+        B, S = ids.shape
+        self.prepare(B, S)
+        c = self.core
+        L.check(c.lib.grl_h2d(c.ctx, self.ids.ptr, ids.ctypes.data, ids.nbytes), "upload ids")
+        self.has_mask = attention_mask is not None
+        if self.has_mask:
+            m = np.ascontiguousarray(attention_mask, dtype=np.float32)
+            if m.shape != (B, S):
+                raise ValueError("attention_mask must be (batch, seq_len)")
+            L.check(c.lib.grl_h2d(c.ctx, self.mask.ptr, m.ctypes.data, m.nbytes), "upload mask")
+
+    def launch(self, pool=True):
+        """Enqueue one full forward on the context stream (no host synchronisation)."""
+        B, S = self._shape
+        cfg, c, lib, code = self.cfg, self.core, self.core.lib, self.code
+        M, d, ff, H, D = B * S, cfg.d_model, cfg.d_ff, cfg.heads, cfg.head_dim
+        es = 2 if code == L.GRL_BF16 else 4
+        mask = self.mask.ptr if self.has_mask else None
+        L.check(lib.grl_embed(c.ctx, code, B, S, d, cfg.vocab, self.ids.ptr, self.tok.ptr, None, None, self.x.ptr), "embed")
+        L.check(lib.grl_layernorm(c.ctx, code, M, d, self.x.ptr, None, self.emb_g.ptr, self.emb_b.ptr, cfg.emb_eps,
+                                  self.x.ptr), "embedding layernorm")
+        for w in self.layers:
+            for i, dst in enumerate((self.q, self.k, self.v)):       # row blocks of the packed weight and bias
+                L.check(lib.grl_gemm_nt(c.ctx, code, code, M, d, d, self.x.ptr, w["w_qkv"].ptr + i * d * d * es,
+                                        w["b_qkv"].ptr + i * d * 4, dst.ptr, L.EPI_NONE), "q/k/v projection")
+            L.check(lib.grl_fa2_fwd(c.ctx, code, B, S, H, D, self.q.ptr, self.k.ptr, self.v.ptr, mask, self.att.ptr,
+                                    1.0 / float(np.sqrt(D)), 0, L.ROPE_HALF, cfg.rope_base, cfg.rope_scaling, None),
+                    "attention")
+            L.check(lib.grl_gemm_nt(c.ctx, code, code, M, d, d, self.att.ptr, w["w_o"].ptr, w["b_o"].ptr, self.t.ptr,
+                                    L.EPI_NONE), "output projection")
+            L.check(lib.grl_add(c.ctx, code, M * d, self.x.ptr, self.t.ptr, self.x.ptr), "residual")
+            L.check(lib.grl_layernorm(c.ctx, code, M, d, self.x.ptr, None, w["ffn_ln_g"].ptr, w["ffn_ln_b"].ptr, cfg.eps,
+                                      self.t.ptr), "mlp layernorm")
+            # the dual GEMM activates its second ("up") operand: that is the first half of Wi here
+            L.check(lib.grl_glu_nt(c.ctx, code, code, M, ff, d, self.t.ptr, w["w_ff_gate"].ptr, w["w_ff_in"].ptr,
+                                   w["b_ff_gate"].ptr, w["b_ff_in"].ptr, self.h.ptr, None, None, L.EPI_GELU), "geglu")
+            L.check(lib.grl_gemm_nt(c.ctx, code, code, M, d, ff, self.h.ptr, w["w_ff2"].ptr, w["b_ff2"].ptr, self.t.ptr,
+                                    L.EPI_NONE), "mlp output")
+            L.check(lib.grl_add(c.ctx, code, M * d, self.x.ptr, self.t.ptr, self.x.ptr), "residual")
+        if self.final is not None:
+            L.check(lib.grl_layernorm(c.ctx, code, M, d, self.x.ptr, None, self.final[0].ptr, self.final[1].ptr,
+                                      cfg.final_eps, self.x.ptr), "final layernorm")
+        if pool:
+            L.check(lib.grl_mean_pool(c.ctx, code, B, S, d, self.x.ptr, self.first.ptr, self.pooled.ptr, 1), "first-token pool")
+
+    def forward(self, input_ids, attention_mask=None, pool=True):
+        """pool=True -> L2-normalised first-token embeddings (B, d); False -> hidden states (B,S,d)."""
+        self.set_inputs(input_ids, attention_mask)
+        self.launch(pool)
+        B, S = self._shape
+        if pool:
+            return self.core.download(self.pooled, (B, self.cfg.d_model))
+        return self.core.download(self.x, (B, S, self.cfg.d_model), self.code)

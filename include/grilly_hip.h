@@ -205,6 +205,8 @@ int grl_swiglu_act(grl_ctx* ctx, int dtype, int64_t rows, int64_t h, const void*
 
 /* ---- encoder pre/post steps ------------------------------------------------------------
  * x[b,s,:] = tok_emb[ids[b,s]] + pos_emb[s] + type_emb[0]   (tables fp32, x of `dtype`).
+ * pos_emb and type_emb may each be NULL (a model without that table: the rotary-position
+ * branch of encode adds neither, utils/vulkan_sentence_transformer.py:1148-1155).
  * Replaces the embedding steps of VulkanSentenceTransformer
  * (utils/vulkan_sentence_transformer.py:563-707). */
 int grl_embed(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t F, int64_t vocab,

@@ -246,6 +246,26 @@ def truth_bert_layer(x, w, mask, H, eps=1e-5, quant=None):
     return qf(truth_layernorm(x1, w["ln2_g"], w["ln2_b"], eps, residual=ff2))
 
 
+def truth_prenorm_geglu_layer(x, w, mask, H, eps=1e-5, rope_base=10000.0, rope_scaling=1.0, quant=None):
+    """Pre-norm layer with rotary positions and a GeGLU MLP, utils/vulkan_sentence_transformer.py:799-970:
+    x += Wo.Attn(rope(Wq x), rope(Wk x), Wv x; key mask) (:806-893, no norm in front of the attention:
+    the reference skips attn_norm in every layer); x += W2.(gelu(Wi_in.LN(x)) * (Wi_gate.LN(x))) (:901-945),
+    rotate-half RoPE on positions 0..S-1 (:829-846, backend/attention.py:795-835), tanh GELU (:933).
+    The +-50 / +-1e6 clips of :924-930 are left out (no effect below those magnitudes)."""
+    qf = (lambda a: a) if quant is None else (lambda a: quant(np.asarray(a, np.float32)).astype(np.float64))
+    x = np.asarray(x, np.float64)
+    B, S, d = x.shape
+    D = d // H
+    q, k, v = (qf(truth_linear(x, w["w_qkv"][i * d:(i + 1) * d], w["b_qkv"][i * d:(i + 1) * d])).reshape(B, S, H, D)
+               for i in range(3))
+    a = qf(truth_attention(q, k, v, mask=mask, rope="half", base=rope_base, scaling=rope_scaling)).reshape(B, S, d)
+    x = qf(x + qf(truth_linear(a, w["w_o"], w["b_o"])))
+    xn = qf(truth_layernorm(x, w["ffn_ln_g"], w["ffn_ln_b"], eps))
+    # truth_fused_glu activates its "up" operand: that is the first half of Wi here
+    h = qf(truth_fused_glu(xn, w["w_ff_gate"], w["w_ff_in"], w["b_ff_gate"], w["b_ff_in"], act="gelu")[0])
+    return qf(x + qf(truth_linear(h, w["w_ff2"], w["b_ff2"])))
+
+
 # ---------------------------------------------------------------- error metrics
 def max_rel(y, ref):
     """max|y-ref| / max|ref|: the scale-relative error the tolerances (1e-4 fp32, 2e-2 bf16) use."""

@@ -135,3 +135,39 @@ def test_imported_checkpoint_runs_like_the_oracle(tmp_path, backend, corc):
     for lw in w["layers"]:
         x = corc.bert_layer(x, lw, mask, cfg.heads, cfg.eps)
     assert O.max_rel(pooled, corc.mean_pool(x, mask)) < 1e-4
+
+
+def test_modernbert_names(tmp_path):
+    """tok_embeddings / Wqkv / Wi-Wo names give the pre-norm configuration; Wi is split first half =
+    activated half, missing biases become zeros, rope base comes from local_rope_theta."""
+    from safetensors.numpy import save_file
+    from grilly_amd.encoder import PreNormEncoderConfig, random_prenorm_weights
+    cfg = PreNormEncoderConfig(layers=2, d_model=64, heads=2, d_ff=48, vocab=90)
+    w = random_prenorm_weights(cfg, seed=4)
+    sd = {"model.embeddings.tok_embeddings.weight": w["tok_emb"], "model.embeddings.norm.weight": w["emb_ln_g"],
+          "model.final_norm.weight": w["final_ln_g"]}
+    for i, lw in enumerate(w["layers"]):
+        p = f"model.layers.{i}."
+        sd[p + "attn.Wqkv.weight"], sd[p + "attn.Wo.weight"] = lw["w_qkv"], lw["w_o"]
+        sd[p + "mlp.Wi.weight"] = np.concatenate([lw["w_ff_in"], lw["w_ff_gate"]], 0)
+        sd[p + "mlp.Wo.weight"], sd[p + "mlp_norm.weight"] = lw["w_ff2"], lw["ffn_ln_g"]
+        if i > 0:
+            sd[p + "attn_norm.weight"] = np.ones(64, np.float32)        # present in real files, unused by the recipe
+    save_file({k: np.ascontiguousarray(v) for k, v in sd.items()}, str(tmp_path / "model.safetensors"))
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump({"num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 2, "intermediate_size": 48,
+                   "vocab_size": 90, "local_rope_theta": 160000.0, "global_rope_theta": 10000.0, "norm_eps": 1e-5}, f)
+    got_cfg, got = load_encoder_checkpoint(str(tmp_path))
+    assert isinstance(got_cfg, PreNormEncoderConfig)
+    assert (got_cfg.layers, got_cfg.d_model, got_cfg.heads, got_cfg.d_ff, got_cfg.vocab) == (2, 64, 2, 48, 90)
+    assert got_cfg.rope_base == 160000.0 and got_cfg.rope_scaling == 1.0
+    np.testing.assert_array_equal(got["tok_emb"], w["tok_emb"])
+    for la, lb in zip(got["layers"], w["layers"]):
+        assert set(la) == set(lb)
+        for k in la:
+            np.testing.assert_array_equal(la[k], lb[k])           # biases: zeros on both sides
+    # a wrong Wi height is reported with the layer and the name
+    sd["model.layers.1.mlp.Wi.weight"] = sd["model.layers.1.mlp.Wi.weight"][:-2]
+    save_file({k: np.ascontiguousarray(v) for k, v in sd.items()}, str(tmp_path / "model.safetensors"))
+    with pytest.raises(ValueError, match="layer 1: w_ff_gate"):
+        load_encoder_checkpoint(str(tmp_path))

@@ -1,0 +1,82 @@
+"""Pre-norm / rotary / GeGLU encoder forward (the reference's ModernBERT branch,
+utils/vulkan_sentence_transformer.py:799-970 and encode :1146-1201) against the float64 oracle
+composed from the pinned pieces (linear, rotate-half RoPE, attention, LayerNorm, GELU-gated GLU)."""
+import numpy as np
+import pytest
+
+from oracle import oracle_np as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _truth_forward(cfg, w, ids, mask, quant=None):
+    qf = (lambda a: a) if quant is None else (lambda a: quant(np.asarray(a, np.float32)).astype(np.float64))
+    x = qf(w["tok_emb"][ids].astype(np.float64))
+    x = qf(O.truth_layernorm(x, w["emb_ln_g"], w["emb_ln_b"], cfg.emb_eps))
+    for lw in w["layers"]:
+        lq = dict(lw)
+        if quant is not None:
+            for k in ("w_qkv", "w_o", "w_ff_in", "w_ff_gate", "w_ff2"):
+                lq[k] = quant(lw[k])
+        x = O.truth_prenorm_geglu_layer(x, lq, mask, cfg.heads, cfg.eps, cfg.rope_base, cfg.rope_scaling, quant)
+    if w.get("final_ln_g") is not None:
+        x = qf(O.truth_layernorm(x, w["final_ln_g"], w["final_ln_b"], cfg.final_eps))
+    cls = x[:, 0, :]
+    return x, cls / np.maximum(np.linalg.norm(cls, axis=-1, keepdims=True), 1e-12)
+
+
+def _case(seed, layers=2, d=128, heads=4, ff=192, vocab=300, B=3, S=40, std=0.08):
+    from grilly_amd.encoder import PreNormEncoderConfig, random_prenorm_weights
+    cfg = PreNormEncoderConfig(layers=layers, d_model=d, heads=heads, d_ff=ff, vocab=vocab, rope_base=160000.0)
+    w = random_prenorm_weights(cfg, seed=seed, std=std)
+    rng = np.random.default_rng(seed + 1)
+    for lw in w["layers"]:                      # non-trivial biases and norm parameters
+        for k in ("b_qkv", "b_o", "b_ff_in", "b_ff_gate", "b_ff2", "ffn_ln_b"):
+            lw[k] = (rng.standard_normal(lw[k].shape) * 0.05).astype(np.float32)
+        lw["ffn_ln_g"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    w["emb_ln_g"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    w["final_ln_b"] = (0.05 * rng.standard_normal(d)).astype(np.float32)
+    ids = rng.integers(0, vocab, (B, S))
+    lens = rng.integers(S // 3, S + 1, B)
+    mask = (np.arange(S)[None, :] < lens[:, None]).astype(np.float32)
+    return cfg, w, ids, mask
+
+
+@pytest.mark.parametrize("dtype,tol", [("fp32", 1e-4), ("bf16", 2e-2)])
+def test_prenorm_encoder_matches_oracle(backend, dtype, tol):
+    from grilly_amd.encoder import PreNormEncoder
+    cfg, w, ids, mask = _case(11)
+    enc = PreNormEncoder(backend, cfg, w, dtype=dtype)
+    hidden = enc.forward(ids, mask, pool=False)
+    pooled = enc.forward(ids, mask, pool=True)
+    ref_h, ref_p = _truth_forward(cfg, w, ids, mask, O.bf16_round if dtype == "bf16" else None)
+    keep = mask.astype(bool)                    # padded positions carry no contract
+    assert O.max_rel(hidden[keep], ref_h[keep]) <= tol
+    assert O.max_rel(pooled, ref_p) <= tol
+    np.testing.assert_allclose(np.linalg.norm(pooled, axis=-1), 1.0, atol=1e-5)
+
+
+def test_prenorm_encoder_without_mask_head_dim_64_no_final_norm(backend):
+    from grilly_amd.encoder import PreNormEncoder
+    cfg, w, ids, _ = _case(5, layers=1, d=128, heads=2, ff=128, B=2, S=33)
+    w["final_ln_g"] = None
+    enc = PreNormEncoder(backend, cfg, w, dtype="fp32")
+    hidden = enc.forward(ids, None, pool=False)
+    ref_h, _ = _truth_forward(cfg, w, ids, None)
+    assert O.max_rel(hidden, ref_h) <= 1e-4
+    # a second shape on the same object re-plans its buffers
+    ids2 = ids[:1, :17]
+    h2 = enc.forward(ids2, None, pool=False)
+    assert O.max_rel(h2, _truth_forward(cfg, w, ids2, None)[0]) <= 1e-4
+
+
+def test_prenorm_encoder_rejects_bad_inputs(backend):
+    from grilly_amd.encoder import PreNormEncoder
+    cfg, w, ids, mask = _case(3, layers=1)
+    enc = PreNormEncoder(backend, cfg, w)
+    with pytest.raises(IndexError):
+        enc.forward(np.full((2, 8), cfg.vocab), None)
+    with pytest.raises(ValueError):
+        enc.forward(ids, mask[:, :-1])
+    with pytest.raises(ValueError):
+        enc.forward(ids[0], None)

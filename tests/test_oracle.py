@@ -301,3 +301,44 @@ def test_bf16_rounding_helpers():
         np.testing.assert_array_equal(t, r[:5])
     except ImportError:
         pass
+
+
+def test_prenorm_geglu_layer_structure():
+    """What the composition must satisfy whatever the weights (utils/vulkan_sentence_transformer.py:799-970):
+    both sub-blocks are residual (zero output projections leave x untouched), the FIRST half of Wi is the
+    one that goes through GELU (:919-933), and the attention sees rotated Q,K (a constant shift of all
+    positions changes nothing, an unrotated score would not care either, so the check is against the
+    un-rotated attention being different)."""
+    rng = np.random.default_rng(7)
+    B, S, H, d, ff = 2, 9, 2, 64, 48
+    n = lambda *s: rng.standard_normal(s) * 0.2
+    w = {"w_qkv": n(3 * d, d), "b_qkv": n(3 * d), "w_o": n(d, d), "b_o": n(d), "ffn_ln_g": 1 + n(d), "ffn_ln_b": n(d),
+         "w_ff_in": n(ff, d), "b_ff_in": n(ff), "w_ff_gate": n(ff, d), "b_ff_gate": n(ff), "w_ff2": n(d, ff), "b_ff2": n(d)}
+    x = n(B, S, d)
+    mask = np.ones((B, S), np.float32); mask[1, 6:] = 0
+    full = O.truth_prenorm_geglu_layer(x, w, mask, H)
+    # residual structure
+    w0 = dict(w, w_o=np.zeros((d, d)), b_o=np.zeros(d), w_ff2=np.zeros((d, ff)), b_ff2=np.zeros(d))
+    np.testing.assert_allclose(O.truth_prenorm_geglu_layer(x, w0, mask, H), x, atol=1e-12)
+    # MLP alone, written out from the reference's formula
+    wa = dict(w, w_o=np.zeros((d, d)), b_o=np.zeros(d))
+    xn = (x - x.mean(-1, keepdims=True)) / np.sqrt(x.var(-1, keepdims=True) + 1e-5) * w["ffn_ln_g"] + w["ffn_ln_b"]
+    a = xn @ w["w_ff_in"].T + w["b_ff_in"]
+    g = xn @ w["w_ff_gate"].T + w["b_ff_gate"]
+    act = 0.5 * a * (1 + np.tanh(np.sqrt(2 / np.pi) * (a + 0.044715 * a ** 3)))
+    np.testing.assert_allclose(O.truth_prenorm_geglu_layer(x, wa, mask, H), x + (act * g) @ w["w_ff2"].T + w["b_ff2"], rtol=1e-9, atol=1e-9)
+    # a strongly negative pre-activation of the activated half switches the MLP off; of the other half it does not
+    off = dict(wa, b_ff_in=np.full(ff, -30.0), w_ff_in=np.zeros((ff, d)))
+    np.testing.assert_allclose(O.truth_prenorm_geglu_layer(x, off, mask, H), x + w["b_ff2"], atol=1e-9)
+    other = dict(wa, b_ff_gate=np.full(ff, -30.0), w_ff_gate=np.zeros((ff, d)))
+    assert np.abs(O.truth_prenorm_geglu_layer(x, other, mask, H) - x - w["b_ff2"]).max() > 1e-2
+    # the attention block uses rotated Q,K: it differs from the same block without rotation
+    wm = dict(w, w_ff2=np.zeros((d, ff)), b_ff2=np.zeros(d))
+    qkv = x @ w["w_qkv"].T + w["b_qkv"]
+    q, k, v = (qkv[..., i * d:(i + 1) * d].reshape(B, S, H, d // H) for i in range(3))
+    plain = x + O.truth_attention(q, k, v, mask=mask).reshape(B, S, d) @ w["w_o"].T + w["b_o"]
+    rot = x + O.truth_attention(O.truth_rope(q, style="half"), O.truth_rope(k, style="half"), v, mask=mask).reshape(B, S, d) @ w["w_o"].T + w["b_o"]
+    got = O.truth_prenorm_geglu_layer(x, wm, mask, H)
+    np.testing.assert_allclose(got, rot, rtol=1e-9, atol=1e-9)
+    assert np.abs(got - plain).max() > 1e-3
+    assert full.shape == x.shape
