@@ -166,7 +166,9 @@ __global__ __launch_bounds__(256) void layernorm_bf16x8_kernel(
                 o[4 + i] = g1[i] * ((t[c][4 + i] - mean) / sd) + b1[i];
             }
             const u32x4 w = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7])};
-            __builtin_nontemporal_store(w, (u32x4*)(yr + ch * 8));
+            // plain store: the next kernel (a GEMM) reads these rows at once, and leaving them in the
+            // cache hierarchy is worth more there than the streaming hint is here
+            *(u32x4*)(yr + ch * 8) = w;
         }
     }
 }
