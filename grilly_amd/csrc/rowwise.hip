@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
             vec4<T> o;
 #pragma unroll
             for (int i = 0; i < 4; ++i) o.set(i, g[i] * ((t[c][i] - mean) / sd) + b[i]);
-            o.store_stream(yr + ch * 4);
+            o.store(yr + ch * 4);      // plain: the next kernel reads these rows at once
         }
     }
 }
