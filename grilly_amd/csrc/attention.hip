@@ -289,7 +289,7 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
                 }
             }
         });
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = halves_max(mx);
         const float m_new = fmaxf(m_run, mx);
         const float alpha = __expf(m_run - m_new);
         m_run = m_new;
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
     }
 
     // ---- normalise and store: lane holds, for its query, dims 32dt + 8qd + 4lg + {0..3}
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float l_tot = halves_sum(l_run);
     const float inv = 1.0f / fmaxf(l_tot, 1e-10f);
     if (qi < S) {
         T* Og = (T*)p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
@@ -630,7 +630,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
                     for (int r = 0; r < 16; r += 2) mx = __builtin_fmaxf(mx, __builtin_fmaxf(sacc[u][t][r], sacc[u][t][r + 1]));
                 });
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = halves_max(mx);
             if (!lazy) {
                 // absolute scores: the classic running maximum
                 mx = fmaxf(m_run[u], mx);

@@ -146,6 +146,20 @@ __device__ __forceinline__ void dma16s(rsrc_words rs, const void* lds_dst_wave_u
     asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(la), "v"(voff), "s"(rs), "s"(so) : "memory");
 }
 
+// Reductions over the two 32-lane halves of a wave (lane i with lane i+32) through the half-swap
+// instruction: one VALU operation instead of an LDS permute and its round trip.  After the swap the
+// first result holds the lower half's values in both halves, the second the upper half's.
+__device__ __forceinline__ float halves_max(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+}
+__device__ __forceinline__ float halves_sum(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
+
 template <typename T> struct elem;
 template <> struct elem<float> {
     static __device__ __forceinline__ float ld(const float* p) { return *p; }
