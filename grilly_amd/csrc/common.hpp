@@ -160,6 +160,27 @@ __device__ __forceinline__ float halves_sum(float v) {
     return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
 }
 
+// All-reduce (sum) over groups of 16, 32 or 64 consecutive lanes without LDS permutes: four rotations
+// inside each 16-lane row (DPP operands of the additions), then the row-pair swap and the half swap.
+// All lanes of a group must be active.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int LANES> __device__ __forceinline__ float group_sum(float v) {
+    static_assert(LANES == 16 || LANES == 32 || LANES == 64, "16, 32 or 64 lanes");
+    v += dpp_move<0x128>(v);      // row_ror:8
+    v += dpp_move<0x124>(v);      // row_ror:4
+    v += dpp_move<0x122>(v);      // row_ror:2
+    v += dpp_move<0x121>(v);      // row_ror:1
+    if constexpr (LANES >= 32) {
+        const unsigned u = __builtin_bit_cast(unsigned, v);
+        const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);   // rows (0,1) and (2,3) exchange
+        v = __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+    }
+    if constexpr (LANES == 64) v = halves_sum(v);
+    return v;
+}
+
 template <typename T> struct elem;
 template <> struct elem<float> {
     static __device__ __forceinline__ float ld(const float* p) { return *p; }

@@ -35,11 +35,7 @@ template <> struct vec4<uint16_t> {
     }
 };
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
+__device__ __forceinline__ float wave_sum(float v) { return group_sum<64>(v); }   // whole wave active
 
 // ------------------------------------------------------------------ LayerNorm
 // One wave per row.  Rows of up to 64*4*MAXC elements (F % 4 == 0) stay in registers
@@ -138,8 +134,7 @@ __global__ __launch_bounds__(256) void layernorm_bf16x8_kernel(
             for (int i = 0; i < 8; ++i) t[c][i] = 0.f;
         }
     }
-#pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    s = group_sum<LPR>(s);
     const float mean = s / (float)F;
     float q = 0.f;
 #pragma unroll
@@ -149,8 +144,7 @@ __global__ __launch_bounds__(256) void layernorm_bf16x8_kernel(
             for (int i = 0; i < 8; ++i) { float d = t[c][i] - mean; q += d * d; }
         }
     }
-#pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) q += __shfl_xor(q, o, 64);
+    q = group_sum<LPR>(q);
     const float sd = sqrtf(q / (float)F + eps);
     uint16_t* yr = y + row * (int64_t)F;
 #pragma unroll
