@@ -454,13 +454,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     issue_bias(n0, bbuf);
 
     for (;;) {
+        // not zeroed: the first slab's multiplications start every accumulator from a constant zero
         f32x16 acc[TM][TN];
-#pragma unroll
-        for (int a = 0; a < TM; ++a)
-#pragma unroll
-            for (int b = 0; b < TN; ++b)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
         // where the next tile is: index arithmetic done here hides under the wait for the first slab
         const int npid = pid + (int)gridDim.x;
@@ -476,7 +471,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
 
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's transfers (and earlier stores) are done
         __syncthreads();                         // ... and everybody else's; all staging reads of the last tile too
-        for (int kt = 0; kt < KT; ++kt) {
+        auto k_slab = [&](int kt, auto ifirst) {
+            constexpr bool FIRST = decltype(ifirst)::value;
             if (kt + 1 < KT) {
                 if (!PAIRED) issue(rsA, rsW, kt + 1);
                 else if (((wave >> 2) & 1) == (kt & 1)) {
@@ -495,13 +491,20 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                 for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ lds_swz<8>(rowW[b])) << 4));
                 static_for<TM>([&](auto ia) {
                     static_for<TN>([&](auto ib) {
-                        MfmaSlab<T>::run(wf[decltype(ib)::value], xf[decltype(ia)::value], acc[decltype(ia)::value][decltype(ib)::value]);
+                        constexpr int a = decltype(ia)::value, b = decltype(ib)::value;
+                        if (FIRST && sl == 0) {
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;      // folds into the MFMA's C operand
+                        }
+                        MfmaSlab<T>::run(wf[b], xf[a], acc[a][b]);
                     });
                 });
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();
-        }
+        };
+        k_slab(0, std::true_type{});              // the host never launches this kernel with K == 0
+        for (int kt = 1; kt < KT; ++kt) k_slab(kt, std::false_type{});
 
         // both LDS stages are free now: request the next tile's first slab into stage 0
         if (has_next) {
