@@ -32,7 +32,7 @@ PEAK_HBM = 8.0e12       # B/s
 # rocprofv3 --pmc FETCH_SIZE (x2, the factor a 1 GiB copy kernel calibrates) + --pmc WRITE_SIZE (x1) on
 # `bench.py --mode gemm`; summary in profiles/gemm_bf16_bert_shapes_hbm_traffic.md.  A profiler reading, not
 # something this script can measure itself, so it is reported only for exactly that workload.
-GEMM_TRAFFIC_BYTES = {("bf16", 128, 512): 618.1e6}
+GEMM_TRAFFIC_BYTES = {("bf16", 128, 512): 617.2e6}
 
 
 WARM = 5
