@@ -59,6 +59,7 @@ SIGNATURES = {
     "grl_gemm_nn": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "grl_swiglu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 8),
     "grl_glu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 8 + [c_int]),
+    "grl_gemm_nt_res": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 5),
     "grl_gemm_nt_act": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 4 + [c_int, c_float, c_float]),
     "grl_fa2_fwd": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64] + [c_void_p] * 5 + [c_float, c_int, c_int, c_float, c_float, c_void_p]),
     "grl_fa2_fwd_strided": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64] + [c_void_p] * 5 + [c_i64] * 4 + [c_float, c_int, c_int, c_float, c_float]),

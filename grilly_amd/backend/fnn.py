@@ -42,6 +42,35 @@ class HipFNN:
         return self.core.pool_stats()
 
     # ------------------------------------------------------------------ GEMM family
+    def fused_linear_residual(self, x, weights, bias, residual, dtype="fp32"):
+        """residual + x.W^T + b in one kernel: the reference's linear followed by residual
+        (backend/fnn.py:1394-1496 then :1950-2014), as its encoder recipes chain them.  Not a method of the
+        reference's VulkanFNN; same shape rules as linear, residual shaped like the result."""
+        code = dtype_code(dtype)
+        x = np.asarray(x)
+        W = np.asarray(weights)
+        if W.ndim != 2:
+            raise ValueError("weights must be (out_features, in_features)")
+        N, K = W.shape
+        x2 = _as2d(x, K)
+        M = x2.shape[0]
+        r = np.asarray(residual)
+        if r.size != M * N:
+            raise ValueError(f"residual has {r.size} elements, expected {M * N}")
+        if bias is not None and np.asarray(bias).size != N:
+            raise ValueError(f"bias has {np.asarray(bias).size} elements, expected {N}")
+        c = self.core
+        dx, dw, dr = c.upload(x2, code), c.upload(W, code), c.upload(r.reshape(M, N), code)
+        db = c.upload(np.asarray(bias).reshape(-1)) if bias is not None else None
+        try:
+            L.check(c.lib.grl_gemm_nt_res(c.ctx, code, code, M, N, K, dx.ptr, dw.ptr, db.ptr if db else None, dr.ptr,
+                                          dr.ptr), "gemm_nt_res")          # in place on the residual buffer
+            return c.download(dr, (M, N), code).reshape(r.shape)
+        finally:
+            for b in (dx, dw, db, dr):
+                if b is not None:
+                    b.free()
+
     def _linear_impl(self, x, weights, bias, epi, dtype, alpha=1.0, beta=1.0):
         code = dtype_code(dtype)
         W = np.asarray(weights)

@@ -33,6 +33,13 @@ __global__ __launch_bounds__(256) void bias_fill_kernel(OutT* C, const float* bi
     elem<OutT>::st(C + i, v);
 }
 
+template <typename OutT>
+__global__ __launch_bounds__(256) void bias_residual_kernel(OutT* C, const OutT* R, const float* bias, int64_t total, int N) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    elem<OutT>::st(C + i, elem<OutT>::ld(R + i) + (bias ? bias[i % N] : 0.f));
+}
+
 extern "C" int grl_gemm_nt_act(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
                                const void* A, const void* W, const float* bias, void* C, int epilogue,
                                float alpha, float beta) {
@@ -57,6 +64,29 @@ extern "C" int grl_gemm_nt_act(grl_ctx* c, int in_dtype, int out_dtype, int64_t 
         return GRL_OK;
     }
     return dispatch_types(c, a, in_dtype, out_dtype, epi);
+}
+
+extern "C" int grl_gemm_nt_res(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                               const void* A, const void* W, const float* bias, const void* residual, void* C) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_gemm_nt_res: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_gemm_nt_res: bad dtype");
+    int rc = check_dims("grl_gemm_nt_res", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    GRL_REQUIRE(C && residual && (K == 0 || (A && W)), GRL_ERR_ARG, "grl_gemm_nt_res: null argument");
+    if (K == 0) {       // empty sum: C = bias + residual (element-wise, so C may be the residual)
+        int64_t total = M * N;
+        GRL_REQUIRE((total + 255) / 256 < (1LL << 31), GRL_ERR_SHAPE, "grl_gemm_nt_res: output too large");
+        const dim3 grid((unsigned)((total + 255) / 256));
+        if (out_dtype == GRL_F32) hipLaunchKernelGGL(bias_residual_kernel<float>, grid, dim3(256), 0, c->stream, (float*)C, (const float*)residual, bias, total, (int)N);
+        else hipLaunchKernelGGL(bias_residual_kernel<uint16_t>, grid, dim3(256), 0, c->stream, (uint16_t*)C, (const uint16_t*)residual, bias, total, (int)N);
+        GRL_CHECK_LAUNCH();
+        return GRL_OK;
+    }
+    GemmArgs a{};
+    a.A = A; a.W = W; a.bias = bias; a.C = C; a.residual = residual;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    return dispatch_types(c, a, in_dtype, out_dtype, EPI_RES);
 }
 
 extern "C" int grl_gemm_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,

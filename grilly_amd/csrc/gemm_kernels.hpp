@@ -41,12 +41,14 @@ struct GemmArgs {
     int group;           // tile-rows per band of the tile walk
     int act;             // run-time activation code of the EPI_RT / dual epilogues (a GRL_EPI_* value)
     float alpha, beta;   // RoSwish parameters
+    const void* residual; // (M,N) of the output type, added to the result (EPI_RES), else null
 };
 
 // Epilogue template codes.  NONE / GELU / SILU are compiled in (the encoder's hot shapes); EPI_RT picks
 // ReLU / GCU / RoSwish from GemmArgs::act at run time (one more instantiation instead of three), and the
 // dual-weight epilogue EPI_GLU picks the gate activation (SiLU / ReLU / GELU) the same way.
-enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_RT = 3, EPI_GLU = 4 };
+// EPI_RES adds a residual tensor of the output type where the result is stored (C may be the residual itself).
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_RT = 3, EPI_GLU = 4, EPI_RES = 5 };
 
 // shaders/fused-linear-relu.glsl:63, fused-linear-gcu.glsl:44-46 (x*cos(x)), fused-linear-roswish.glsl:46-58
 // ((x+alpha)*sigmoid(beta*x) - alpha/2; the shader's sign-split sigmoid equals 1/(1+exp(-beta*x)) with the
@@ -108,6 +110,35 @@ template <> __device__ __forceinline__ void store4<uint16_t>(uint16_t* p, float 
     *(u32x2*)p = v;
 }
 
+// residual helpers: 4 values of the output type at r added to v; one 16-byte chunk of outputs plus the
+// matching residual chunk (8 bf16 or 4 fp32 values, fp32 sum, one rounding)
+template <typename OutT> __device__ __forceinline__ void add4(const OutT* r, float (&v)[4]);
+template <> __device__ __forceinline__ void add4<float>(const float* r, float (&v)[4]) {
+    const f32x4 t = *(const f32x4*)r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] += t[e];
+}
+template <> __device__ __forceinline__ void add4<uint16_t>(const uint16_t* r, float (&v)[4]) {
+    const u32x2 t = *(const u32x2*)r;
+    v[0] += bf16lo(t[0]); v[1] += bf16hi(t[0]); v[2] += bf16lo(t[1]); v[3] += bf16hi(t[1]);
+}
+template <typename OutT> __device__ __forceinline__ u32x4 add_chunk(u32x4 c, u32x4 r);
+template <> __device__ __forceinline__ u32x4 add_chunk<float>(u32x4 c, u32x4 r) {
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = f2u(u2f(c[e]) + u2f(r[e]));
+    return o;
+}
+template <> __device__ __forceinline__ u32x4 add_chunk<uint16_t>(u32x4 c, u32x4 r) {
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t cw = c[e], rw = r[e];
+        o[e] = pack_bf16x2(bf16lo(cw) + bf16lo(rw), bf16hi(cw) + bf16hi(rw));
+    }
+    return o;
+}
+
 // ---- direct epilogue: lane (li, lg) holds, for output row m = .. + li, the columns
 // n = .. + 8*q + 4*lg + {0..3} in accumulator registers 4q..4q+3 and stores them itself
 // (8- or 16-byte stores).  Every index into the accumulators is a compile-time constant so
@@ -152,6 +183,7 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
+                            if constexpr (EPI == EPI_RES) add4<OutT>((const OutT*)p.residual + o, v);
                         }
                         store4<OutT>(C + o, v[0], v[1], v[2], v[3]);
                     } else {
@@ -166,6 +198,7 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
                                     x = glu_apply(x, y, p);
                                 } else {
                                     x = epi_apply<EPI>(x, p);
+                                    if constexpr (EPI == EPI_RES) x += elem<OutT>::ld((const OutT*)p.residual + o + e);
                                 }
                                 elem<OutT>::st(C + o + e, x);
                             }
@@ -568,7 +601,23 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                     val[i] = *(const u32x4*)(reg + r * CROWB + ((cc ^ (r & (CPR - 1))) << 4));
                 }
             };
-            auto store_band = [&](auto ia, const u32x4 (&val)[PER]) {
+            // EPI_RES: this thread's residual chunks of band a, requested while the band is still on its way
+            // through LDS (chunks outside the matrix are not read)
+            auto fetch_res = [&](auto ia, u32x4 (&res)[PER]) {
+                constexpr int a = decltype(ia)::value;
+                if constexpr (EPI == EPI_RES) {
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) {
+                        const int id = tid + i * NT;
+                        const int r = id / CPR, cc = id % CPR;
+                        const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
+                        const int n = n0 + cc * EPCO;
+                        res[i] = u32x4{0u, 0u, 0u, 0u};
+                        if (m < p.M && n < p.N) res[i] = __builtin_nontemporal_load((const u32x4*)((const OutT*)p.residual + (int64_t)m * p.N + n));
+                    }
+                }
+            };
+            auto store_band = [&](auto ia, const u32x4 (&val)[PER], const u32x4 (&res)[PER]) {
                 constexpr int a = decltype(ia)::value;
 #pragma unroll
                 for (int i = 0; i < PER; ++i) {
@@ -576,8 +625,10 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                     const int r = id / CPR, cc = id % CPR;
                     const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
                     const int n = n0 + cc * EPCO;
+                    u32x4 out = val[i];
+                    if constexpr (EPI == EPI_RES) out = add_chunk<OutT>(out, res[i]);
                     // written once, read by another kernel: keep it from displacing the operand panels in L2
-                    if (m < p.M && n < p.N) __builtin_nontemporal_store(val[i], (u32x4*)(C + (int64_t)m * p.N + n));
+                    if (m < p.M && n < p.N) __builtin_nontemporal_store(out, (u32x4*)(C + (int64_t)m * p.N + n));
                 }
             };
             // Barriers here are LDS-only (a fence would also wait for the global stores of earlier bands).
@@ -588,10 +639,11 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                 static_for<TM>([&](auto ia) {
                     constexpr int a = decltype(ia)::value;
                     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                    u32x4 val[PER];
+                    u32x4 val[PER], res[PER];
                     fetch_band(ia, val);
+                    fetch_res(ia, res);
                     if constexpr (a + 1 < TM) stage_band(std::integral_constant<int, a + 1>{});
-                    store_band(ia, val);
+                    store_band(ia, val, res);
                 });
             } else {
                 static_for<TM>([&](auto ia) {
@@ -599,7 +651,38 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
                     u32x4 val[PER];
                     fetch_band(ia, val);
-                    store_band(ia, val);
+                    if constexpr (EPI == EPI_RES) {
+                        // residual chunks in two halves: a whole band of them next to the staged values and
+                        // the other band's accumulators does not fit the register file
+                        constexpr int a = decltype(ia)::value;
+                        constexpr int HP = PER >= 2 ? PER / 2 : PER;
+#pragma unroll
+                        for (int h = 0; h < PER / HP; ++h) {
+                            u32x4 rr[HP];
+                            bool in[HP];
+#pragma unroll
+                            for (int j = 0; j < HP; ++j) {
+                                const int id = tid + (h * HP + j) * NT;
+                                const int r = id / CPR, cc = id % CPR;
+                                const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
+                                const int n = n0 + cc * EPCO;
+                                in[j] = m < p.M && n < p.N;
+                                rr[j] = u32x4{0u, 0u, 0u, 0u};
+                                if (in[j]) rr[j] = __builtin_nontemporal_load((const u32x4*)((const OutT*)p.residual + (int64_t)m * p.N + n));
+                            }
+#pragma unroll
+                            for (int j = 0; j < HP; ++j) {
+                                const int id = tid + (h * HP + j) * NT;
+                                const int r = id / CPR, cc = id % CPR;
+                                const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
+                                const int n = n0 + cc * EPCO;
+                                if (in[j]) __builtin_nontemporal_store(add_chunk<OutT>(val[h * HP + j], rr[j]), (u32x4*)(C + (int64_t)m * p.N + n));
+                            }
+                        }
+                    } else {
+                        u32x4 res[PER];
+                        store_band(ia, val, res);
+                    }
                     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
                 });
             }
@@ -633,6 +716,7 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmArgs p) {
         s = glu_apply(s, u, p);
     } else {
         s = epi_apply<EPI>(s, p);
+        if constexpr (EPI == EPI_RES) s += elem<OutT>::ld((const OutT*)p.residual + idx);
     }
     elem<OutT>::st((OutT*)p.C + idx, s);
 }
@@ -642,7 +726,7 @@ template <typename T, typename OutT, int EPI, bool DUAL>
 static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     const int64_t epc = 16 / (int64_t)sizeof(T);
     const bool aligned = (a.K % epc == 0) && ((((uintptr_t)a.A) | ((uintptr_t)a.W) | ((uintptr_t)a.W2)) & 15u) == 0 &&
-                         ((((uintptr_t)a.C) | ((uintptr_t)a.bias) | ((uintptr_t)a.bias2) | ((uintptr_t)a.cache1) | ((uintptr_t)a.cache2)) & 15u) == 0;
+                         ((((uintptr_t)a.C) | ((uintptr_t)a.bias) | ((uintptr_t)a.bias2) | ((uintptr_t)a.cache1) | ((uintptr_t)a.cache2) | ((uintptr_t)a.residual)) & 15u) == 0;
     if (!aligned) {
         int64_t total = (int64_t)a.M * a.N;
         GRL_REQUIRE((total + 255) / 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: unaligned problem too large for the scalar kernel");
@@ -697,6 +781,7 @@ int dispatch_epi(grl_ctx* c, GemmArgs& a, int epi) {
         case EPI_SILU: return launch_gemm<T, OutT, EPI_SILU, false>(c, a);
         case EPI_RT: return launch_gemm<T, OutT, EPI_RT, false>(c, a);
         case EPI_GLU: return launch_gemm<T, OutT, EPI_GLU, true>(c, a);
+        case EPI_RES: return launch_gemm<T, OutT, EPI_RES, false>(c, a);
     }
     grl_set_error("gemm: bad epilogue %d", epi);
     return GRL_ERR_ARG;

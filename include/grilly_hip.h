@@ -132,6 +132,13 @@ int grl_gemm_nt_act(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_
                     const void* A, const void* W, const float* bias, void* C, int epilogue,
                     float alpha, float beta);
 
+/* C = A.W^T + bias + residual, the residual (M,N) of the output type; C may be the residual buffer itself.
+ * One pass for what the reference does as a linear followed by VulkanFNN.residual
+ * (backend/fnn.py:1950-2014, shaders/fnn-residual.glsl:25-34; the pair as the encoder recipes use it,
+ * utils/vulkan_sentence_transformer.py:893, 945 and, in front of the LayerNorm, :1001-1004, :1023-1026). */
+int grl_gemm_nt_res(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                    const void* A, const void* W, const float* bias, const void* residual, void* C);
+
 /* out[m,n] = (x.Wg^T + bg)[m,n] * act((x.Wu^T + bu)[m,n]) with act = GRL_EPI_SILU (SwiGLU, below),
  * GRL_EPI_RELU (fused_reglu, backend/_glu_append.py:131-222, shaders/fused-reglu.glsl:42-75) or
  * GRL_EPI_GELU (fused_geglu, backend/_glu_append.py:224-315, shaders/fused-geglu.glsl:43-82: tanh GELU

@@ -261,3 +261,50 @@ def test_buffer_pool_stats(backend):
     s1 = backend.fnn.get_buffer_pool_stats()
     assert s1["hits"] - s0["hits"] >= 60 and s1["allocations"] - s0["allocations"] < 10    # reference claims <10 allocs / 100 ops
     assert 0.0 <= s1["hit_rate"] <= 1.0 and s1["bytes_in_use"] == s0["bytes_in_use"]
+
+
+RES_SHAPES = [(1, 8, 4), (3, 16, 5), (33, 40, 17), (130, 264, 250), (257, 72, 513), (300, 2056, 136),
+              (1024, 384, 1536), (2048, 768, 768), (16384, 768, 768), (4096, 3072, 768)]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("M,K,N", RES_SHAPES)
+def test_linear_residual_parity(backend, dtype, M, K, N):
+    """residual + x.W^T + b in one kernel against linear followed by residual
+    (backend/fnn.py:1394-1496, :1950-2014): every kernel variant (ragged, 128- and 256-wide tiles)."""
+    rng = np.random.default_rng(M * 5 + K * 11 + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    W = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    r = (3.0 * rng.standard_normal((M, N))).astype(np.float32)
+    x, W, r = prep(dtype, x, W, r)
+    ref = O.truth_linear(x, W, b) + r.astype(np.float64)
+    y = backend.fnn.fused_linear_residual(x, W, b, r, dtype=dtype)
+    assert y.shape == (M, N) and y.dtype == np.float32
+    assert O.max_rel(y, ref) < tol(dtype)
+    y0 = backend.fnn.fused_linear_residual(x, W, None, r, dtype=dtype)
+    assert O.max_rel(y0, O.truth_linear(x, W) + r.astype(np.float64)) < tol(dtype)
+
+
+def test_linear_residual_shapes_and_errors(backend):
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((2, 5, 16)).astype(np.float32)
+    W = rng.standard_normal((24, 16)).astype(np.float32)
+    r = rng.standard_normal((2, 5, 24)).astype(np.float32)
+    y = backend.fnn.fused_linear_residual(x, W, None, r)
+    assert y.shape == (2, 5, 24)
+    assert O.max_rel(y, O.truth_linear(x.reshape(10, 16), W).reshape(2, 5, 24) + r) < TOL_F32
+    with pytest.raises(ValueError):
+        backend.fnn.fused_linear_residual(x, W, None, r[:, :4])
+    with pytest.raises(ValueError):
+        backend.fnn.fused_linear_residual(x, W, np.zeros(23, np.float32), r)
+    # the C entry point: empty K gives bias + residual; a missing residual is an argument error
+    c = backend.core
+    M, N = 7, 12
+    b = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    db, dr = c.upload(b), c.upload(res)
+    L.check(c.lib.grl_gemm_nt_res(c.ctx, L.GRL_F32, L.GRL_F32, M, N, 0, None, None, db.ptr, dr.ptr, dr.ptr))
+    np.testing.assert_allclose(c.download(dr, (M, N)), res + b, rtol=1e-6, atol=1e-6)
+    assert c.lib.grl_gemm_nt_res(c.ctx, L.GRL_F32, L.GRL_F32, M, N, 0, None, None, db.ptr, None, dr.ptr) != 0
+    db.free(); dr.free()
