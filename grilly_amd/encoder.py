@@ -205,7 +205,8 @@ class PreNormEncoder:
         pooled = x[:, 0, :] (first token), L2-normalised                       (:1179-1183, :1194-1201)
 
     Built from the same entry points as the post-LN encoder: the projection GEMMs, attention with the
-    rotate-half rotation fused, LayerNorm, the dual GEMM with the GELU gate and the elementwise add.
+    rotate-half rotation fused, LayerNorm, the dual GEMM with the GELU gate, and the GEMM that adds the
+    residual stream in place.
     The packed Wqkv is read through three row blocks (no split copy).  The +-50 / +-1e6 clips the
     reference puts around the gate (:924-930) are not applied: they only act beyond those magnitudes."""
 
@@ -296,17 +297,15 @@ class PreNormEncoder:
             L.check(lib.grl_fa2_fwd(c.ctx, code, B, S, H, D, self.q.ptr, self.k.ptr, self.v.ptr, mask, self.att.ptr,
                                     1.0 / float(np.sqrt(D)), 0, L.ROPE_HALF, cfg.rope_base, cfg.rope_scaling, None),
                     "attention")
-            L.check(lib.grl_gemm_nt(c.ctx, code, code, M, d, d, self.att.ptr, w["w_o"].ptr, w["b_o"].ptr, self.t.ptr,
-                                    L.EPI_NONE), "output projection")
-            L.check(lib.grl_add(c.ctx, code, M * d, self.x.ptr, self.t.ptr, self.x.ptr), "residual")
+            L.check(lib.grl_gemm_nt_res(c.ctx, code, code, M, d, d, self.att.ptr, w["w_o"].ptr, w["b_o"].ptr, self.x.ptr,
+                                        self.x.ptr), "output projection + residual")
             L.check(lib.grl_layernorm(c.ctx, code, M, d, self.x.ptr, None, w["ffn_ln_g"].ptr, w["ffn_ln_b"].ptr, cfg.eps,
                                       self.t.ptr), "mlp layernorm")
             # the dual GEMM activates its second ("up") operand: that is the first half of Wi here
             L.check(lib.grl_glu_nt(c.ctx, code, code, M, ff, d, self.t.ptr, w["w_ff_gate"].ptr, w["w_ff_in"].ptr,
                                    w["b_ff_gate"].ptr, w["b_ff_in"].ptr, self.h.ptr, None, None, L.EPI_GELU), "geglu")
-            L.check(lib.grl_gemm_nt(c.ctx, code, code, M, d, ff, self.h.ptr, w["w_ff2"].ptr, w["b_ff2"].ptr, self.t.ptr,
-                                    L.EPI_NONE), "mlp output")
-            L.check(lib.grl_add(c.ctx, code, M * d, self.x.ptr, self.t.ptr, self.x.ptr), "residual")
+            L.check(lib.grl_gemm_nt_res(c.ctx, code, code, M, d, ff, self.h.ptr, w["w_ff2"].ptr, w["b_ff2"].ptr, self.x.ptr,
+                                        self.x.ptr), "mlp output + residual")
         if self.final is not None:
             L.check(lib.grl_layernorm(c.ctx, code, M, d, self.x.ptr, None, self.final[0].ptr, self.final[1].ptr,
                                       cfg.final_eps, self.x.ptr), "final layernorm")
