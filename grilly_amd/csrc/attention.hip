@@ -637,7 +637,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
                 pneg[u] = -mx;
                 const float alpha = __builtin_amdgcn_exp2f(m_run[u] - mx);
                 // rescale the running output and sum only when some row of the wave raised its maximum
-                if (__builtin_amdgcn_ballot_w64(mx != m_run[u]) != 0) {
+                // (never for the first tile: there is nothing accumulated yet)
+                if (kt > 0 && __builtin_amdgcn_ballot_w64(mx != m_run[u]) != 0) {
                     lacc[u][0] *= alpha;
                     sfor<DT>([&](auto idt) {
                         constexpr int dt = decltype(idt)::value;
