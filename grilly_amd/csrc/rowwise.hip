@@ -431,6 +431,11 @@ __global__ __launch_bounds__(256) void rope_kernel(const T* __restrict__ x, cons
 
 int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
                      const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling);
+int grl_build_rope_table_styled(grl_ctx* c, float* tab, int S, int D, float base, float scaling, int style);
+int grl_rope_apply_table(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                         void* y, const float* table);
+int grl_rope_half_apply_table(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                              void* y, const float* table);
 
 extern "C" int grl_rope(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x,
                         const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling) {
@@ -449,6 +454,20 @@ int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int
     GRL_REQUIRE(S < (1LL << 31) && H < (1LL << 31), GRL_ERR_SHAPE, "grl_rope: dimension too large");
     int64_t pairs = B * S * H * (D / 2);
     if (pairs == 0) return GRL_OK;
+    // Positions 0..S-1 and 16-byte granular rows: angles from a (S, D/2) table built once per call with the same
+    // fp32 angle arithmetic, rows moved as 16-byte chunks (the per-pair kernel below evaluates sincosf per pair).
+    {
+        const int64_t es = (int64_t)grl_dtype_size(dtype), epc = 16 / es;
+        const bool chunks = style == GRL_ROPE_HALF ? (D / 2) % epc == 0 : D % epc == 0;
+        if (!position_ids && chunks && ((((uintptr_t)x) | ((uintptr_t)y)) & 15u) == 0 && (x_stride * es) % 16 == 0 && S * (D / 2) < (1LL << 31)) {
+            grl_temp tab(c, (size_t)S * (D / 2) * sizeof(float2));
+            if (!tab.p) return GRL_ERR_OOM;
+            int rc = grl_build_rope_table_styled(c, (float*)tab.p, (int)S, (int)D, rope_base, rope_scaling, style);
+            if (rc) return rc;
+            return style == GRL_ROPE_HALF ? grl_rope_half_apply_table(c, dtype, B, S, H, D, x, x_stride, y, (const float*)tab.p)
+                                          : grl_rope_apply_table(c, dtype, B, S, H, D, x, x_stride, y, (const float*)tab.p);
+        }
+    }
     RopeFreq fr; grl_rope_freqs(&fr, (int)D, rope_base);
     dim3 g(ew_grid(pairs)), b(256);
     if (dtype == GRL_F32) hipLaunchKernelGGL(rope_kernel<float>, g, b, 0, c->stream, (const float*)x, position_ids, (float*)y, pairs, (int)S, (int)H, (int)D, style, rope_scaling, fr, x_stride);
@@ -458,22 +477,25 @@ int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int
 }
 
 // cos/sin table (S, D/2) pairs for the fused-RoPE attention kernel, interleaved-style angle.
-__global__ __launch_bounds__(256) void rope_table_kernel(float2* __restrict__ tab, int S, int half, float scaling, RopeFreq fr) {
+__global__ __launch_bounds__(256) void rope_table_kernel(float2* __restrict__ tab, int S, int half, float scaling, RopeFreq fr, int style) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= S * half) return;
     int s = i / half, p = i - s * half;
-    float theta = ((float)s * fr.inv_freq[p]) / scaling;
+    float theta = style == GRL_ROPE_HALF ? ((float)s / scaling) * fr.inv_freq[p] : ((float)s * fr.inv_freq[p]) / scaling;
     float sn, cs;
     sincosf(theta, &sn, &cs);
     tab[i] = make_float2(cs, sn);
 }
 
-int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling) {
+int grl_build_rope_table_styled(grl_ctx* c, float* tab, int S, int D, float base, float scaling, int style) {
     RopeFreq fr; grl_rope_freqs(&fr, D, base);
     int n = S * (D / 2);
-    hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, c->stream, (float2*)tab, S, D / 2, scaling, fr);
+    hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, c->stream, (float2*)tab, S, D / 2, scaling, fr, style);
     GRL_CHECK_LAUNCH();
     return GRL_OK;
+}
+int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling) {
+    return grl_build_rope_table_styled(c, tab, S, D, base, scaling, GRL_ROPE_INTERLEAVED);
 }
 
 // Interleaved RoPE from a precomputed (S, D/2) {cos, sin} table: one 16-byte chunk per thread,
@@ -520,6 +542,58 @@ int grl_rope_apply_table(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H,
     dim3 g(ew_grid(nchunks)), b(256);
     if (dtype == GRL_F32) hipLaunchKernelGGL(rope_table_apply_kernel<float>, g, b, 0, c->stream, (const float*)x, x_stride, (float*)y, (const float2*)table, nchunks, (int)S, (int)H, (int)D);
     else hipLaunchKernelGGL(rope_table_apply_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, x_stride, (uint16_t*)y, (const float2*)table, nchunks, (int)S, (int)H, (int)D);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+// Rotate-half RoPE from a (S, D/2) {cos, sin} table: a thread takes one 16-byte chunk of the first half of a
+// (position, head) row and its partner chunk D/2 further on (shaders/rope.glsl:74-125 pairs d with d + D/2).
+template <typename T>
+__global__ __launch_bounds__(256) void rope_half_apply_kernel(const T* __restrict__ x, int64_t x_stride, T* __restrict__ y,
+                                                             const float2* __restrict__ tab, int64_t nchunks, int S, int H, int D) {
+    constexpr int EPC = 16 / (int)sizeof(T);
+    const int half = D / 2, cph = half / EPC;      // chunks per half row
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nchunks; i += stride) {
+        const int c = (int)(i % cph);
+        const int64_t vec = i / cph;               // (b,s,h) flat
+        const int64_t bs = vec / H;
+        const int h = (int)(vec - bs * H), s = (int)(bs % S);
+        const T* xr = x + bs * x_stride + (int64_t)h * D + c * EPC;
+        const u32x4 lo = *(const u32x4*)xr, hi = *(const u32x4*)(xr + half);
+        const float2* t = tab + (int64_t)s * half + c * EPC;
+        u32x4 olo, ohi;
+        if (sizeof(T) == 2) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float2 c0 = t[2 * j], c1 = t[2 * j + 1];
+                const float a0 = bf16lo(lo[j]), a1 = bf16hi(lo[j]), b0 = bf16lo(hi[j]), b1 = bf16hi(hi[j]);
+                olo[j] = pack_bf16x2(a0 * c0.x - b0 * c0.y, a1 * c1.x - b1 * c1.y);
+                ohi[j] = pack_bf16x2(b0 * c0.x + a0 * c0.y, b1 * c1.x + a1 * c1.y);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float2 cs = t[j];
+                const float a = u2f(lo[j]), b = u2f(hi[j]);
+                olo[j] = f2u(a * cs.x - b * cs.y);
+                ohi[j] = f2u(b * cs.x + a * cs.y);
+            }
+        }
+        T* yr = y + vec * D + c * EPC;
+        *(u32x4*)yr = olo;
+        *(u32x4*)(yr + half) = ohi;
+    }
+}
+
+int grl_rope_half_apply_table(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                              void* y, const float* table) {
+    const int64_t epc = dtype == GRL_BF16 ? 8 : 4;
+    const int64_t nchunks = B * S * H * ((D / 2) / epc);
+    if (nchunks == 0) return GRL_OK;
+    dim3 g(ew_grid(nchunks)), b(256);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(rope_half_apply_kernel<float>, g, b, 0, c->stream, (const float*)x, x_stride, (float*)y, (const float2*)table, nchunks, (int)S, (int)H, (int)D);
+    else hipLaunchKernelGGL(rope_half_apply_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, x_stride, (uint16_t*)y, (const float2*)table, nchunks, (int)S, (int)H, (int)D);
     GRL_CHECK_LAUNCH();
     return GRL_OK;
 }

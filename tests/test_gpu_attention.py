@@ -156,3 +156,25 @@ def test_full_size_long_causal_rope_properties(backend):
         p = np.exp(s - s.max(-1, keepdims=True)); p /= p.sum(-1, keepdims=True)
         ref = np.einsum("hj,jhd->hd", p, v[0, :i + 1].astype(np.float64))
         assert O.max_rel(o[0, i], ref) < TOL_BF16, i
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("style", ["half", "interleaved"])
+@pytest.mark.parametrize("B,S,H,D", [(2, 37, 3, 32), (1, 130, 2, 64), (2, 19, 4, 128), (1, 9, 2, 24), (2, 11, 3, 6)])
+def test_apply_rope_parity_table_and_pairwise_paths(backend, dtype, style, B, S, H, D):
+    """apply_rope (backend/attention.py:599-676, shaders/rope.glsl:74-125) with default positions takes the
+    table-driven 16-byte path when the (half) row is 16-byte granular and the per-pair path otherwise
+    (D = 24, 6), and the per-pair path whenever position ids are given; all must agree with the oracle,
+    including base / scaling other than the defaults."""
+    rng = np.random.default_rng(B * 1000 + S * 10 + D)
+    x = rng.standard_normal((B, S, H, D)).astype(np.float32)
+    if dtype == "bf16":
+        x = O.bf16_round(x)
+    t = TOL_F32 if dtype == "fp32" else TOL_BF16
+    ref = O.truth_rope(x, 500.0, 1.5, style)
+    y = backend.attention.apply_rope(x, None, 500.0, 1.5, rope_style=style, dtype=dtype)
+    assert y.shape == x.shape and O.max_rel(y, ref) < t
+    pid = np.tile(np.arange(S, dtype=np.int32), (B, 1))
+    y2 = backend.attention.apply_rope(x, pid, 500.0, 1.5, rope_style=style, dtype=dtype)
+    assert O.max_rel(y2, ref) < t
+    assert O.max_rel(y2, y) < (1e-6 if dtype == "fp32" else 1e-2)      # same angles, same arithmetic
