@@ -8,12 +8,11 @@
 // The online-softmax state (running max m, running sum l) and the rescale factor are then
 // per-lane scalars; the only cross-lane step is one exchange with lane^32 for the row max.
 //
+// fp32 kernel (fa2_fwd_kernel, register-staged tiles):
 //   HBM --128-bit loads--> VGPR --(RoPE on K) --> LDS: K tile [key][d], XOR-swizzled chunks
-//                                              --> LDS: V tile, fp32 [key][d]; bf16 transposed
-//                                                  to [d][key] in 4-key groups so that the MFMA
-//                                                  operand is two 8-byte reads
+//                                              --> LDS: V tile [key][d]
 //   K/V tiles are double buffered; the next tile's loads are in flight during the MFMAs.
-//   S, P and O never leave registers; P is rounded to bf16 only as MFMA operand (bf16 path).
+//   S, P and O never leave registers.  The bf16 kernel further down moves its tiles HBM -> LDS directly.
 //
 // Semantics (constants of shaders/flash-attention2.glsl:95,152,214):
 //   score = <q,k>*scale + (mask[b,k]-1)*1e9 ; running max starts at -1e10 ;
@@ -109,16 +108,15 @@ template <> __device__ __forceinline__ void fa_store4<uint16_t>(uint16_t* p, flo
 
 template <typename T, int D, bool ROPE>
 __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
-    constexpr bool BF = sizeof(T) == 2;
+    static_assert(sizeof(T) == 4, "the register-staged kernel is the fp32 path");
     constexpr int ES = (int)sizeof(T), RB = D * ES, NCH = RB / 16, NS = RB / 32, EPC = 16 / ES;
-    constexpr int KT = (BF && D <= 64) ? 128 : 64;      // keys per tile
+    constexpr int KT = 64;                              // keys per tile
     constexpr int NKB = KT / 32, DT = D / 32;
     constexpr int CK = KT * NCH / 256;                  // K chunks per thread
-    constexpr int NU = BF ? (KT / 4) * (D / 8) : 0;     // bf16 V transposition units (4 keys x 8 dims)
-    constexpr int CV = BF ? 4 : CK;
+    constexpr int CV = CK;
     constexpr int TILE = KT * RB;
     constexpr int PPC = EPC / 2;                        // RoPE pairs per chunk
-    static_assert(KT * NCH % 256 == 0 && NU <= 256, "tile does not divide over 256 threads");
+    static_assert(KT * NCH % 256 == 0, "tile does not divide over 256 threads");
     __shared__ __attribute__((aligned(16))) char ldsK[2][TILE];
     __shared__ __attribute__((aligned(16))) char ldsV[2][TILE];
     __shared__ __attribute__((aligned(16))) float ldsBias[2][KT];
@@ -172,22 +170,11 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
                 for (int j = 0; j < PPC; ++j) kcs[i][j] = p.rope[(int64_t)kc * (D / 2) + c * PPC + j];
             }
         }
-        if (BF) {
-            if (tid < NU) {
-                const int dc = tid % (D / 8), kg = tid / (D / 8);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int kk = k0 + 4 * kg + j, kc = kk < S ? kk : S - 1;
-                    vreg[j] = *(const u32x4*)(Vg + (int64_t)kc * p.v_stride + dc * 8);
-                }
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < CV; ++i) {
-                const int q = tid + i * 256, key = q / NCH, c = q % NCH;
-                const int kk = k0 + key, kc = kk < S ? kk : S - 1;
-                vreg[i] = *(const u32x4*)(Vg + (int64_t)kc * p.v_stride + c * EPC);
-            }
+        for (int i = 0; i < CV; ++i) {
+            const int q = tid + i * 256, key = q / NCH, c = q % NCH;
+            const int kk = k0 + key, kc = kk < S ? kk : S - 1;
+            vreg[i] = *(const u32x4*)(Vg + (int64_t)kc * p.v_stride + c * EPC);
         }
         if (tid < KT) {
             const int kk = k0 + tid;
@@ -210,30 +197,10 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
             const int slot = c ^ lds_swz<NCH>(key);
             *(u32x4*)(Kb + key * RB + slot * 16) = v;
         }
-        if (BF) {
-            if (tid < NU) {
-                const int dc = tid % (D / 8), kg = tid / (D / 8);
-                u32x4 r[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) r[j] = (k0 + 4 * kg + j >= S) ? zero : vreg[j];
-#pragma unroll
-                for (int dd = 0; dd < 8; ++dd) {
-                    const int w = dd >> 1;
-                    uint32_t e0, e1, e2, e3;
-                    if (dd & 1) { e0 = r[0][w] >> 16; e1 = r[1][w] & 0xffff0000u; e2 = r[2][w] >> 16; e3 = r[3][w] & 0xffff0000u; }
-                    else { e0 = r[0][w] & 0xffffu; e1 = r[1][w] << 16; e2 = r[2][w] & 0xffffu; e3 = r[3][w] << 16; }
-                    const int d = dc * 8 + dd;
-                    const int slot = (kg + d + (d >> 4)) & (KT / 4 - 1);
-                    u32x2 o = {e0 | e1, e2 | e3};
-                    *(u32x2*)(Vb + d * (KT * 2) + slot * 8) = o;
-                }
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < CV; ++i) {
-                const int q = tid + i * 256, key = q / NCH, c = q % NCH;
-                *(u32x4*)(Vb + key * RB + c * 16) = (k0 + key >= S) ? zero : vreg[i];
-            }
+        for (int i = 0; i < CV; ++i) {
+            const int q = tid + i * 256, key = q / NCH, c = q % NCH;
+            *(u32x4*)(Vb + key * RB + c * 16) = (k0 + key >= S) ? zero : vreg[i];
         }
         if (tid < KT) ldsBias[st][tid] = breg;
     };
@@ -311,39 +278,18 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
         });
 
         // ---- O^T += V^T . P^T
-        if (BF) {
-            sfor<NKB>([&](auto it) {
-                constexpr int t = decltype(it)::value;
-#pragma unroll
-                for (int hh = 0; hh < 2; ++hh) {
-                    u32x4 pf;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) pf[e] = pack_bf16x2(sacc[t][8 * hh + 2 * e], sacc[t][8 * hh + 2 * e + 1]);
-                    const int kgA = 8 * t + 4 * hh + lg;
-                    sfor<DT>([&](auto idt) {
-                        constexpr int dt = decltype(idt)::value;
-                        const int d = 32 * dt + li, f = d + (d >> 4);
-                        u32x2 va = *(const u32x2*)(Vb + d * (KT * 2) + ((kgA + f) & (KT / 4 - 1)) * 8);
-                        u32x2 vb = *(const u32x2*)(Vb + d * (KT * 2) + ((kgA + 2 + f) & (KT / 4 - 1)) * 8);
-                        u32x4 vf = {va[0], va[1], vb[0], vb[1]};
-                        Slab<uint16_t>::run(vf, pf, oacc[dt]);
-                    });
-                }
-            });
-        } else {
-            sfor<NKB>([&](auto it) {
-                constexpr int t = decltype(it)::value;
-                sfor<16>([&](auto ir) {
-                    constexpr int r = decltype(ir)::value;
-                    const int kl = 32 * t + 8 * (r / 4) + 4 * lg + (r % 4);
-                    sfor<DT>([&](auto idt) {
-                        constexpr int dt = decltype(idt)::value;
-                        float vv = *(const float*)(Vb + kl * RB + (32 * dt + li) * 4);
-                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, sacc[t][r], oacc[dt], 0, 0, 0);
-                    });
+        sfor<NKB>([&](auto it) {
+            constexpr int t = decltype(it)::value;
+            sfor<16>([&](auto ir) {
+                constexpr int r = decltype(ir)::value;
+                const int kl = 32 * t + 8 * (r / 4) + 4 * lg + (r % 4);
+                sfor<DT>([&](auto idt) {
+                    constexpr int dt = decltype(idt)::value;
+                    float vv = *(const float*)(Vb + kl * RB + (32 * dt + li) * 4);
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, sacc[t][r], oacc[dt], 0, 0, 0);
                 });
             });
-        }
+        });
 
         if (more) stash_tile(kt + 1);
         __syncthreads();

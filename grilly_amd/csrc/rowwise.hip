@@ -44,8 +44,8 @@ __device__ __forceinline__ float wave_sum(float v) { return group_sum<64>(v); } 
 // shaders/fnn-layernorm.glsl:44-103).
 template <typename T, int MAXC, bool HAS_RES>
 __global__ __launch_bounds__(256) void layernorm_rows_kernel(
-    const T* __restrict__ x, const T* __restrict__ res, const float* __restrict__ gamma,
-    const float* __restrict__ beta, T* __restrict__ y, int64_t rows, int F, float eps) {
+    const T* x, const T* res, const float* __restrict__ gamma,
+    const float* __restrict__ beta, T* y, int64_t rows, int F, float eps) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -104,8 +104,8 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
 // wave (two rows per wave for F <= 1024 keeps 96 B of loads in flight per lane at F = 768 instead of 48).
 template <int MAXC, bool HAS_RES, int LPR>
 __global__ __launch_bounds__(256) void layernorm_bf16x8_kernel(
-    const uint16_t* __restrict__ x, const uint16_t* __restrict__ res, const float* __restrict__ gamma,
-    const float* __restrict__ beta, uint16_t* __restrict__ y, int64_t rows, int F, float eps) {
+    const uint16_t* x, const uint16_t* res, const float* __restrict__ gamma,
+    const float* __restrict__ beta, uint16_t* y, int64_t rows, int F, float eps) {
     constexpr int RPW = 64 / LPR;
     const int lane = threadIdx.x & 63, sub = lane % LPR;
     const int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPR;
@@ -170,8 +170,8 @@ __global__ __launch_bounds__(256) void layernorm_bf16x8_kernel(
 // Any F: three passes over the row from global memory (the second and third hit L2).
 template <typename T, bool HAS_RES>
 __global__ __launch_bounds__(256) void layernorm_rows_generic_kernel(
-    const T* __restrict__ x, const T* __restrict__ res, const float* __restrict__ gamma,
-    const float* __restrict__ beta, T* __restrict__ y, int64_t rows, int F, float eps) {
+    const T* x, const T* res, const float* __restrict__ gamma,
+    const float* __restrict__ beta, T* y, int64_t rows, int F, float eps) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -269,8 +269,7 @@ template <int OP> __device__ __forceinline__ float ew_apply(float a, float b) {
 }
 
 template <typename T, int OP, bool VEC>
-__global__ __launch_bounds__(256) void elementwise_kernel(const T* __restrict__ a, const T* __restrict__ b,
-                                                         T* __restrict__ out, int64_t n) {
+__global__ __launch_bounds__(256) void elementwise_kernel(const T* a, const T* b, T* out, int64_t n) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (VEC) {

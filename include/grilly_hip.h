@@ -194,11 +194,16 @@ int grl_rope(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D
  * biased variance, two-pass statistics in fp32.
  * Replaces VulkanFNN.layernorm (backend/fnn.py:1285-1389, shaders/fnn-layernorm.glsl:44-103);
  * the optional residual folds VulkanFNN.residual (backend/fnn.py:1950-2014) into the same
- * pass, which is how the encoder uses the pair (utils/vulkan_sentence_transformer.py:1004,1026). */
+ * pass, which is how the encoder uses the pair (utils/vulkan_sentence_transformer.py:1004,1026).
+ * In-place use is allowed: y may be x or residual (each element is read and written by the same lane).
+ * x and residual may also be the same buffer. */
 int grl_layernorm(grl_ctx* ctx, int dtype, int64_t rows, int64_t F, const void* x,
                   const void* residual, const float* gamma, const float* beta, float eps, void* y);
 
-/* out = a + b.  Replaces VulkanFNN.residual (shaders/fnn-residual.glsl:25-34). */
+/* out = a + b.  Replaces VulkanFNN.residual (shaders/fnn-residual.glsl:25-34).
+ * grl_add, grl_gelu, grl_silu and grl_relu may run in place (out == a, out == b, y == x).
+ * Every other entry point of this header needs its outputs distinct from its inputs unless its own
+ * comment says otherwise (grl_gemm_nt_res: C may be the residual; grl_bert_layer_fwd: x is updated in place). */
 int grl_add(grl_ctx* ctx, int dtype, int64_t n, const void* a, const void* b, void* out);
 /* Replaces VulkanFNN.activation_gelu (backend/fnn.py:285-342, shaders/activation-gelu.glsl:23-53). */
 int grl_gelu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);

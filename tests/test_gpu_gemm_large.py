@@ -1,0 +1,149 @@
+"""GPU parity of the GEMM family at shapes that select the kernels the benchmark times: the persistent
+256x256-tile kernel (chosen from 192 such tiles on), with every epilogue, both storage types, ragged edges,
+the register-staged variant for K rows that are not whole 128-byte slabs, and BASELINE configs[3]'s
+N = 11008 / K = 4096 / K = 11008 shapes (narrow-band tile walk).  The oracle (float64 closed forms of the
+reference shaders, shaders/fused-linear-gelu.glsl:42-93, fused-linear-silu.glsl:42-78,
+fused-swiglu.glsl:43-79, fnn-linear.glsl:33-58) is evaluated on sampled output rows that cover every
+256-row tile band (first row, last row and two random rows of each band).
+Tolerances: max|y-ref|/max|ref| <= 1e-4 (fp32), <= 2e-2 (bf16)."""
+import numpy as np
+import pytest
+
+from conftest import TOL_F32, TOL_BF16, rng_for
+from oracle import oracle_np as O
+
+pytestmark = pytest.mark.gpu
+
+
+def tol(dtype):
+    return TOL_F32 if dtype == "fp32" else TOL_BF16
+
+
+def prep(dtype, *arrs):
+    return [O.bf16_round(a) if dtype == "bf16" else a for a in arrs]
+
+
+def band_rows(M, rng, band=256, per=2):
+    """first and last row of every `band`-row tile band plus `per` random rows inside it"""
+    rows = []
+    for r0 in range(0, M, band):
+        r1 = min(M, r0 + band)
+        rows += [r0, r1 - 1] + list(rng.integers(r0, r1, per))
+    return np.unique(np.asarray(rows, dtype=np.int64))
+
+
+def big_tiles(M, N, dual=False):
+    return -(-M // 256) * -(-N // (128 if dual else 256))
+
+
+def gen(rng, M, K, N, wstd):
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    W = rng.standard_normal((N, K), dtype=np.float32) * np.float32(wstd)
+    b = rng.standard_normal(N, dtype=np.float32)
+    return x, W, b
+
+
+# (M, K, N): all >= 192 tiles of 256x256.  N = 3080 leaves an 8-column edge tile, M = 16384+37 a 37-row edge band.
+BIG = [(16384, 768, 3072), (16384 + 37, 768, 3072 + 8), (16384, 768, 768)]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("epi", ["none", "gelu", "silu", "relu", "roswish", "gcu"])
+@pytest.mark.parametrize("M,K,N", BIG)
+def test_big_tile_fused_linear(backend, dtype, epi, M, K, N):
+    if (M, K, N) == BIG[2] and epi in ("roswish", "gcu"):
+        pytest.skip("run-time epilogue is covered at the two wider shapes")
+    assert big_tiles(M, N) >= 192
+    rng = np.random.default_rng(M + 3 * N + len(epi))
+    x, W, b = gen(rng, M, K, N, 1.0 / np.sqrt(K))
+    x, W = prep(dtype, x, W)
+    f = backend.fnn
+    call = {"none": lambda bb: f.linear(x, W, bb, dtype=dtype),
+            "gelu": lambda bb: f.fused_linear_gelu(x, W, bb, dtype=dtype),
+            "silu": lambda bb: f.fused_linear_silu(x, W, bb, dtype=dtype),
+            "relu": lambda bb: f.fused_linear_relu(x, W, bb, dtype=dtype),
+            "gcu": lambda bb: f.fused_linear_gcu(x, W, bb, dtype=dtype),
+            "roswish": lambda bb: f.fused_linear_roswish(x, W, bb, alpha=0.7, beta=1.3, dtype=dtype)}[epi]
+    rows = band_rows(M, rng)
+    y = call(b)
+    assert y.shape == (M, N) and np.isfinite(y).all()
+    ref = O.truth_linear(x[rows], W, b, epi, 0.7, 1.3)
+    assert O.max_rel(y[rows], ref) < tol(dtype)
+    # without bias (the bias slice is not fetched at all then)
+    y0 = call(None)
+    ref0 = O.truth_linear(x[rows], W, None, epi, 0.7, 1.3)
+    assert O.max_rel(y0[rows], ref0) < tol(dtype)
+    # every element was written by exactly the row it belongs to: a second run is bit-identical
+    np.testing.assert_array_equal(call(b), y)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("act", ["silu", "gelu", "relu"])
+@pytest.mark.parametrize("M,K,N,bias", [(16384, 512, 3072, True), (16384 + 37, 512, 1152 + 8, False)])
+def test_big_tile_glu(backend, dtype, act, M, K, N, bias):
+    assert big_tiles(M, N, dual=True) >= 192
+    rng = np.random.default_rng(M + N + len(act))
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    Wg = rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.06)
+    Wu = rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.06)
+    bg = rng.standard_normal(N, dtype=np.float32) if bias else None
+    bu = rng.standard_normal(N, dtype=np.float32) if bias else None
+    x, Wg, Wu = prep(dtype, x, Wg, Wu)
+    fn = {"silu": backend.fnn.fused_swiglu, "gelu": backend.fnn.fused_geglu, "relu": backend.fnn.fused_reglu}[act]
+    rows = band_rows(M, rng)
+    t_out, t_g, t_u = (O.truth_fused_swiglu(x[rows], Wg, Wu, bg, bu) if act == "silu"
+                       else O.truth_fused_glu(x[rows], Wg, Wu, bg, bu, act))
+    out = fn(x, Wg, Wu, bg, bu, dtype=dtype)                      # LDS-staged epilogue
+    assert out.shape == (M, N) and np.isfinite(out).all()
+    assert O.max_rel(out[rows], t_out) < tol(dtype)
+    if act == "silu":
+        out2, g, u = fn(x, Wg, Wu, bg, bu, return_cache=True, dtype=dtype)     # direct epilogue with the fp32 pre-activations
+        assert O.max_rel(out2[rows], t_out) < tol(dtype)
+        assert O.max_rel(g[rows], t_g) < tol(dtype) and O.max_rel(u[rows], t_u) < tol(dtype)
+        np.testing.assert_array_equal(out2, out)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_big_tile_register_staged_variant(backend, dtype):
+    """K = 776: rows are 16-byte aligned but not whole 128-byte slabs, so the 256x256 register-staged kernel
+    with its zero-filled K tail runs (plain and with the residual epilogue)."""
+    M, K, N = 16384, 776, 3072
+    rng = np.random.default_rng(776)
+    x, W, b = gen(rng, M, K, N, 1.0 / np.sqrt(K))
+    r = 3.0 * rng.standard_normal((M, N), dtype=np.float32)
+    x, W, r = prep(dtype, x, W, r)
+    rows = band_rows(M, rng)
+    ref = O.truth_linear(x[rows], W, b)
+    y = backend.fnn.linear(x, W, b, dtype=dtype)
+    assert O.max_rel(y[rows], ref) < tol(dtype)
+    yr = backend.fnn.fused_linear_residual(x, W, b, r, dtype=dtype)
+    assert O.max_rel(yr[rows], ref + r[rows].astype(np.float64)) < tol(dtype)
+
+
+def test_config4_swiglu_mlp_shapes(backend):
+    """BASELINE configs[3] (reference backend/_glu_append.py:8-129 then backend/fnn.py:1394-1496):
+    X . (W_g, W_u)[11008,4096]^T -> silu(X.W_g) * (X.W_u) -> . W_d[4096,11008]^T in bf16 with fp32 accumulation,
+    at the full feature sizes (N = 11008, K = 4096, then K = 11008: the narrow-band tile walk) and M = 4096 of
+    the 16384 rows (16 x 86 and 16 x 16 tiles still select the persistent kernel).  Row-sampled against the
+    float64 oracle on the bf16-rounded inputs, plus exact homogeneity of the down projection under x2."""
+    rng = rng_for(4)
+    M, Kd, F = 4096, 4096, 11008
+    X = O.bf16_round(rng.standard_normal((M, Kd), dtype=np.float32))
+    Wg = O.bf16_round(rng.standard_normal((F, Kd), dtype=np.float32) * np.float32(0.02))
+    Wu = O.bf16_round(rng.standard_normal((F, Kd), dtype=np.float32) * np.float32(0.02))
+    Wd = O.bf16_round(rng.standard_normal((Kd, F), dtype=np.float32) * np.float32(0.02))
+    assert big_tiles(M, F, dual=True) >= 192 and big_tiles(M, Kd) >= 192
+    rows = band_rows(M, rng)
+    # config 4 wants SiLU on the gate product: the reference's fused_swiglu puts it on its W_up argument
+    Hh = backend.fnn.fused_swiglu(X, Wu, Wg, dtype="bf16")
+    assert Hh.shape == (M, F) and np.isfinite(Hh).all()
+    xs = X[rows].astype(np.float64)
+    want_h = O.truth_silu(xs @ Wg.T.astype(np.float64)) * (xs @ Wu.T.astype(np.float64))
+    assert O.max_rel(Hh[rows], want_h) < TOL_BF16
+    Hq = O.bf16_round(Hh)                        # the device buffer held exactly these values
+    np.testing.assert_array_equal(Hq, Hh)
+    Y = backend.fnn.linear(Hq, Wd, dtype="bf16")
+    assert Y.shape == (M, Kd) and np.isfinite(Y).all()
+    assert O.max_rel(Y[rows], O.truth_linear(Hq[rows], Wd)) < TOL_BF16
+    Y2 = backend.fnn.linear(2 * Hq[:1024], Wd, dtype="bf16")
+    np.testing.assert_array_equal(Y2, 2 * Y[:1024])
