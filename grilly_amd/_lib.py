@@ -57,6 +57,8 @@ SIGNATURES = {
     "grl_cast": (c_int, [c_void_p, c_int, c_int, c_i64, c_void_p, c_void_p]),
     "grl_gemm_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
     "grl_gemm_nn": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "grl_gemm_nn_noalloc": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p]),
+    "grl_gemm_nn_noalloc_max_bytes": (c_i64, []),
     "grl_swiglu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 8),
     "grl_glu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 8 + [c_int]),
     "grl_gemm_nt_res": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 5),

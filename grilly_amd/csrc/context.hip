@@ -4,6 +4,8 @@
 
 static thread_local char g_err[512] = "";
 
+int grl_gemm_scratch_init(grl_ctx* c);    // gemm.hip: device address of the static scratch of grl_gemm_nn_noalloc
+
 void grl_set_error(const char* fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -37,6 +39,11 @@ extern "C" grl_ctx* grl_create(int device) {
     }
     if (strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
         grl_set_error("device %d is %s; this library carries gfx950 code only", device, c->prop.gcnArchName);
+        hipStreamDestroy(c->stream);
+        delete c;
+        return nullptr;
+    }
+    if (grl_gemm_scratch_init(c) != GRL_OK) {      // message already set
         hipStreamDestroy(c->stream);
         delete c;
         return nullptr;

@@ -142,3 +142,61 @@ extern "C" int grl_gemm_nn(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, i
     if (own) grl_free(c, own);   // stream order keeps the block alive until the GEMM has read it
     return rc;
 }
+
+// ---------------------------------------------------------------------------------------------------
+// C = A.B without any allocation: the transposed copy of B that grl_gemm_nn takes from the caching pool (or
+// from a caller's workspace) lives in a file-scope device array instead.  Every GPU the library runs on
+// holds its own copy of the array (at its own address) until the process ends.  The array's name is only a
+// host-side handle: its device address is looked up once per device with that device current, and from
+// then on only that address is handed to kernels.
+#define GRL_NN_SCRATCH_BYTES (32u << 20)
+static __device__ __align__(256) unsigned char scratch[GRL_NN_SCRATCH_BYTES];
+
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[64];          // per device ordinal; null until looked up
+
+// device address of this GPU's copy of `scratch` (looked up on first use, with the device current)
+static int nn_scratch_address(grl_ctx* c, void** out) {
+    GRL_REQUIRE(c->device >= 0 && c->device < 64, GRL_ERR_ARG, "grl_gemm_nn_noalloc: device ordinal %d out of range", c->device);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[c->device]) {
+        GRL_CHECK_HIP(hipSetDevice(c->device));
+        void* ptr = nullptr;
+        GRL_CHECK_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+        GRL_REQUIRE(ptr, GRL_ERR_HIP, "grl_gemm_nn_noalloc: the scratch array has no device address");
+        g_scratch_ptr[c->device] = ptr;
+    }
+    *out = g_scratch_ptr[c->device];
+    return GRL_OK;
+}
+
+// called by grl_create so that the lookup happens at set-up, not inside a caller's no-allocation region
+int grl_gemm_scratch_init(grl_ctx* c) {
+    void* p = nullptr;
+    return nn_scratch_address(c, &p);
+}
+
+extern "C" int64_t grl_gemm_nn_noalloc_max_bytes(void) { return (int64_t)GRL_NN_SCRATCH_BYTES; }
+
+extern "C" int grl_gemm_nn_noalloc(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                   const void* A, const void* B, void* C) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_gemm_nn_noalloc: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_gemm_nn_noalloc: bad dtype");
+    int rc = check_dims("grl_gemm_nn_noalloc", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    if (K == 0) return grl_gemm_nt(c, in_dtype, out_dtype, M, N, 0, A, B, nullptr, C, GRL_EPI_NONE);
+    GRL_REQUIRE(A && B && C, GRL_ERR_ARG, "grl_gemm_nn_noalloc: null argument");
+    const int64_t need = K * N * (int64_t)grl_dtype_size(in_dtype);
+    GRL_REQUIRE(need <= (int64_t)GRL_NN_SCRATCH_BYTES, GRL_ERR_SHAPE,
+                "grl_gemm_nn_noalloc: B (%lld x %lld, %lld bytes) exceeds the %u-byte static scratch; use grl_gemm_nn",
+                (long long)K, (long long)N, (long long)need, GRL_NN_SCRATCH_BYTES);
+    void* ws = nullptr;
+    rc = nn_scratch_address(c, &ws);
+    if (rc) return rc;
+    // the transpose overwrites every byte of the (N,K) image the GEMM reads, so nothing of the previous
+    // call's contents needs clearing
+    rc = grl_transpose2d(c, in_dtype, K, N, B, ws);   // (K,N) -> (N,K)
+    if (!rc) rc = grl_gemm_nt(c, in_dtype, out_dtype, M, N, K, A, ws, nullptr, C, GRL_EPI_NONE);
+    return rc;
+}

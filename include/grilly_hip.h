@@ -123,6 +123,17 @@ int grl_gemm_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N,
 int grl_gemm_nn(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
                 const void* A, const void* B, void* C, void* workspace);
 
+/* C = A.B with B (K,N) row-major, like grl_gemm_nn, but allocating nothing: no hipMalloc / hipFree, no pool
+ * request.  No counterpart in the reference; it is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid device allocation.  The transposed copy of B goes into
+ * a static device array of grl_gemm_nn_noalloc_max_bytes() = 32 MiB that every GPU the library runs on holds
+ * until the process ends (its address is looked up in grl_create); K*N*sizeof(in_dtype) beyond that returns
+ * GRL_ERR_SHAPE.  All calls on one GPU share the array: calls that overlap on one GPU (two contexts, i.e. two
+ * streams, of the same device) race, calls on one context are ordered by its stream. */
+int grl_gemm_nn_noalloc(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                        const void* A, const void* B, void* C);
+int64_t grl_gemm_nn_noalloc_max_bytes(void);
+
 /* grl_gemm_nt with every epilogue of the reference's fused-linear family: additionally
  * GRL_EPI_RELU (VulkanFNN.fused_linear_relu, backend/fnn.py:2125-2212, shaders/fused-linear-relu.glsl:40-68),
  * GRL_EPI_GCU (fused_linear_gcu, backend/fnn.py:2307-2383, shaders/fused-linear-gcu.glsl:43-75) and
