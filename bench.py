@@ -4,16 +4,22 @@ FFN 3072 GELU, fused QKV) at batch 128 x seq 512, bf16 storage with fp32 accumul
 MI355X.  A step = one full forward over one synthetic batch already resident in HBM.
 
 Prints one JSON line: encoder tokens/s, plus
-  roofline     -- the dominant kernel (the bf16 MFMA GEMM): algorithmic FLOPs per launch divided
+  roofline     -- the dominant kernel (the plain bf16 MFMA GEMM): algorithmic FLOPs per launch divided
                   by its average launch duration, measured here with HIP events on the library's
                   own stream, against the 2.5 PFLOP/s dense bf16 MFMA peak;
   kernels      -- the same measurement for every kernel of the layer (GEMMs and attention against
-                  the MFMA peak, LayerNorm against 8 TB/s HBM);
+                  the MFMA peak, LayerNorm against 8 TB/s HBM), each launched on the data the layer really
+                  hands it, each with a sampled check of the timed output buffer against the float64 closed form;
+  extra        -- outside the timed region: the fp32 forward of the same configuration, BASELINE configs[3]
+                  (SwiGLU MLP) and configs[4] (long causal attention with RoPE), each with flops, ms,
+                  fraction of the matrix peak and a sampled check of its own output buffers;
   cpu_baseline -- the C restatement of the reference shaders (oracle/oracle.c) timed on the host
-                  cores on a bounded sample (--cpu-sequences of the 128 sequences through all 12 layers).
+                  cores on a bounded sample (--cpu-sequences of the 128 sequences through all 12 layers);
+                  the GPU's hidden states of the same sequences are compared with its result;
+  cpu_baseline_blas -- what the reference's gemm() really executes on the host: numpy `@` (OpenBLAS) on the
+                  layer's four GEMM shapes, a bounded number of rows.
 """
 import argparse
-import ctypes
 import json
 import os
 import sys
@@ -27,15 +33,24 @@ sys.path.insert(0, ROOT)
 PEAK_BF16 = 2.5e15      # MI355X dense bf16 MFMA, FLOP/s
 PEAK_FP32 = 157.3e12
 PEAK_HBM = 8.0e12       # B/s
-
-# HBM bytes per launch of the plain bf16 GEMM kernel, mean over its three layer shapes at batch 128 x seq 512:
-# rocprofv3 --pmc FETCH_SIZE (x2, the factor a 1 GiB copy kernel calibrates) + --pmc WRITE_SIZE (x1) on
-# `bench.py --mode gemm`; summary in profiles/gemm_bf16_bert_shapes_hbm_traffic.md.  A profiler reading, not
-# something this script can measure itself, so it is reported only for exactly that workload.
-GEMM_TRAFFIC_BYTES = {("bf16", 128, 512): 617.2e6}
-
+TOL = {"bf16": 2e-2, "fp32": 1e-4}
 
 WARM = 5
+
+
+def gemm_traffic(dtype, B, S):
+    """HBM bytes per launch of the dominant kernel: a profiler reading (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE),
+    not something this script can measure itself, so it comes from the tracked record next to the profile
+    summary and is reported only for exactly the workload it was taken on."""
+    path = os.path.join(ROOT, "profiles", "gemm_bf16_bert_shapes_hbm_traffic.json")
+    try:
+        rec = json.load(open(path))
+    except (OSError, ValueError):
+        return None, None
+    k = rec.get("key", {})
+    if (k.get("dtype"), k.get("batch"), k.get("seq")) != (dtype, B, S):
+        return None, None
+    return rec.get("traffic_bytes_per_launch"), rec.get("measured_at_commit")
 
 
 def time_launches(core, fn, reps, warm=WARM):
@@ -49,32 +64,71 @@ def time_launches(core, fn, reps, warm=WARM):
     return core.timer_stop() / reps
 
 
-def kernel_table(backend, enc, B, S, reps, only=None):
-    """per-kernel average duration of one encoder layer's launches at the benchmark shape"""
+def download_rows(core, buf, row0, nrows, ncols, code):
+    """rows [row0, row0+nrows) of a device matrix with `ncols` columns -> float32 numpy"""
+    from grilly_amd import _lib as L
+    es = 2 if code == L.GRL_BF16 else 4
+    out = np.empty((nrows, ncols), np.float32)
+    n = nrows * ncols
+    src = buf.ptr + row0 * ncols * es
+    if code == L.GRL_BF16:
+        with core.alloc(n * 4) as tmp:
+            L.check(core.lib.grl_cast(core.ctx, L.GRL_BF16, L.GRL_F32, n, src, tmp.ptr), "cast")
+            L.check(core.lib.grl_d2h(core.ctx, out.ctypes.data, tmp.ptr, n * 4), "download")
+    else:
+        L.check(core.lib.grl_d2h(core.ctx, out.ctypes.data, src, n * 4), "download")
+    return out
+
+
+class _Ptr:
+    """a raw device address with the .ptr attribute of a DeviceBuffer (weights held in the layer structs)"""
+
+    def __init__(self, ptr):
+        self.ptr = ptr
+
+
+def gather_rows(core, buf, rows, ncols, code):
+    return np.concatenate([download_rows(core, buf, int(r), 1, ncols, code) for r in rows])
+
+
+def max_rel(y, ref):
+    ref = np.asarray(ref, np.float64)
+    return float(np.abs(np.asarray(y, np.float64) - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def kernel_table(backend, enc, B, S, reps, only=None, check=True):
+    """per-kernel average duration of one encoder layer's launches at the benchmark shape.  The buffers are
+    first filled by one untimed pass in data-flow order (QKV -> attention -> out-proj -> LayerNorm -> FFN1 -> FFN2),
+    so every timed launch reads what the layer really hands it; after timing, sampled rows of every output
+    buffer are compared with the float64 closed form of the same inputs (CPU leg, checker only)."""
     from grilly_amd import _lib as L
     cfg, c, lib, code = enc.cfg, backend.core, backend.core.lib, enc.code
     M, d, ff, H, D = B * S, cfg.d_model, cfg.d_ff, cfg.heads, cfg.head_dim
     es = 2 if code == L.GRL_BF16 else 4
+    dt = "bf16" if code == L.GRL_BF16 else "fp32"
     s = enc.layer_structs[0]
     qkv, attn, ffb = c.alloc(M * 3 * d * es), c.alloc(M * d * es), c.alloc(M * ff * es)
-    proj = c.alloc(M * d * es)
+    proj, x1, y2 = c.alloc(M * d * es), c.alloc(M * d * es), c.alloc(M * d * es)
     x = enc.x
     peak = PEAK_BF16 if code == L.GRL_BF16 else PEAK_FP32
     scale = 1.0 / np.sqrt(D)
+    f_qkv = lambda: lib.grl_gemm_nt(c.ctx, code, code, M, 3 * d, d, x.ptr, s.w_qkv, s.b_qkv, qkv.ptr, 0)
+    f_fa = lambda: lib.grl_fa2_fwd_strided(c.ctx, code, B, S, H, D, qkv.ptr, qkv.ptr + d * es, qkv.ptr + 2 * d * es,
+                                           None, attn.ptr, 3 * d, 3 * d, 3 * d, d, scale, 0, 0, 1e4, 1.0)
+    f_out = lambda: lib.grl_gemm_nt(c.ctx, code, code, M, d, d, attn.ptr, s.w_o, s.b_o, proj.ptr, 0)
+    f_ln = lambda: lib.grl_layernorm(c.ctx, code, M, d, x.ptr, proj.ptr, s.ln1_g, s.ln1_b, cfg.eps, x1.ptr)
+    f_ff1 = lambda: lib.grl_gemm_nt(c.ctx, code, code, M, ff, d, x1.ptr, s.w_ff1, s.b_ff1, ffb.ptr, 1)
+    f_ff2 = lambda: lib.grl_gemm_nt(c.ctx, code, code, M, d, ff, ffb.ptr, s.w_ff2, s.b_ff2, y2.ptr, 0)
+    for f in (f_qkv, f_fa, f_out, f_ln, f_ff1, f_ff2):       # data-flow order, untimed
+        L.check(f())
+    c.sync()
     runs = [
-        ("gemm_qkv", "gemm_nt", lambda: lib.grl_gemm_nt(c.ctx, code, code, M, 3 * d, d, x.ptr, s.w_qkv, s.b_qkv, qkv.ptr, 0),
-         2.0 * M * 3 * d * d, (M * d + 3 * d * d + M * 3 * d) * es),
-        ("gemm_out", "gemm_nt", lambda: lib.grl_gemm_nt(c.ctx, code, code, M, d, d, attn.ptr, s.w_o, s.b_o, proj.ptr, 0),
-         2.0 * M * d * d, (2 * M * d + d * d) * es),
-        ("gemm_ffn2", "gemm_nt", lambda: lib.grl_gemm_nt(c.ctx, code, code, M, d, ff, ffb.ptr, s.w_ff2, s.b_ff2, proj.ptr, 0),
-         2.0 * M * d * ff, (M * ff + d * ff + M * d) * es),
-        ("gemm_ffn1_gelu", "gemm_nt_gelu", lambda: lib.grl_gemm_nt(c.ctx, code, code, M, ff, d, x.ptr, s.w_ff1, s.b_ff1, ffb.ptr, 1),
-         2.0 * M * d * ff, (M * d + d * ff + M * ff) * es),
-        ("fa2_fwd", "fa2", lambda: lib.grl_fa2_fwd_strided(c.ctx, code, B, S, H, D, qkv.ptr, qkv.ptr + d * es, qkv.ptr + 2 * d * es,
-                                                           None, attn.ptr, 3 * d, 3 * d, 3 * d, d, scale, 0, 0, 1e4, 1.0),
-         4.0 * B * H * S * S * D, 4 * M * d * es),
-        ("layernorm_residual", "ln", lambda: lib.grl_layernorm(c.ctx, code, M, d, x.ptr, proj.ptr, s.ln1_g, s.ln1_b, cfg.eps, attn.ptr),
-         0.0, 3 * M * d * es),
+        ("gemm_qkv", "gemm_nt", f_qkv, 2.0 * M * 3 * d * d, (M * d + 3 * d * d + M * 3 * d) * es),
+        ("gemm_out", "gemm_nt", f_out, 2.0 * M * d * d, (2 * M * d + d * d) * es),
+        ("gemm_ffn2", "gemm_nt", f_ff2, 2.0 * M * d * ff, (M * ff + d * ff + M * d) * es),
+        ("gemm_ffn1_gelu", "gemm_nt_gelu", f_ff1, 2.0 * M * d * ff, (M * d + d * ff + M * ff) * es),
+        ("fa2_fwd", "fa2", f_fa, 4.0 * B * H * S * S * D, 4 * M * d * es),
+        ("layernorm_residual", "ln", f_ln, 0.0, 3 * M * d * es),
     ]
     out = {}
     for name, group, fn, flops, nbytes in runs:
@@ -88,30 +142,64 @@ def kernel_table(backend, enc, B, S, reps, only=None):
         rec["gbps"] = round(nbytes / ms / 1e6, 1)
         rec["frac_hbm"] = round(nbytes / (ms * 1e-3) / PEAK_HBM, 4)
         out[name] = rec
-    for b in (qkv, attn, ffb, proj):
+    if check:
+        from oracle import oracle_np as O          # checker only: the timed buffers against the float64 closed form
+        rng = np.random.default_rng(7)
+        rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 30)]))
+        dl = lambda ptr, n: download_rows(c, _Ptr(ptr), 0, 1, n, L.GRL_F32)[0]
+        wt = lambda ptr, r, k: download_rows(c, _Ptr(ptr), 0, r, k, code)
+
+        def gemm_err(a_buf, K, w_ptr, b_ptr, N, c_buf, epi):
+            a = gather_rows(c, a_buf, rows, K, code)
+            ref = O.truth_linear(a, wt(w_ptr, N, K), dl(b_ptr, N), epi)
+            return max_rel(gather_rows(c, c_buf, rows, N, code), ref)
+        errs = {"gemm_qkv": gemm_err(x, d, s.w_qkv, s.b_qkv, 3 * d, qkv, "none"),
+                "gemm_out": gemm_err(attn, d, s.w_o, s.b_o, d, proj, "none"),
+                "gemm_ffn1_gelu": gemm_err(x1, d, s.w_ff1, s.b_ff1, ff, ffb, "gelu"),
+                "gemm_ffn2": gemm_err(ffb, ff, s.w_ff2, s.b_ff2, d, y2, "none")}
+        b0 = int(rng.integers(0, B))
+        q3 = download_rows(c, qkv, b0 * S, S, 3 * d, code).reshape(1, S, 3, H, D)
+        at = download_rows(c, attn, b0 * S, S, d, code).reshape(1, S, H, D)
+        hs = [0, H - 1]
+        errs["fa2_fwd"] = max_rel(at[:, :, hs], O.truth_attention(q3[:, :, 0][:, :, hs], q3[:, :, 1][:, :, hs], q3[:, :, 2][:, :, hs]))
+        errs["layernorm_residual"] = max_rel(gather_rows(c, x1, rows, d, code),
+                                            O.truth_layernorm(gather_rows(c, x, rows, d, code), dl(s.ln1_g, d), dl(s.ln1_b, d), cfg.eps,
+                                                              residual=gather_rows(c, proj, rows, d, code)))
+        for k, e in errs.items():
+            if k in out:
+                out[k]["max_rel_vs_float64"] = float(f"{e:.3g}")
+                out[k]["within_tolerance"] = bool(e < TOL[dt])
+    for b in (qkv, attn, ffb, proj, x1, y2):
         b.free()
     return out
 
 
-def fill_normal(core, nbytes_elems, rng, std, code):
-    """device buffer of `nbytes_elems` elements ~N(0,std), tiled from a 4 Mi-element random block"""
+def fill_normal(core, n_elems, rng, std, code):
+    """device buffer of `n_elems` elements ~N(0,std), tiled from a 4 Mi-element random block; returns the
+    buffer and the host copy of the block (element i of the buffer is block[i % block.size], rounded to `code`)"""
     from grilly_amd import _lib as L
     es = 2 if code == L.GRL_BF16 else 4
     blk = (rng.standard_normal(1 << 22) * std).astype(np.float32)
     src = core.upload(blk, code)
-    dst = core.alloc(nbytes_elems * es)
+    dst = core.alloc(n_elems * es)
     off = 0
-    while off < nbytes_elems * es:
-        m = min(blk.size * es, nbytes_elems * es - off)
+    while off < n_elems * es:
+        m = min(blk.size * es, n_elems * es - off)
         L.check(core.lib.grl_d2d(core.ctx, dst.ptr + off, src.ptr, m))
         off += m
     core.sync()
     src.free()
-    return dst
+    return dst, blk
 
 
-def side_workload(backend, mode, seed, reps):
-    """the two single-operator configurations: long causal attention with RoPE, and the SwiGLU MLP"""
+def tiled(blk, start, n):
+    """elements [start, start+n) of the tiled buffer fill_normal made from blk"""
+    idx = (np.int64(start) + np.arange(n, dtype=np.int64)) % blk.size
+    return blk[idx]
+
+
+def side_workload(backend, mode, seed, reps, check=True):
+    """the single-operator configurations: long causal attention with RoPE, the SwiGLU MLP, and the pre-norm encoder"""
     from grilly_amd import _lib as L
     c, lib, code = backend.core, backend.core.lib, L.GRL_BF16
     rng = np.random.default_rng(seed)
@@ -131,49 +219,124 @@ def side_workload(backend, mode, seed, reps):
     if mode == "fa2_long":
         B, H, S, D = 4, 32, 8192, 128
         n = B * S * H * D
-        q, k, v = (fill_normal(c, n, rng, 1.0, code) for _ in range(3))
+        (q, qb), (k, kb), (v, vb) = (fill_normal(c, n, rng, 1.0, code) for _ in range(3))
         o = c.alloc(n * 2)
         fn = lambda: L.check(lib.grl_fa2_fwd(c.ctx, code, B, S, H, D, q.ptr, k.ptr, v.ptr, None, o.ptr,
                                              1.0 / np.sqrt(D), 1, L.ROPE_INTERLEAVED, 1e4, 1.0, None))
         ms = time_launches(c, fn, reps)
         flops = 4.0 * B * H * S * S * D * 0.5    # causal: half of the score matrix
-        return {"mode": mode, "workload": "BASELINE configs[4]: causal FA2 forward with RoPE, (B,S,H,D)=(4,8192,32,128), bf16",
-                "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_mfma": round(flops / (ms * 1e-3) / PEAK_BF16, 4),
-                "flops": flops, "includes": "cos/sin table kernel + K pre-rotation kernel + attention kernel (buffers from the caching pool)", "launches": reps + WARM}
+        res = {"mode": mode, "workload": "BASELINE configs[4]: causal FA2 forward with RoPE, (B,S,H,D)=(4,8192,32,128), bf16",
+               "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_mfma": round(flops / (ms * 1e-3) / PEAK_BF16, 4),
+               "flops": flops, "includes": "every kernel the entry point launches for this call (cos/sin table, rotation, attention)", "launches": reps + WARM}
+        if check:
+            from oracle import oracle_np as O      # checker only
+            worst = 0.0
+            for (b, h, i) in [(0, 0, 0), (1, 5, 127), (2, 17, 128), (3, 31, 4097), (0, 9, 8191), (1, 30, 2049)]:
+                row = lambda blk, s0, cnt: O.bf16_round(np.stack([tiled(blk, ((b * S + s) * H + h) * D, D) for s in range(s0, s0 + cnt)]))
+                qr = O.truth_rope(row(qb, i, 1).reshape(1, 1, 1, D), style="interleaved", position_ids=np.array([[i]]))[0, 0, 0]
+                kr = O.truth_rope(row(kb, 0, i + 1).reshape(1, i + 1, 1, D), style="interleaved")[0, :, 0]
+                sc = kr @ qr / np.sqrt(D)
+                pw = np.exp(sc - sc.max()); pw /= pw.sum()
+                ref = pw @ row(vb, 0, i + 1).astype(np.float64)
+                got = download_rows(c, o, (b * S + i) * H + h, 1, D, code)[0]
+                worst = max(worst, max_rel(got, ref))
+            res["max_rel_vs_float64"] = float(f"{worst:.3g}"); res["within_tolerance"] = bool(worst < TOL["bf16"])
+        for t in (q, k, v, o):
+            t.free()
+        return res
     M, Kd, F = 16384, 4096, 11008
-    x = fill_normal(c, M * Kd, rng, 1.0, code)
-    wg, wu = fill_normal(c, F * Kd, rng, 0.02, code), fill_normal(c, F * Kd, rng, 0.02, code)
-    wd = fill_normal(c, Kd * F, rng, 0.02, code)
+    x, xb = fill_normal(c, M * Kd, rng, 1.0, code)
+    (wg, wgb), (wu, wub) = fill_normal(c, F * Kd, rng, 0.02, code), fill_normal(c, F * Kd, rng, 0.02, code)
+    wd, wdb = fill_normal(c, Kd * F, rng, 0.02, code)
     h, y = c.alloc(M * F * 2), c.alloc(M * Kd * 2)
     f1 = lambda: L.check(lib.grl_swiglu_nt(c.ctx, code, code, M, F, Kd, x.ptr, wg.ptr, wu.ptr, None, None, h.ptr, None, None))
     f2 = lambda: L.check(lib.grl_gemm_nt(c.ctx, code, code, M, Kd, F, h.ptr, wd.ptr, None, y.ptr, 0))
     ms1, ms2 = time_launches(c, f1, reps), time_launches(c, f2, reps)
     fl1, fl2 = 4.0 * M * F * Kd, 2.0 * M * F * Kd
-    return {"mode": mode, "workload": "BASELINE configs[3]: X[16384,4096] . (W_g,W_u)[11008,4096]^T -> silu(up)*gate -> . W_d[4096,11008]^T, bf16",
-            "gate_up_swiglu": {"ms": round(ms1, 4), "tflops": round(fl1 / ms1 / 1e9, 1), "frac_mfma": round(fl1 / (ms1 * 1e-3) / PEAK_BF16, 4)},
-            "down": {"ms": round(ms2, 4), "tflops": round(fl2 / ms2 / 1e9, 1), "frac_mfma": round(fl2 / (ms2 * 1e-3) / PEAK_BF16, 4)},
-            "total_ms": round(ms1 + ms2, 4), "tflops": round((fl1 + fl2) / (ms1 + ms2) / 1e9, 1),
-            "frac_mfma": round((fl1 + fl2) / ((ms1 + ms2) * 1e-3) / PEAK_BF16, 4), "launches_each": reps + WARM}
+    res = {"mode": mode, "workload": "BASELINE configs[3]: X[16384,4096] . (W_g,W_u)[11008,4096]^T -> silu(up)*gate -> . W_d[4096,11008]^T, bf16",
+           "gate_up_swiglu": {"ms": round(ms1, 4), "tflops": round(fl1 / ms1 / 1e9, 1), "frac_mfma": round(fl1 / (ms1 * 1e-3) / PEAK_BF16, 4)},
+           "down": {"ms": round(ms2, 4), "tflops": round(fl2 / ms2 / 1e9, 1), "frac_mfma": round(fl2 / (ms2 * 1e-3) / PEAK_BF16, 4)},
+           "total_ms": round(ms1 + ms2, 4), "tflops": round((fl1 + fl2) / (ms1 + ms2) / 1e9, 1), "flops": fl1 + fl2,
+           "frac_mfma": round((fl1 + fl2) / ((ms1 + ms2) * 1e-3) / PEAK_BF16, 4), "launches_each": reps + WARM}
+    if check:
+        from oracle import oracle_np as O          # checker only
+        r2 = np.random.default_rng(11)
+        rows = np.unique(np.concatenate([[0, M - 1], r2.integers(0, M, 10)]))
+        cols = np.unique(np.concatenate([[0, F - 1], r2.integers(0, F, 254)]))
+        xs = O.bf16_round(np.stack([tiled(xb, int(r) * Kd, Kd) for r in rows])).astype(np.float64)
+        wgs = O.bf16_round(np.stack([tiled(wgb, int(n) * Kd, Kd) for n in cols])).astype(np.float64)
+        wus = O.bf16_round(np.stack([tiled(wub, int(n) * Kd, Kd) for n in cols])).astype(np.float64)
+        hrows = gather_rows(c, h, rows, F, code)
+        e1 = max_rel(hrows[:, cols], (xs @ wgs.T) * O.truth_silu(xs @ wus.T))
+        ocols = np.unique(np.concatenate([[0, Kd - 1], r2.integers(0, Kd, 126)]))
+        wds = O.bf16_round(np.stack([tiled(wdb, int(n) * F, F) for n in ocols])).astype(np.float64)
+        e2 = max_rel(gather_rows(c, y, rows, Kd, code)[:, ocols], hrows.astype(np.float64) @ wds.T)
+        res["gate_up_swiglu"]["max_rel_vs_float64"] = float(f"{e1:.3g}"); res["down"]["max_rel_vs_float64"] = float(f"{e2:.3g}")
+        res["within_tolerance"] = bool(e1 < TOL["bf16"] and e2 < TOL["bf16"])
+    for t in (x, wg, wu, wd, h, y):
+        t.free()
+    return res
 
 
-def cpu_baseline(cfg, weights, seed, nseq):
-    """C restatement of the reference shaders on the host cores: `nseq` sequences of the workload
-    (S=512 each) through embeddings + all layers.  tokens/s = nseq*512 / elapsed."""
+def cpu_baseline(cfg, weights, ids, nseq):
+    """C restatement of the reference shaders on the host cores: the first `nseq` sequences of the workload
+    (S=512 each) through embeddings + all layers.  tokens/s = nseq*512 / elapsed.  Returns the record and the
+    hidden states it computed (the checker for the GPU's hidden states of the same sequences)."""
     from oracle import oracle_np as O
     O.build()
     C = O.COracle()
-    rng = np.random.default_rng(seed)
-    S = 512
-    ids = rng.integers(0, cfg.vocab, (nseq, S))
+    S = ids.shape[1]
     t0 = time.perf_counter()
-    x = C.layernorm(C.embed(ids, weights["tok_emb"], weights["pos_emb"], weights["type_emb"]),
+    x = C.layernorm(C.embed(ids[:nseq], weights["tok_emb"], weights["pos_emb"], weights["type_emb"]),
                     weights["emb_ln_g"], weights["emb_ln_b"], cfg.eps)
     for lw in weights["layers"]:
         x = C.bert_layer(x, lw, None, cfg.heads, cfg.eps)
     dt = time.perf_counter() - t0
-    return {"value": round(nseq * S / dt, 2), "unit": "tokens/s", "cores": C.num_threads(), "kind": "port",
-            "sample": f"{nseq} of the 128 sequences x {S} tokens through embeddings + {cfg.layers} layers, fp32, "
-                      f"oracle/oracle.c (one-output-per-invocation shader loops, OpenMP over rows); {dt:.1f} s"}
+    rec = {"value": round(nseq * S / dt, 2), "unit": "tokens/s", "cores": C.num_threads(), "kind": "port",
+           "sample": f"{nseq} of the 128 sequences x {S} tokens through embeddings + {cfg.layers} layers, fp32, "
+                     f"oracle/oracle.c (one-output-per-invocation shader loops, OpenMP over rows); {dt:.1f} s"}
+    return rec, x
+
+
+def cpu_baseline_blas(cfg, S, rows=4096, budget_s=8.0):
+    """What the reference's gemm() executes on the host (backend/fnn.py:110-124): numpy `@`, fp32, on the four
+    GEMM shapes of one layer at `rows` rows; the encoder's other operators are not included, so the figure is
+    an upper bound for a numpy-backed reference forward."""
+    rng = np.random.default_rng(5)
+    d, ff = cfg.d_model, cfg.d_ff
+    shapes = [(d, 3 * d), (d, d), (d, ff), (ff, d)]
+    try:
+        import threadpoolctl
+        threads = max((p.get("num_threads", 1) for p in threadpoolctl.threadpool_info()), default=os.cpu_count())
+    except Exception:
+        threads = os.cpu_count()
+    per_layer = 0.0
+    t_all = time.perf_counter()
+    for K, N in shapes:
+        a = rng.standard_normal((rows, K)).astype(np.float32)
+        w = rng.standard_normal((K, N)).astype(np.float32)
+        a @ w
+        t0 = time.perf_counter(); reps = 0
+        while reps < 3 or (time.perf_counter() - t0 < budget_s / 8 and reps < 50):
+            a @ w; reps += 1
+        per_layer += (time.perf_counter() - t0) / reps
+    tok = rows / (per_layer * cfg.layers)
+    return {"value": round(tok, 1), "unit": "tokens/s", "cores": int(threads), "kind": "reference-blas",
+            "sample": f"numpy @ (OpenBLAS, fp32) on the four GEMMs of one layer at {rows} rows, x{cfg.layers} layers; attention, "
+                      f"LayerNorm and GELU excluded; {time.perf_counter() - t_all:.1f} s"}
+
+
+def timed_forward(backend, enc, steps, warmup):
+    for _ in range(warmup):
+        enc.launch(pool=True)
+    backend.core.sync()
+    t0 = time.perf_counter()
+    backend.core.timer_start()
+    for _ in range(steps):
+        enc.launch(pool=True)
+    ev_ms = backend.core.timer_stop()         # records the stop event and waits for it
+    backend.core.sync()
+    return time.perf_counter() - t0, ev_ms
 
 
 def main():
@@ -187,6 +350,7 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the fp32 forward and the two single-operator configurations")
     ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "kernels", "copy", "fa2_long", "swiglu_mlp", "prenorm_forward"],
                     help="forward: the benchmark; gemm / copy: only launch the dominant GEMM kernel at its three "
                          "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs); kernels: every kernel of "
@@ -218,7 +382,7 @@ def main():
         backend.cleanup()
         return
     if a.mode in ("fa2_long", "swiglu_mlp", "prenorm_forward"):
-        print(json.dumps(side_workload(backend, a.mode, seed, a.kernel_reps)))
+        print(json.dumps(side_workload(backend, a.mode, seed, a.kernel_reps, check=not a.no_cpu_baseline)))
         backend.cleanup()
         return
     weights = random_bert_weights(cfg, seed=seed)
@@ -230,24 +394,16 @@ def main():
 
     if a.mode in ("gemm", "kernels"):
         only = ("gemm_qkv", "gemm_out", "gemm_ffn2") if a.mode == "gemm" else None
-        kt = kernel_table(backend, enc, B, S, a.kernel_reps, only=only)
+        kt = kernel_table(backend, enc, B, S, a.kernel_reps, only=only, check=False)
         print(json.dumps({"mode": a.mode, "kernels": kt, "launches_each": a.kernel_reps + WARM}))
         backend.cleanup()
         return
 
-    for _ in range(a.warmup):
-        enc.launch(pool=True)
-    backend.core.sync()
-    t0 = time.perf_counter()
-    backend.core.timer_start()
-    for _ in range(a.steps):
-        enc.launch(pool=True)
-    ev_ms = backend.core.timer_stop()         # records the stop event and waits for it
-    backend.core.sync()
-    wall = time.perf_counter() - t0
+    wall, ev_ms = timed_forward(backend, enc, a.steps, a.warmup)
     ms_per_step = wall * 1e3 / a.steps
     tokens_per_s = B * S * a.steps / wall
     flops = enc.flops_per_forward(B, S)
+    peak = PEAK_BF16 if a.dtype == "bf16" else PEAK_FP32
 
     out = {
         "metric": "encoder tokens/s (BERT-base, L=512)", "value": round(tokens_per_s, 1), "unit": "tokens/s",
@@ -258,11 +414,14 @@ def main():
                    "batch": B, "seq_len": S, "tokens_per_step": B * S, "flops_per_step": flops},
         "event_ms_per_step": round(ev_ms / a.steps, 3),
         "model_tflops": round(flops / (ms_per_step * 1e-3) / 1e12, 1),
+        "model_frac_mfma": round(flops / (ms_per_step * 1e-3) / peak, 4),
         "device": info,
     }
-    peak = PEAK_BF16 if a.dtype == "bf16" else PEAK_FP32
+    nseq = min(a.cpu_sequences, B)
+    # hidden states of the first sequences after the timed steps (the pooled output is computed from them)
+    gpu_hidden = download_rows(backend.core, enc.x, 0, nseq * S, cfg.d_model, enc.code).reshape(nseq, S, cfg.d_model)
     if not a.no_kernels:
-        kt = kernel_table(backend, enc, B, S, a.kernel_reps)
+        kt = kernel_table(backend, enc, B, S, a.kernel_reps, check=not a.no_cpu_baseline)
         out["kernels"] = kt
         # dominant kernel = the plain (no activation) GEMM instantiation, launched three times per layer
         # (QKV, out-proj, FFN2): average FLOPs per launch over average duration per launch
@@ -270,15 +429,53 @@ def main():
         avg_flops = sum(r["flops"] for r in g) / 3
         avg_ms = sum(r["ms"] for r in g) / 3
         ach = avg_flops / (avg_ms * 1e-3) / 1e12
+        traffic, at_commit = gemm_traffic(a.dtype, B, S)
         out["roofline"] = {"kernel": "gemm_nt_dma_kernel<bf16,bf16,256,256,2,4,EPI_NONE>" if a.dtype == "bf16" else "gemm_nt_dma_kernel<f32,f32,256,256,2,4,EPI_NONE>",
                            "bound": "mfma", "achieved": round(ach, 1), "peak": peak / 1e12, "unit": "TFLOP/s",
                            "frac": round(ach * 1e12 / peak, 4),
-                           "traffic": GEMM_TRAFFIC_BYTES.get((a.dtype, B, S)),
+                           "traffic": traffic, "traffic_measured_at_commit": at_commit,
                            "algorithmic_bytes": sum(r["bytes"] for r in g) / 3,
                            "avg_launch_ms": round(avg_ms, 4), "flops_per_launch": avg_flops,
-                           "launches_per_step": 3 * cfg.layers}
+                           "launches_per_step": 3 * cfg.layers,
+                           "note": "launches timed back to back on the layer's real operands; inside the forward the same launches "
+                                   "run about 10 % longer (operands come from HBM): see profiles/encoder_forward_bert_base_bf16_kernel_stats.md"}
+    extra = {}
+    hidden32 = None
+    if not a.no_extra and a.dtype == "bf16":
+        enc.release_activations()
+        # fp32 leg of the same configuration (BASELINE configs[2], fp32 storage and true-fp32 matrix instructions)
+        enc32 = BertEncoder(backend, cfg, weights, dtype="fp32")
+        enc32.set_inputs(ids, None)
+        w32, _ = timed_forward(backend, enc32, 3, 1)
+        ms32 = w32 * 1e3 / 3
+        extra["fp32_forward"] = {"workload": "BASELINE configs[2] in fp32", "ms": round(ms32, 3), "tokens_per_s": round(B * S / ms32 * 1e3, 1),
+                                 "flops": flops, "tflops": round(flops / ms32 / 1e9, 1), "frac_mfma": round(flops / (ms32 * 1e-3) / PEAK_FP32, 4),
+                                 "peak": "fp32 MFMA 157.3 TFLOP/s", "steps": 3}
+        hidden32 = download_rows(backend.core, enc32.x, 0, nseq * S, cfg.d_model, enc32.code).reshape(nseq, S, cfg.d_model)
+        enc32.release_activations()
+        del enc32
+        backend.core.lib.grl_pool_trim(backend.core.ctx)
+        for mode in ("swiglu_mlp", "fa2_long"):
+            r = side_workload(backend, mode, seed, 10, check=not a.no_cpu_baseline)
+            r.pop("mode")
+            extra[mode] = r
+            backend.core.lib.grl_pool_trim(backend.core.ctx)
+        out["extra"] = extra
     if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, weights, seed, a.cpu_sequences)
+        rec, cpu_hidden = cpu_baseline(cfg, weights, ids, nseq)
+        # the CPU leg's result is also the checker for the forwards timed above (same token ids, same weights)
+        e16 = max_rel(gpu_hidden, cpu_hidden)
+        rec["gpu_forward_max_rel_vs_cpu"] = {a.dtype: float(f"{e16:.3g}")}
+        ok = e16 < (TOL[a.dtype] if a.dtype == "fp32" else 5e-2)      # bf16 storage against an unquantised fp32 run
+        if hidden32 is not None:
+            e32 = max_rel(hidden32, cpu_hidden)
+            rec["gpu_forward_max_rel_vs_cpu"]["fp32"] = float(f"{e32:.3g}")
+            ok = ok and e32 < TOL["fp32"]
+            extra["fp32_forward"]["max_rel_vs_cpu_port"] = float(f"{e32:.3g}")
+            extra["fp32_forward"]["within_tolerance"] = bool(e32 < TOL["fp32"])
+        rec["gpu_forward_within_tolerance"] = bool(ok)
+        out["cpu_baseline"] = rec
+        out["cpu_baseline_blas"] = cpu_baseline_blas(cfg, S)
     backend.cleanup()
     print(json.dumps(out))
 

@@ -78,8 +78,10 @@ def load_encoder_checkpoint(path):
         L_, dm, H, ff = hf["n_layers"], hf["dim"], hf["n_heads"], hf["hidden_dim"]
     else:
         L_, dm, H, ff = hf["num_hidden_layers"], hf["hidden_size"], hf["num_attention_heads"], hf["intermediate_size"]
+    # the embedding LayerNorm runs with the model's own eps (utils/vulkan_sentence_transformer.py:729-736: BERT and
+    # DistilBERT configurations say 1e-12), the layer norms with the reference's hard-coded 1e-5 (:1004, :1026)
     cfg = EncoderConfig(layers=L_, d_model=dm, heads=H, d_ff=ff, vocab=hf["vocab_size"],
-                        max_pos=hf["max_position_embeddings"])
+                        max_pos=hf["max_position_embeddings"], emb_eps=float(hf.get("layer_norm_eps", 1e-12)))
     tok = get("embeddings.word_embeddings.weight")
     pos = get("embeddings.position_embeddings.weight")
     typ = get("embeddings.token_type_embeddings.weight", optional=True)

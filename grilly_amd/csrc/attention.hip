@@ -696,7 +696,9 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
 template <int D, int QT, int NW, int NSTG, int KT, int OCC = (NW == 4 ? 2 : 1)>
 static int launch_fa16_cfg(grl_ctx* c, const Fa16Args& f, bool rope_q) {
     const int qb = 32 * QT * NW;
-    dim3 grid((unsigned)(((f.S + qb - 1) / qb) * f.H * f.B)), block(NW * 64);
+    const int64_t nwg = (int64_t)((f.S + qb - 1) / qb) * f.H * f.B;
+    GRL_REQUIRE(nwg < (1LL << 31), GRL_ERR_SHAPE, "attention: %lld workgroups exceed the grid limit", (long long)nwg);
+    dim3 grid((unsigned)nwg), block(NW * 64);
     if (f.mask) {
         if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
         else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);

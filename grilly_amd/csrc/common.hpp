@@ -16,7 +16,8 @@ struct grl_ctx {
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     hipDeviceProp_t prop{};
-    std::mutex mu;
+    std::mutex mu;          // guards the pool
+    std::mutex timer_mu;    // guards the event pair
     // caching pool: bucket size -> free blocks; live pointer -> bucket size
     std::map<size_t, std::vector<void*>> free_blocks;
     std::map<void*, size_t> live;
@@ -213,9 +214,11 @@ __device__ __forceinline__ float silu_plain(float x) {
 }
 // shaders/fused-linear-gelu.glsl:45-63 rewritten with tanh(u) = 2/(1+exp(-2u)) - 1:
 //   0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (c + 0.044715 c^3), c = clamp(x, +-50).
-// No clamp instruction is needed: beyond |x| = 50 (already from |x| > 7) the exponential saturates to
-// 0 / +inf, also when x*x overflows, which yields x and (-)0: the shader's rule for |x| > 50.
+// The +-50 clamp needs no instruction of its own: beyond |x| = 50 (already from |x| > 7) the exponential saturates
+// to 0 / +inf, also when x*x overflows, which yields x and (-)0: the shader's rule for |x| > 50.  Only x = -inf
+// would give (-inf)*0; the lower bound keeps that at -0 (the shader returns 0 there), +inf stays +inf.
 __device__ __forceinline__ float gelu_fast(float x) {
+    x = fmaxf(x, -3.0e38f);
     float e = x * (-2.302208198f + -0.10294324f * (x * x));     // -2u*log2(e)
     return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e));
 }

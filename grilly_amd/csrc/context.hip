@@ -204,11 +204,13 @@ extern "C" int grl_sync(grl_ctx* c) {
 
 extern "C" int grl_timer_start(grl_ctx* c) {
     GRL_REQUIRE(c, GRL_ERR_ARG, "grl_timer_start: null context");
+    std::lock_guard<std::mutex> lk(c->timer_mu);      // one event pair per context: calls are serialised, timings are not nestable
     GRL_CHECK_HIP(hipEventRecord(c->ev0, c->stream));
     return GRL_OK;
 }
 extern "C" int grl_timer_stop(grl_ctx* c, float* ms) {
     GRL_REQUIRE(c && ms, GRL_ERR_ARG, "grl_timer_stop: null argument");
+    std::lock_guard<std::mutex> lk(c->timer_mu);
     GRL_CHECK_HIP(hipEventRecord(c->ev1, c->stream));
     GRL_CHECK_HIP(hipEventSynchronize(c->ev1));
     GRL_CHECK_HIP(hipEventElapsedTime(ms, c->ev0, c->ev1));

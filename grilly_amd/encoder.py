@@ -26,10 +26,15 @@ class EncoderConfig:
     vocab: int = 30522
     max_pos: int = 512
     eps: float = 1e-5          # the reference hard-codes 1e-5 in the layer LayerNorms (:1004, :1026)
+    emb_eps: float = None      # embedding LayerNorm: the checkpoint's own eps in the reference (:729-736); None = eps
 
     @property
     def head_dim(self):
         return self.d_model // self.heads
+
+    @property
+    def embedding_eps(self):
+        return self.eps if self.emb_eps is None else self.emb_eps
 
 
 BERT_BASE = EncoderConfig()
@@ -133,7 +138,7 @@ class BertEncoder:
         L.check(lib.grl_embed(c.ctx, self.code, B, S, cfg.d_model, cfg.vocab, self.ids.ptr, self.tok.ptr,
                               self.pos.ptr, self.typ.ptr, self.x.ptr), "embed")
         L.check(lib.grl_layernorm(c.ctx, self.code, B * S, cfg.d_model, self.x.ptr, None, self.emb_g.ptr,
-                                  self.emb_b.ptr, cfg.eps, self.x.ptr), "embedding layernorm")
+                                  self.emb_b.ptr, cfg.embedding_eps, self.x.ptr), "embedding layernorm")
         for s in self.layer_structs:
             L.check(lib.grl_bert_layer_fwd(c.ctx, self.code, B, S, cfg.heads, cfg.head_dim, cfg.d_ff, ctypes.byref(s),
                                            mask, cfg.eps, self.x.ptr, self.ws.ptr), "bert_layer_fwd")

@@ -99,7 +99,9 @@ int grl_memset(grl_ctx* ctx, void* dst_dev, int byte, size_t bytes);
 int grl_sync(grl_ctx* ctx);
 
 /* HIP-event stopwatch on the context stream (there is no counterpart in the reference,
- * which times whole numpy->numpy calls with time.perf_counter). */
+ * which times whole numpy->numpy calls with time.perf_counter).  A context holds one event pair: one timing
+ * at a time; calls from several threads are serialised but share the pair, so concurrent timings overwrite
+ * each other's start. */
 int grl_timer_start(grl_ctx* ctx);
 int grl_timer_stop(grl_ctx* ctx, float* elapsed_ms);   /* synchronises */
 

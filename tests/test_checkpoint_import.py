@@ -4,6 +4,7 @@ import os
 
 import numpy as np
 import pytest
+from dataclasses import replace as dataclasses_replace
 
 from grilly_amd.checkpoint import load_encoder_checkpoint
 from grilly_amd.encoder import EncoderConfig, random_bert_weights
@@ -51,7 +52,7 @@ def same(a, b):
 def write_config(d, distil=False):
     hf = ({"n_layers": 2, "dim": 64, "n_heads": 2, "hidden_dim": 128} if distil else
           {"num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 2, "intermediate_size": 128, "hidden_act": "gelu"})
-    hf.update({"vocab_size": 100, "max_position_embeddings": 32})
+    hf.update({"vocab_size": 100, "max_position_embeddings": 32, "layer_norm_eps": 1e-12})
     with open(os.path.join(d, "config.json"), "w") as f:
         json.dump(hf, f)
 
@@ -62,7 +63,9 @@ def test_bert_safetensors_roundtrip(tmp_path):
     write_config(tmp_path)
     save_file(bert_state(w), str(tmp_path / "model.safetensors"))
     cfg, got = load_encoder_checkpoint(str(tmp_path))
-    assert cfg == CFG
+    import dataclasses
+    assert cfg == dataclasses.replace(CFG, emb_eps=1e-12)      # the embedding LayerNorm keeps the checkpoint's own eps
+    assert cfg.embedding_eps == 1e-12 and cfg.eps == 1e-5 and CFG.embedding_eps == CFG.eps
     same(got, w)
 
 
@@ -74,7 +77,9 @@ def test_sentence_transformers_layout_and_torch_bin(tmp_path):
     write_config(sub)
     torch.save({k: torch.from_numpy(v) for k, v in bert_state(w, prefix="").items()}, str(sub / "pytorch_model.bin"))
     cfg, got = load_encoder_checkpoint(str(tmp_path))
-    assert cfg == CFG
+    import dataclasses
+    assert cfg == dataclasses.replace(CFG, emb_eps=1e-12)      # the embedding LayerNorm keeps the checkpoint's own eps
+    assert cfg.embedding_eps == 1e-12 and cfg.eps == 1e-5 and CFG.embedding_eps == CFG.eps
     same(got, w)
 
 
@@ -96,7 +101,9 @@ def test_distilbert_names(tmp_path):
     write_config(tmp_path, distil=True)
     save_file({k: np.ascontiguousarray(v) for k, v in sd.items()}, str(tmp_path / "model.safetensors"))
     cfg, got = load_encoder_checkpoint(str(tmp_path))
-    assert cfg == CFG
+    import dataclasses
+    assert cfg == dataclasses.replace(CFG, emb_eps=1e-12)      # the embedding LayerNorm keeps the checkpoint's own eps
+    assert cfg.embedding_eps == 1e-12 and cfg.eps == 1e-5 and CFG.embedding_eps == CFG.eps
     same(got, w)
 
 
@@ -123,15 +130,25 @@ def test_imported_checkpoint_runs_like_the_oracle(tmp_path, backend, corc):
     from grilly_amd import BertEncoder
     from oracle import oracle_np as O
     w = noisy_weights(5)
+    # small embeddings (variance ~1e-7 per row): the embedding LayerNorm's eps = 1e-12 of the checkpoint
+    # (reference utils/vulkan_sentence_transformer.py:729-736) and the layers' 1e-5 give visibly different rows
+    for k in ("tok_emb", "pos_emb", "type_emb"):
+        w[k] = (w[k] * 1e-2).astype(np.float32)
     write_config(tmp_path)
     save_file(bert_state(w), str(tmp_path / "model.safetensors"))
     cfg, got = load_encoder_checkpoint(str(tmp_path))
+    assert cfg.embedding_eps == 1e-12
     rng = np.random.default_rng(6)
     ids = rng.integers(0, cfg.vocab, (3, 20))
     mask = (np.arange(20)[None] < np.array([20, 9, 14])[:, None]).astype(np.float32)
     enc = BertEncoder(backend, cfg, got, dtype="fp32")
     pooled = enc.forward(ids, mask)
-    x = corc.layernorm(corc.embed(ids, w["tok_emb"], w["pos_emb"], w["type_emb"]), w["emb_ln_g"], w["emb_ln_b"], cfg.eps)
+    emb = corc.embed(ids, w["tok_emb"], w["pos_emb"], w["type_emb"])
+    x = corc.layernorm(emb, w["emb_ln_g"], w["emb_ln_b"], cfg.embedding_eps)
+    wrong = corc.layernorm(emb, w["emb_ln_g"], w["emb_ln_b"], cfg.eps)
+    assert O.max_rel(wrong, x) > 0.5                       # the two eps values are told apart by this input
+    h0 = BertEncoder(backend, dataclasses_replace(cfg, layers=0), dict(got, layers=[]), dtype="fp32").forward(ids, mask, pool=False)
+    assert O.max_rel(h0, x) < 1e-4
     for lw in w["layers"]:
         x = corc.bert_layer(x, lw, mask, cfg.heads, cfg.eps)
     assert O.max_rel(pooled, corc.mean_pool(x, mask)) < 1e-4
