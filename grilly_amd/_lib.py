@@ -71,6 +71,9 @@ SIGNATURES = {
     "grl_gelu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),
     "grl_silu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),
     "grl_relu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),
+    "grl_gcu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),
+    "grl_roswish": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p, c_float, c_float]),
+    "grl_softmax": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_void_p]),
     "grl_swiglu_act": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_void_p]),
     "grl_embed": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "grl_mean_pool": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_int]),

@@ -59,6 +59,49 @@ class HipAttention:
                 if b is not None:
                     b.free()
 
+    def attention_with_weights(self, queries, keys, values, scale=None, mask=None):
+        """Attention that also returns the softmax weights, for key / value sequences of any length: queries
+        (B,Sq,H,D), keys and values (B,Sk,H,D), optional key keep-mask (B,Sk) -> (output (B,Sq,H,D), weights
+        (B,H,Sq,Sk)).  What the reference's MultiheadAttention builds from separate score / softmax / output steps
+        (nn/modules.py:1131-1216); here: one score GEMM and one output GEMM per (batch, head) on device-resident
+        operands, one softmax kernel over all rows, fp32.  The fused kernel (flash_attention2) never forms the
+        weights and is the fast path when they are not needed."""
+        q, k, v = (np.asarray(t, dtype=np.float32) for t in (queries, keys, values))
+        if q.ndim != 4 or k.ndim != 4 or v.shape != k.shape or q.shape[0] != k.shape[0] or q.shape[2:] != k.shape[2:]:
+            raise ValueError("expected queries (B,Sq,H,D) and keys / values (B,Sk,H,D)")
+        B, Sq, H, D = q.shape
+        Sk = k.shape[1]
+        if scale is None:
+            scale = 1.0 / np.sqrt(D)
+        bias = None
+        if mask is not None:
+            m = np.asarray(mask, dtype=np.float32)
+            if m.shape != (B, Sk):
+                raise ValueError(f"mask must be (batch, key_len) = {(B, Sk)}, got {m.shape}")
+            bias = (m - np.float32(1.0)) * np.float32(1e9)
+        if q.size == 0 or Sk == 0:
+            return np.zeros((B, Sq, H, D), np.float32), np.zeros((B, H, Sq, Sk), np.float32)
+        c, code = self.core, L.GRL_F32
+        dq = c.upload(np.ascontiguousarray(q.transpose(0, 2, 1, 3)) * np.float32(scale))      # (B,H,Sq,D)
+        dk = c.upload(np.ascontiguousarray(k.transpose(0, 2, 1, 3)))                           # (B,H,Sk,D)
+        dvt = c.upload(np.ascontiguousarray(v.transpose(0, 2, 3, 1)))                          # (B,H,D,Sk)
+        db = c.upload(bias) if bias is not None else None
+        dsc, dw, do = c.alloc(B * H * Sq * Sk * 4), c.alloc(B * H * Sq * Sk * 4), c.alloc(B * H * Sq * D * 4)
+        try:
+            for bh in range(B * H):
+                L.check(c.lib.grl_gemm_nt(c.ctx, code, code, Sq, Sk, D, dq.ptr + bh * Sq * D * 4, dk.ptr + bh * Sk * D * 4,
+                                          db.ptr + (bh // H) * Sk * 4 if db else None, dsc.ptr + bh * Sq * Sk * 4, L.EPI_NONE), "scores")
+            L.check(c.lib.grl_softmax(c.ctx, code, B * H * Sq, Sk, dsc.ptr, dw.ptr), "softmax")
+            for bh in range(B * H):
+                L.check(c.lib.grl_gemm_nt(c.ctx, code, code, Sq, D, Sk, dw.ptr + bh * Sq * Sk * 4, dvt.ptr + bh * D * Sk * 4,
+                                          None, do.ptr + bh * Sq * D * 4, L.EPI_NONE), "weights x values")
+            out = c.download(do, (B, H, Sq, D)).transpose(0, 2, 1, 3)
+            return np.ascontiguousarray(out), c.download(dw, (B, H, Sq, Sk))
+        finally:
+            for t in (dq, dk, dvt, db, dsc, dw, do):
+                if t is not None:
+                    t.free()
+
     def flash_attention2(self, queries, keys, values, num_heads, head_dim, tile_size_q=64, tile_size_k=64,
                          scale=None, mask=None, causal=False, dtype="fp32", layout="bshd"):
         """tile_size_q / tile_size_k are accepted for call compatibility; the kernel's tiling is fixed."""

@@ -37,6 +37,9 @@ class HipCompute:
     def activation_silu(self, *a, **k): return self.fnn.activation_silu(*a, **k)
     def activation_relu(self, *a, **k): return self.fnn.activation_relu(*a, **k)
     def activation_swiglu(self, *a, **k): return self.fnn.activation_swiglu(*a, **k)
+    def activation_gcu(self, *a, **k): return self.fnn.activation_gcu(*a, **k)
+    def activation_roswish(self, *a, **k): return self.fnn.activation_roswish(*a, **k)
+    def activation_softmax(self, *a, **k): return self.fnn.activation_softmax(*a, **k)
     def fused_linear_gelu(self, *a, **k): return self.fnn.fused_linear_gelu(*a, **k)
     def fused_linear_silu(self, *a, **k): return self.fnn.fused_linear_silu(*a, **k)
     def fused_swiglu(self, *a, **k): return self.fnn.fused_swiglu(*a, **k)

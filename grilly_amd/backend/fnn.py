@@ -271,14 +271,14 @@ class HipFNN:
             for t in (dx, dg, db, dy):
                 t.free()
 
-    def _unary(self, fn, x, dtype, what):
+    def _unary(self, fn, x, dtype, what, *params):
         code = dtype_code(dtype)
         x = np.asarray(x)
         c = self.core
         dx = c.upload(x, code)
         dy = c.alloc(max(x.size, 1) * (2 if code == L.GRL_BF16 else 4))
         try:
-            L.check(fn(c.ctx, code, x.size, dx.ptr, dy.ptr), what)
+            L.check(fn(c.ctx, code, x.size, dx.ptr, dy.ptr, *params), what)
             return c.download(dy, x.shape, code)
         finally:
             dx.free(); dy.free()
@@ -298,22 +298,52 @@ class HipFNN:
         finally:
             da.free(); db.free(); dy.free()
 
-    def activation_gelu(self, x, dtype="fp32"):
+    # the activations take the reference's argument name `input_data` (backend/fnn.py:232, 285, 344, 393, 442, 499, 574)
+    def activation_gelu(self, input_data, dtype="fp32"):
         """Reference backend/fnn.py:285-342 (tanh form with the +-50 rule)."""
-        return self._unary(self.core.lib.grl_gelu, x, dtype, "gelu")
+        return self._unary(self.core.lib.grl_gelu, input_data, dtype, "gelu")
 
-    def activation_silu(self, x, dtype="fp32"):
+    def activation_silu(self, input_data, dtype="fp32"):
         """Reference backend/fnn.py:344-391."""
-        return self._unary(self.core.lib.grl_silu, x, dtype, "silu")
+        return self._unary(self.core.lib.grl_silu, input_data, dtype, "silu")
 
-    def activation_relu(self, x, dtype="fp32"):
+    def activation_relu(self, input_data, dtype="fp32"):
         """Reference backend/fnn.py:232-283."""
-        return self._unary(self.core.lib.grl_relu, x, dtype, "relu")
+        return self._unary(self.core.lib.grl_relu, input_data, dtype, "relu")
 
-    def activation_swiglu(self, x, dtype="fp32"):
+    def activation_gcu(self, input_data, dtype="fp32"):
+        """x*cos(x) (reference backend/fnn.py:393-440)."""
+        return self._unary(self.core.lib.grl_gcu, input_data, dtype, "gcu")
+
+    def activation_roswish(self, input_data, alpha=1.0, beta=1.0, dtype="fp32"):
+        """(x+alpha)*sigmoid(beta*x) - alpha/2 (reference backend/fnn.py:442-497)."""
+        return self._unary(self.core.lib.grl_roswish, input_data, dtype, "roswish", float(alpha), float(beta))
+
+    def activation_softmax(self, input_data, axis=-1, dtype="fp32"):
+        """exp(x - max) / sum over `axis` (reference backend/fnn.py:574-700; its shader normalises the last
+        dimension, other axes are moved there and back)."""
+        code = dtype_code(dtype)
+        x = np.asarray(input_data, dtype=np.float32)
+        if x.ndim == 0:
+            raise ValueError("activation_softmax needs at least one dimension")
+        xm = np.moveaxis(x, axis, -1)
+        F = xm.shape[-1]
+        if F == 0:
+            return np.empty(x.shape, np.float32)
+        rows = xm.size // F
+        c = self.core
+        dx = c.upload(xm, code)
+        dy = c.alloc(max(xm.size, 1) * (2 if code == L.GRL_BF16 else 4))
+        try:
+            L.check(c.lib.grl_softmax(c.ctx, code, rows, F, dx.ptr, dy.ptr), "softmax")
+            return np.ascontiguousarray(np.moveaxis(c.download(dy, xm.shape, code), -1, axis))
+        finally:
+            dx.free(); dy.free()
+
+    def activation_swiglu(self, input_data, dtype="fp32"):
         """Last dim 2h -> h: x1 * silu(x2) (reference backend/fnn.py:499-572); any rank >= 1."""
         code = dtype_code(dtype)
-        x = np.asarray(x)
+        x = np.asarray(input_data)
         if x.ndim < 1 or x.shape[-1] % 2:
             raise ValueError("activation_swiglu needs an even last dimension")
         h = x.shape[-1] // 2

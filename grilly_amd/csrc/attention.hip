@@ -22,9 +22,10 @@
 #include <algorithm>
 #include <cstdlib>
 
-int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling);
 int grl_rope_apply_table(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
                          void* y, const float* table);
+int grl_rope_half_apply_table(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
+                              void* y, const float* table);
 int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int64_t D, const void* x, int64_t x_stride,
                      const int32_t* position_ids, void* y, int style, float rope_base, float rope_scaling);
 
@@ -350,7 +351,9 @@ template <int IPT, int MAXT> __device__ __forceinline__ void wait_tiles_outstand
     }
 }
 
-template <int D, bool ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK, int KT, int OCC = (NW == 4 ? 2 : 1)>
+// ROPE_Q: rotation applied to the query rows as they are loaded: 0 none, 1 interleaved pairs (2p, 2p+1), 2 the
+// (d, d+D/2) pairing (both halves of a pair sit in chunks this lane loads itself)
+template <int D, int ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK, int KT, int OCC = (NW == 4 ? 2 : 1)>
 __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     // QT = 32-query MFMA tiles per wave (every K / V fragment read from LDS feeds QT MFMAs),
     // NW waves per workgroup, NSTG-deep ring of 64-key K/V tiles in LDS (NSTG-1 tiles in flight).
@@ -469,17 +472,40 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     for (int t = 0; t < QT; ++t) {
         const int qi = qw0 + 32 * t + li;
         const int qc = qi < S ? qi : S - 1;
+        if constexpr (ROPE_Q == 2) {
+            // chunk c = 2s+lg holds dims 8c .. 8c+7; its partner for the (d, d+D/2) pairing is chunk c + NCH/2,
+            // i.e. slab s + NS/2 of this same lane.  Table row qc holds {cos, sin} of pair d at [d], d < D/2.
+            static_assert(NS % 2 == 0, "the two halves of the head dim split the slabs evenly");
+#pragma unroll
+            for (int s = 0; s < NS / 2; ++s) {
+                const int c = 2 * s + lg;
+                const u32x4 lo = *(const u32x4*)(Qg + (int64_t)qc * p.q_stride + c * 8);
+                const u32x4 hi = *(const u32x4*)(Qg + (int64_t)qc * p.q_stride + (c + NCH / 2) * 8);
+                const float2* cs = p.rope + (int64_t)qc * (D / 2) + c * 8;
+                u32x4 olo, ohi;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float2 c0 = cs[2 * i], c1 = cs[2 * i + 1];
+                    const float a0 = bf16lo(lo[i]), a1 = bf16hi(lo[i]), b0 = bf16lo(hi[i]), b1 = bf16hi(hi[i]);
+                    olo[i] = pack_bf16x2((a0 * c0.x - b0 * c0.y) * c2, (a1 * c1.x - b1 * c1.y) * c2);
+                    ohi[i] = pack_bf16x2((b0 * c0.x + a0 * c0.y) * c2, (b1 * c1.x + a1 * c1.y) * c2);
+                }
+                qf[t][s] = olo;
+                qf[t][s + NS / 2] = ohi;
+            }
+        } else {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             const int c = 2 * s + lg;
             u32x4 v = *(const u32x4*)(Qg + (int64_t)qc * p.q_stride + c * 8);
             // queries carry scale*log2(e): the matrix core then delivers scores in the base-2 softmax domain
             float2 cs[4];
-            if (ROPE_Q) {
+            if (ROPE_Q == 1) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) cs[i] = p.rope[(int64_t)qc * (D / 2) + c * 4 + i];
             }
-            qf[t][s] = scale_chunk_bf16<ROPE_Q>(v, cs, c2);
+            qf[t][s] = scale_chunk_bf16<ROPE_Q == 1>(v, cs, c2);
+        }
         }
     }
 
@@ -694,24 +720,26 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
 }
 
 template <int D, int QT, int NW, int NSTG, int KT, int OCC = (NW == 4 ? 2 : 1)>
-static int launch_fa16_cfg(grl_ctx* c, const Fa16Args& f, bool rope_q) {
+static int launch_fa16_cfg(grl_ctx* c, const Fa16Args& f, int rope_q) {
     const int qb = 32 * QT * NW;
     const int64_t nwg = (int64_t)((f.S + qb - 1) / qb) * f.H * f.B;
     GRL_REQUIRE(nwg < (1LL << 31), GRL_ERR_SHAPE, "attention: %lld workgroups exceed the grid limit", (long long)nwg);
     dim3 grid((unsigned)nwg), block(NW * 64);
     if (f.mask) {
-        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
-        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
+        if (rope_q == 2) hipLaunchKernelGGL((fa2_bf16_kernel<D, 2, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
+        else if (rope_q == 1) hipLaunchKernelGGL((fa2_bf16_kernel<D, 1, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, 0, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
     } else {
-        if (rope_q) hipLaunchKernelGGL((fa2_bf16_kernel<D, true, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
-        else hipLaunchKernelGGL((fa2_bf16_kernel<D, false, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
+        if (rope_q == 2) hipLaunchKernelGGL((fa2_bf16_kernel<D, 2, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
+        else if (rope_q == 1) hipLaunchKernelGGL((fa2_bf16_kernel<D, 1, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, 0, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
     }
     GRL_CHECK_LAUNCH();
     return GRL_OK;
 }
 
 template <int D>
-static int launch_fa16(grl_ctx* c, const FaArgs& a, bool rope_q) {
+static int launch_fa16(grl_ctx* c, const FaArgs& a, int rope_q) {
     Fa16Args f{};
     f.Q = (const uint16_t*)a.Q; f.K = (const uint16_t*)a.K; f.V = (const uint16_t*)a.V;
     f.mask = a.mask; f.O = (uint16_t*)a.O; f.rope = a.rope;
@@ -750,6 +778,144 @@ static int launch_fa(grl_ctx* c, FaArgs& a, bool rope) {
     return GRL_OK;
 }
 
+// ---- head dims the MFMA kernels have no instantiation for ------------------------------------------
+// (b,s,h) rows of D values -> dense rows of DP >= D values, zero filled (and back): a head dim below 128 that is
+// not 32 / 64 / 128, or operands that are not 16-byte granular, run the MFMA kernels on zero-padded copies
+// (zero columns add nothing to q.k, and the padded output columns are dropped).
+template <typename T>
+__global__ __launch_bounds__(256) void pad_heads_kernel(const T* src, int64_t src_stride, T* dst, int64_t rows, int H, int D, int DP) {
+    const int64_t total = rows * DP, step = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int d = (int)(i % DP);
+        const int64_t row = i / DP, bs = row / H;
+        const int h = (int)(row - bs * H);
+        dst[i] = d < D ? src[bs * src_stride + (int64_t)h * D + d] : (T)0;
+    }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void unpad_heads_kernel(const T* src, T* dst, int64_t dst_stride, int64_t rows, int H, int D, int DP) {
+    const int64_t total = rows * D, step = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int d = (int)(i % D);
+        const int64_t row = i / D, bs = row / H;
+        const int h = (int)(row - bs * H);
+        dst[bs * dst_stride + (int64_t)h * D + d] = src[row * DP + d];
+    }
+}
+
+// Head dims above 128: one wave per query, lanes split the head dim, keys one after the other with the online
+// softmax (same constants as the MFMA kernels).  Correct for any D up to 64*NAIVE_MAX; not a fast path.
+constexpr int NAIVE_MAX = 16;
+template <typename T>
+__global__ __launch_bounds__(256) void fa2_naive_kernel(FaArgs p, int D) {
+    const int lane = threadIdx.x & 63;
+    const int64_t qid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);          // (b, h, i) flat, i fastest
+    const int64_t total = (int64_t)p.B * p.H * p.S;
+    if (qid >= total) return;
+    const int S = p.S, i = (int)(qid % S), h = (int)((qid / S) % p.H), b = (int)(qid / ((int64_t)S * p.H));
+    const T* q = (const T*)p.Q + ((int64_t)b * S + i) * p.q_stride + (int64_t)h * D;
+    float qv[NAIVE_MAX], o[NAIVE_MAX];
+#pragma unroll
+    for (int t = 0; t < NAIVE_MAX; ++t) {
+        const int d = lane + 64 * t;
+        qv[t] = d < D ? elem<T>::ld(q + d) : 0.f;
+        o[t] = 0.f;
+    }
+    float m = -1e10f, l = 0.f;
+    const int last = p.causal ? i : S - 1;
+    for (int j = 0; j <= last; ++j) {
+        const T* k = (const T*)p.K + ((int64_t)b * S + j) * p.k_stride + (int64_t)h * D;
+        const T* v = (const T*)p.V + ((int64_t)b * S + j) * p.v_stride + (int64_t)h * D;
+        float dot = 0.f;
+#pragma unroll
+        for (int t = 0; t < NAIVE_MAX; ++t) {
+            const int d = lane + 64 * t;
+            if (d < D) dot += qv[t] * elem<T>::ld(k + d);
+        }
+        dot = group_sum<64>(dot);
+        float sc = dot * p.scale;
+        if (p.mask) sc += (p.mask[(int64_t)b * S + j] - 1.0f) * 1e9f;
+        const float mn = fmaxf(m, sc);
+        const float alpha = __expf(m - mn), pw = __expf(sc - mn);
+        l = l * alpha + pw;
+        m = mn;
+#pragma unroll
+        for (int t = 0; t < NAIVE_MAX; ++t) {
+            const int d = lane + 64 * t;
+            if (d < D) o[t] = o[t] * alpha + pw * elem<T>::ld(v + d);
+        }
+    }
+    const float inv = 1.0f / fmaxf(l, 1e-10f);
+    T* out = (T*)p.O + ((int64_t)b * S + i) * p.o_stride + (int64_t)h * D;
+#pragma unroll
+    for (int t = 0; t < NAIVE_MAX; ++t) {
+        const int d = lane + 64 * t;
+        if (d < D) elem<T>::st(out + d, o[t] * inv);
+    }
+}
+
+static unsigned fa_ew_grid(int64_t n) {
+    int64_t g = (n + 255) / 256;
+    return (unsigned)(g < 1 ? 1 : (g > 8192 ? 8192 : g));
+}
+
+static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                      const void* Q, const void* K, const void* V, const float* mask, void* O,
+                      int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                      float scale, int causal, int rope, float rope_base, float rope_scaling, void* workspace);
+
+// Any head dim from 1 to 64*NAIVE_MAX and any alignment (reference backend/attention.py:403-410 reshapes with
+// whatever head_dim it is given): up to 128 through zero-padded copies and the MFMA kernels, above through the
+// one-wave-per-query kernel.  RoPE (even head dims up to 128) is applied to dense copies first.
+static int fa2_generic(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                       const void* Q, const void* K, const void* V, const float* mask, void* O,
+                       int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                       float scale, int causal, int rope, float rope_base, float rope_scaling) {
+    const int64_t es = (int64_t)grl_dtype_size(dtype), rows = B * S * H;
+    if (D > 128) {
+        GRL_REQUIRE(rope == GRL_ROPE_NONE, GRL_ERR_SHAPE, "%s: RoPE needs head_dim <= 128 (got %lld)", who, (long long)D);
+        GRL_REQUIRE((rows + 3) / 4 < (1LL << 31), GRL_ERR_SHAPE, "%s: too many queries", who);
+        FaArgs a{};
+        a.Q = Q; a.K = K; a.V = V; a.mask = mask; a.O = O;
+        a.B = (int)B; a.S = (int)S; a.H = (int)H; a.scale = scale; a.causal = causal ? 1 : 0;
+        a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.o_stride = o_stride;
+        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+        if (dtype == GRL_F32) hipLaunchKernelGGL(fa2_naive_kernel<float>, grid, block, 0, c->stream, a, (int)D);
+        else hipLaunchKernelGGL(fa2_naive_kernel<uint16_t>, grid, block, 0, c->stream, a, (int)D);
+        GRL_CHECK_LAUNCH();
+        return GRL_OK;
+    }
+    const int64_t DP = D <= 32 ? 32 : (D <= 64 ? 64 : 128);
+    const size_t dense = (size_t)(rows * D * es), padded = (size_t)(rows * DP * es);
+    const void* qs = Q; const void* ks = K;
+    int64_t qst = q_stride, kst = k_stride;
+    grl_temp qr(c, rope != GRL_ROPE_NONE ? dense : 16), kr(c, rope != GRL_ROPE_NONE ? dense : 16);
+    grl_temp qp(c, padded), kp(c, padded), vp(c, padded), op(c, padded);
+    if (!qr.p || !kr.p || !qp.p || !kp.p || !vp.p || !op.p) return GRL_ERR_OOM;
+    int rc = GRL_OK;
+    if (rope != GRL_ROPE_NONE) {
+        GRL_REQUIRE(D % 2 == 0, GRL_ERR_SHAPE, "%s: RoPE needs an even head_dim (got %lld)", who, (long long)D);
+        rc = grl_rope_strided(c, dtype, B, S, H, D, Q, q_stride, nullptr, qr.p, rope, rope_base, rope_scaling);
+        if (!rc) rc = grl_rope_strided(c, dtype, B, S, H, D, K, k_stride, nullptr, kr.p, rope, rope_base, rope_scaling);
+        if (rc) return rc;
+        qs = qr.p; ks = kr.p; qst = kst = H * D;
+    }
+    const dim3 grid(fa_ew_grid(rows * DP)), block(256);
+    auto pad = [&](const void* src, int64_t stride, void* dst) {
+        if (dtype == GRL_F32) hipLaunchKernelGGL(pad_heads_kernel<float>, grid, block, 0, c->stream, (const float*)src, stride, (float*)dst, rows, (int)H, (int)D, (int)DP);
+        else hipLaunchKernelGGL(pad_heads_kernel<uint16_t>, grid, block, 0, c->stream, (const uint16_t*)src, stride, (uint16_t*)dst, rows, (int)H, (int)D, (int)DP);
+    };
+    pad(qs, qst, qp.p); pad(ks, kst, kp.p); pad(V, v_stride, vp.p);
+    GRL_CHECK_LAUNCH();
+    rc = fa2_common(c, who, dtype, B, S, H, DP, qp.p, kp.p, vp.p, mask, op.p, H * DP, H * DP, H * DP, H * DP, scale, causal,
+                    GRL_ROPE_NONE, rope_base, rope_scaling, nullptr);
+    if (rc) return rc;
+    if (dtype == GRL_F32) hipLaunchKernelGGL(unpad_heads_kernel<float>, grid, block, 0, c->stream, (const float*)op.p, (float*)O, o_stride, rows, (int)H, (int)D, (int)DP);
+    else hipLaunchKernelGGL(unpad_heads_kernel<uint16_t>, grid, block, 0, c->stream, (const uint16_t*)op.p, (uint16_t*)O, o_stride, rows, (int)H, (int)D, (int)DP);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
 static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
                       const void* Q, const void* K, const void* V, const float* mask, void* O,
                       int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
@@ -758,17 +924,19 @@ static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t
     GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "%s: bad dtype %d", who, dtype);
     GRL_REQUIRE(rope >= GRL_ROPE_NONE && rope <= GRL_ROPE_HALF, GRL_ERR_ARG, "%s: bad rope style %d", who, rope);
     GRL_REQUIRE(B >= 0 && S >= 0 && H >= 0, GRL_ERR_SHAPE, "%s: negative dimension", who);
-    GRL_REQUIRE(D == 32 || D == 64 || D == 128, GRL_ERR_SHAPE, "%s: head_dim must be 32, 64 or 128 (got %lld)", who, (long long)D);
+    GRL_REQUIRE(D >= 1 && D <= 64 * NAIVE_MAX, GRL_ERR_SHAPE, "%s: head_dim must be between 1 and %d (got %lld)", who, 64 * NAIVE_MAX, (long long)D);
     GRL_REQUIRE(B < 65536 && H < 65536 && S < (1LL << 24), GRL_ERR_SHAPE, "%s: B,H must be < 65536 and S < 2^24", who);
     if (B == 0 || S == 0 || H == 0) return GRL_OK;
     GRL_REQUIRE(Q && K && V && O, GRL_ERR_ARG, "%s: null argument", who);
     const int64_t es = (int64_t)grl_dtype_size(dtype), hd = H * D;
     GRL_REQUIRE(q_stride >= hd && k_stride >= hd && v_stride >= hd && o_stride >= hd, GRL_ERR_SHAPE,
                 "%s: position stride smaller than num_heads*head_dim", who);
-    GRL_REQUIRE(((((uintptr_t)Q) | ((uintptr_t)K) | ((uintptr_t)V) | ((uintptr_t)O)) & 15u) == 0 &&
-                ((q_stride | k_stride | v_stride | o_stride) * es) % 16 == 0, GRL_ERR_ARG,
-                "%s: Q,K,V,O and their position strides must be 16-byte aligned", who);
     if (rope != GRL_ROPE_NONE) GRL_REQUIRE(rope_base > 0.f && rope_scaling != 0.f, GRL_ERR_ARG, "%s: bad rope base/scaling", who);
+    const bool granular = ((((uintptr_t)Q) | ((uintptr_t)K) | ((uintptr_t)V) | ((uintptr_t)O)) & 15u) == 0 &&
+                          ((q_stride | k_stride | v_stride | o_stride) * es) % 16 == 0;
+    if (!((D == 32 || D == 64 || D == 128) && granular))
+        return fa2_generic(c, who, dtype, B, S, H, D, Q, K, V, mask, O, q_stride, k_stride, v_stride, o_stride, scale, causal, rope,
+                           rope_base, rope_scaling);
 
     FaArgs a{};
     a.Q = Q; a.K = K; a.V = V; a.mask = mask; a.O = O;
@@ -777,12 +945,25 @@ static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t
 
     GRL_REQUIRE(S * std::max(std::max(q_stride, k_stride), std::max(v_stride, o_stride)) * es < (1LL << 31), GRL_ERR_SHAPE,
                 "%s: one batch entry must span less than 2 GiB", who);
-    void* own = nullptr;      // RoPE table or rotate-half workspace
+    void* own = nullptr;      // rotate-half workspace
     void* own2 = nullptr;     // rotated K of the bf16 fused path
     int rc = GRL_OK;
-    if (rope == GRL_ROPE_HALF) {
-        // (d, d+D/2) pairs straddle MFMA chunks: rotate Q and K once into a workspace with the
-        // standalone kernel, then run the plain kernel on the rotated copies.
+    int rope_q = rope == GRL_ROPE_INTERLEAVED ? 1 : 0;
+    if (rope == GRL_ROPE_HALF && dtype == GRL_BF16) {
+        // bf16: the kernel rotates the query rows as it loads them (both halves of a pair are chunks of the same
+        // lane); every K row is rotated exactly once here, from the table kept on the context
+        const float* tab = nullptr;
+        rc = grl_rope_table_get(c, (int)S, (int)D, rope_base, rope_scaling, GRL_ROPE_HALF, &tab);
+        if (rc) return rc;
+        a.rope = (const float2*)tab;
+        own2 = grl_malloc(c, (size_t)B * S * H * D * 2);
+        if (!own2) return GRL_ERR_OOM;
+        rc = grl_rope_half_apply_table(c, dtype, B, S, H, D, K, k_stride, own2, tab);
+        a.K = own2; a.k_stride = hd;
+        rope_q = 2;
+    } else if (rope == GRL_ROPE_HALF) {
+        // fp32: rotate Q and K once into a workspace with the standalone kernel, then run the plain kernel on
+        // the rotated copies.
         const size_t n = (size_t)B * S * H * D, bytes = n * grl_dtype_size(dtype);
         char* ws = (char*)workspace;
         if (!ws) { own = grl_malloc(c, 2 * bytes); if (!own) return GRL_ERR_OOM; ws = (char*)own; }
@@ -790,16 +971,16 @@ static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t
         if (!rc) rc = grl_rope_strided(c, dtype, B, S, H, D, K, k_stride, nullptr, ws + bytes, GRL_ROPE_HALF, rope_base, rope_scaling);
         a.Q = ws; a.K = ws + bytes; a.q_stride = hd; a.k_stride = hd;
     } else if (rope == GRL_ROPE_INTERLEAVED) {
-        const size_t bytes = (size_t)S * (D / 2) * sizeof(float2);
-        own = grl_malloc(c, bytes);
-        if (!own) return GRL_ERR_OOM;
-        rc = grl_build_rope_table(c, (float*)own, (int)S, (int)D, rope_base, rope_scaling);
-        a.rope = (const float2*)own;
-        if (!rc && dtype == GRL_BF16) {
+        // the (S, D/2) cos/sin table lives on the context and is built once per (D, base, scaling)
+        const float* tab = nullptr;
+        rc = grl_rope_table_get(c, (int)S, (int)D, rope_base, rope_scaling, GRL_ROPE_INTERLEAVED, &tab);
+        if (rc) return rc;
+        a.rope = (const float2*)tab;
+        if (dtype == GRL_BF16) {
             // every K row is rotated exactly once here; the kernel rotates Q rows as it loads them
             own2 = grl_malloc(c, (size_t)B * S * H * D * 2);
-            if (!own2) { grl_free(c, own); return GRL_ERR_OOM; }
-            rc = grl_rope_apply_table(c, dtype, B, S, H, D, K, k_stride, own2, (const float*)own);
+            if (!own2) return GRL_ERR_OOM;
+            rc = grl_rope_apply_table(c, dtype, B, S, H, D, K, k_stride, own2, tab);
             a.K = own2; a.k_stride = hd;
         }
     }
@@ -808,7 +989,7 @@ static int fa2_common(grl_ctx* c, const char* who, int dtype, int64_t B, int64_t
         if (dtype == GRL_F32) {
             rc = D == 32 ? launch_fa<float, 32>(c, a, fused) : D == 64 ? launch_fa<float, 64>(c, a, fused) : launch_fa<float, 128>(c, a, fused);
         } else {
-            rc = D == 32 ? launch_fa16<32>(c, a, fused) : D == 64 ? launch_fa16<64>(c, a, fused) : launch_fa16<128>(c, a, fused);
+            rc = D == 32 ? launch_fa16<32>(c, a, rope_q) : D == 64 ? launch_fa16<64>(c, a, rope_q) : launch_fa16<128>(c, a, rope_q);
         }
     }
     if (own) grl_free(c, own);   // stream order keeps the blocks alive until the kernel has finished

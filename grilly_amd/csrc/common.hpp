@@ -22,7 +22,15 @@ struct grl_ctx {
     std::map<size_t, std::vector<void*>> free_blocks;
     std::map<void*, size_t> live;
     grl_pool_stats stats{};
+    // cos/sin tables of the rotary embedding, built once per (head dim, base, scaling, pairing) and kept until the
+    // context goes away; a table built for S positions serves every shorter sequence
+    struct rope_table { int S, D, style; float base, scaling; void* dev; };
+    std::mutex tab_mu;
+    std::vector<rope_table> rope_tables;
 };
+
+// device pointer to a (>= S, D/2) table of {cos, sin}; builds it on first use (on the context stream)
+int grl_rope_table_get(grl_ctx* c, int S, int D, float base, float scaling, int style, const float** out);
 
 void grl_set_error(const char* fmt, ...);
 

@@ -22,7 +22,7 @@ extern "C" int grl_bert_layer_fwd(grl_ctx* c, int dtype, int64_t B, int64_t S, i
     GRL_REQUIRE(c && w && x && workspace, GRL_ERR_ARG, "grl_bert_layer_fwd: null argument");
     GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_bert_layer_fwd: bad dtype %d", dtype);
     GRL_REQUIRE(B >= 0 && S >= 0 && H > 0 && d_ff > 0, GRL_ERR_SHAPE, "grl_bert_layer_fwd: bad shape");
-    GRL_REQUIRE(D == 32 || D == 64 || D == 128, GRL_ERR_SHAPE, "grl_bert_layer_fwd: head_dim must be 32, 64 or 128 (got %lld)", (long long)D);
+    GRL_REQUIRE(D >= 1 && D <= 1024, GRL_ERR_SHAPE, "grl_bert_layer_fwd: head_dim must be between 1 and 1024 (got %lld)", (long long)D);
     GRL_REQUIRE(w->w_qkv && w->w_o && w->w_ff1 && w->w_ff2 && w->ln1_g && w->ln1_b && w->ln2_g && w->ln2_b,
                 GRL_ERR_ARG, "grl_bert_layer_fwd: null weight");
     if (B == 0 || S == 0) return GRL_OK;

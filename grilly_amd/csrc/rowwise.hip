@@ -252,7 +252,7 @@ extern "C" int grl_layernorm(grl_ctx* c, int dtype, int64_t rows, int64_t F, con
 }
 
 // ------------------------------------------------------------------ elementwise
-enum { OP_ADD = 0, OP_GELU = 1, OP_SILU = 2, OP_RELU = 3 };
+enum { OP_ADD = 0, OP_GELU = 1, OP_SILU = 2, OP_RELU = 3, OP_GCU = 4, OP_ROSWISH = 5 };
 
 // shaders/activation-swiglu.glsl:40-49: sign-split stable sigmoid
 __device__ __forceinline__ float sigmoid_stable(float v) {
@@ -261,15 +261,18 @@ __device__ __forceinline__ float sigmoid_stable(float v) {
     return e / (1.0f + e);
 }
 
-template <int OP> __device__ __forceinline__ float ew_apply(float a, float b) {
+// p0, p1: alpha and beta of RoSwish, unused otherwise
+template <int OP> __device__ __forceinline__ float ew_apply(float a, float b, float p0, float p1) {
     if (OP == OP_ADD) return a + b;
     if (OP == OP_GELU) return gelu_ref(a);
     if (OP == OP_RELU) return fmaxf(a, 0.0f);   // shaders/activation-relu.glsl (backend/fnn.py:232-283)
+    if (OP == OP_GCU) return a * cosf(a);       // shaders/activation-gcu.glsl:29-31 (backend/fnn.py:393-440)
+    if (OP == OP_ROSWISH) return (a + p0) * sigmoid_stable(p1 * a) - 0.5f * p0;   // shaders/activation-roswish.glsl:30-46
     return a * sigmoid_stable(a);   // backend/fnn.py:344-391 (activation_silu): x*sigmoid(x)
 }
 
 template <typename T, int OP, bool VEC>
-__global__ __launch_bounds__(256) void elementwise_kernel(const T* a, const T* b, T* out, int64_t n) {
+__global__ __launch_bounds__(256) void elementwise_kernel(const T* a, const T* b, T* out, int64_t n, float p0, float p1) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (VEC) {
@@ -279,14 +282,14 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const T* a, const T* b
             x.load(a + v * 4);
             if (OP == OP_ADD) y.load(b + v * 4);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) o.set(k, ew_apply<OP>(x.get(k), OP == OP_ADD ? y.get(k) : 0.f));
+            for (int k = 0; k < 4; ++k) o.set(k, ew_apply<OP>(x.get(k), OP == OP_ADD ? y.get(k) : 0.f, p0, p1));
             o.store(out + v * 4);
         }
         for (int64_t t = (nv << 2) + i; t < n; t += stride)
-            elem<T>::st(out + t, ew_apply<OP>(elem<T>::ld(a + t), OP == OP_ADD ? elem<T>::ld(b + t) : 0.f));
+            elem<T>::st(out + t, ew_apply<OP>(elem<T>::ld(a + t), OP == OP_ADD ? elem<T>::ld(b + t) : 0.f, p0, p1));
     } else {
         for (int64_t t = i; t < n; t += stride)
-            elem<T>::st(out + t, ew_apply<OP>(elem<T>::ld(a + t), OP == OP_ADD ? elem<T>::ld(b + t) : 0.f));
+            elem<T>::st(out + t, ew_apply<OP>(elem<T>::ld(a + t), OP == OP_ADD ? elem<T>::ld(b + t) : 0.f, p0, p1));
     }
 }
 
@@ -299,10 +302,10 @@ static inline unsigned ew_grid(int64_t work_items) {
 }
 
 template <typename T, int OP>
-static int launch_ew(grl_ctx* c, int64_t n, const void* a, const void* b, void* out) {
+static int launch_ew(grl_ctx* c, int64_t n, const void* a, const void* b, void* out, float p0 = 0.f, float p1 = 0.f) {
     bool vec = aligned16(a) && aligned16(out) && (!b || aligned16(b));
-    if (vec) hipLaunchKernelGGL((elementwise_kernel<T, OP, true>), dim3(ew_grid(n / 4 + 1)), dim3(256), 0, c->stream, (const T*)a, (const T*)b, (T*)out, n);
-    else     hipLaunchKernelGGL((elementwise_kernel<T, OP, false>), dim3(ew_grid(n)), dim3(256), 0, c->stream, (const T*)a, (const T*)b, (T*)out, n);
+    if (vec) hipLaunchKernelGGL((elementwise_kernel<T, OP, true>), dim3(ew_grid(n / 4 + 1)), dim3(256), 0, c->stream, (const T*)a, (const T*)b, (T*)out, n, p0, p1);
+    else     hipLaunchKernelGGL((elementwise_kernel<T, OP, false>), dim3(ew_grid(n)), dim3(256), 0, c->stream, (const T*)a, (const T*)b, (T*)out, n, p0, p1);
     GRL_CHECK_LAUNCH();
     return GRL_OK;
 }
@@ -318,6 +321,46 @@ extern "C" int grl_add(grl_ctx* c, int dtype, int64_t n, const void* a, const vo
 extern "C" int grl_gelu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_gelu", OP_GELU, false) }
 extern "C" int grl_silu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_silu", OP_SILU, false) }
 extern "C" int grl_relu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_relu", OP_RELU, false) }
+extern "C" int grl_gcu(grl_ctx* c, int dtype, int64_t n, const void* a, void* out) { const void* b = nullptr; EW_ENTRY("grl_gcu", OP_GCU, false) }
+extern "C" int grl_roswish(grl_ctx* c, int dtype, int64_t n, const void* a, void* out, float alpha, float beta) {
+    GRL_REQUIRE(c && a && out, GRL_ERR_ARG, "grl_roswish: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_roswish: bad dtype %d", dtype);
+    GRL_REQUIRE(n >= 0, GRL_ERR_SHAPE, "grl_roswish: negative size");
+    if (n == 0) return GRL_OK;
+    return dtype == GRL_F32 ? launch_ew<float, OP_ROSWISH>(c, n, a, nullptr, out, alpha, beta) : launch_ew<uint16_t, OP_ROSWISH>(c, n, a, nullptr, out, alpha, beta);
+}
+
+// softmax over the last dimension, one wave per row: maximum (starting from -1e10 like the shader's first pass),
+// sum of exp(x - max), quotient; the second and third pass read the row again (from cache for rows of usual length)
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const T* x, T* y, int64_t rows, int F) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * (int64_t)F;
+    T* yr = y + row * (int64_t)F;
+    float m = -1e10f;
+    for (int i = lane; i < F; i += 64) m = fmaxf(m, elem<T>::ld(xr + i));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    float sum = 0.f;
+    for (int i = lane; i < F; i += 64) sum += __expf(elem<T>::ld(xr + i) - m);
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+    for (int i = lane; i < F; i += 64) elem<T>::st(yr + i, __expf(elem<T>::ld(xr + i) - m) * inv);
+}
+
+extern "C" int grl_softmax(grl_ctx* c, int dtype, int64_t rows, int64_t F, const void* x, void* y) {
+    GRL_REQUIRE(c && x && y, GRL_ERR_ARG, "grl_softmax: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_softmax: bad dtype %d", dtype);
+    GRL_REQUIRE(rows >= 0 && F > 0 && F < (1 << 30) && rows < ((int64_t)1 << 33), GRL_ERR_SHAPE, "grl_softmax: bad shape rows=%lld F=%lld", (long long)rows, (long long)F);
+    if (rows == 0) return GRL_OK;
+    const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(softmax_rows_kernel<float>, grid, block, 0, c->stream, (const float*)x, (float*)y, rows, (int)F);
+    else hipLaunchKernelGGL(softmax_rows_kernel<uint16_t>, grid, block, 0, c->stream, (const uint16_t*)x, (uint16_t*)y, rows, (int)F);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
 
 // x (rows, 2h) -> y (rows, h)
 template <typename T>
@@ -459,12 +502,11 @@ int grl_rope_strided(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t H, int
         const int64_t es = (int64_t)grl_dtype_size(dtype), epc = 16 / es;
         const bool chunks = style == GRL_ROPE_HALF ? (D / 2) % epc == 0 : D % epc == 0;
         if (!position_ids && chunks && ((((uintptr_t)x) | ((uintptr_t)y)) & 15u) == 0 && (x_stride * es) % 16 == 0 && S * (D / 2) < (1LL << 31)) {
-            grl_temp tab(c, (size_t)S * (D / 2) * sizeof(float2));
-            if (!tab.p) return GRL_ERR_OOM;
-            int rc = grl_build_rope_table_styled(c, (float*)tab.p, (int)S, (int)D, rope_base, rope_scaling, style);
+            const float* tab = nullptr;
+            int rc = grl_rope_table_get(c, (int)S, (int)D, rope_base, rope_scaling, style, &tab);
             if (rc) return rc;
-            return style == GRL_ROPE_HALF ? grl_rope_half_apply_table(c, dtype, B, S, H, D, x, x_stride, y, (const float*)tab.p)
-                                          : grl_rope_apply_table(c, dtype, B, S, H, D, x, x_stride, y, (const float*)tab.p);
+            return style == GRL_ROPE_HALF ? grl_rope_half_apply_table(c, dtype, B, S, H, D, x, x_stride, y, tab)
+                                          : grl_rope_apply_table(c, dtype, B, S, H, D, x, x_stride, y, tab);
         }
     }
     RopeFreq fr; grl_rope_freqs(&fr, (int)D, rope_base);
@@ -495,6 +537,31 @@ int grl_build_rope_table_styled(grl_ctx* c, float* tab, int S, int D, float base
 }
 int grl_build_rope_table(grl_ctx* c, float* tab, int S, int D, float base, float scaling) {
     return grl_build_rope_table_styled(c, tab, S, D, base, scaling, GRL_ROPE_INTERLEAVED);
+}
+
+int grl_rope_table_get(grl_ctx* c, int S, int D, float base, float scaling, int style, const float** out) {
+    std::lock_guard<std::mutex> lk(c->tab_mu);
+    for (auto& t : c->rope_tables)
+        if (t.D == D && t.style == style && t.base == base && t.scaling == scaling && t.S >= S) { *out = (const float*)t.dev; return GRL_OK; }
+    // not there (or too short): build one; a shorter table of the same kind is replaced.  Kernels already queued
+    // on the stream may still read the old one, and the pool hands a freed block to the next request of its
+    // size, so the old table is only dropped once the stream has drained.
+    for (size_t i = 0; i < c->rope_tables.size(); ++i) {
+        auto& t = c->rope_tables[i];
+        if ((t.D == D && t.style == style && t.base == base && t.scaling == scaling) || c->rope_tables.size() >= 16) {
+            GRL_CHECK_HIP(hipStreamSynchronize(c->stream));
+            grl_free(c, t.dev);
+            c->rope_tables.erase(c->rope_tables.begin() + i);
+            break;
+        }
+    }
+    void* dev = grl_malloc(c, (size_t)S * (D / 2) * sizeof(float2));
+    if (!dev) return GRL_ERR_OOM;
+    int rc = grl_build_rope_table_styled(c, (float*)dev, S, D, base, scaling, style);
+    if (rc) { grl_free(c, dev); return rc; }
+    c->rope_tables.push_back({S, D, style, base, scaling, dev});
+    *out = (const float*)dev;
+    return GRL_OK;
 }
 
 // Interleaved RoPE from a precomputed (S, D/2) {cos, sin} table: one 16-byte chunk per thread,

@@ -68,8 +68,8 @@ class BertEncoder:
         self.core = core.core if hasattr(core, "core") else core
         if not isinstance(self.core, HipCore):
             raise TypeError("BertEncoder needs a Compute() backend or its HipCore")
-        if cfg.head_dim not in (32, 64, 128) or cfg.head_dim * cfg.heads != cfg.d_model:
-            raise ValueError("d_model must be heads*head_dim with head_dim 32, 64 or 128")
+        if cfg.head_dim * cfg.heads != cfg.d_model:
+            raise ValueError("d_model must be heads*head_dim")
         self.cfg, self.dtype, self.code = cfg, dtype, dtype_code(dtype)
         c = self.core
         self._keep = []                       # device buffers owned by the encoder
@@ -212,7 +212,7 @@ class PreNormEncoder:
     Built from the same entry points as the post-LN encoder: the projection GEMMs, attention with the
     rotate-half rotation fused, LayerNorm, the dual GEMM with the GELU gate, and the GEMM that adds the
     residual stream in place.
-    The packed Wqkv is read through three row blocks (no split copy).  The +-50 / +-1e6 clips the
+    The packed Wqkv is one GEMM; attention reads its three column blocks in place.  The +-50 / +-1e6 clips the
     reference puts around the gate (:924-930) are not applied: they only act beyond those magnitudes."""
 
     _MATS = ("w_qkv", "w_o", "w_ff_in", "w_ff_gate", "w_ff2")
@@ -222,8 +222,8 @@ class PreNormEncoder:
         self.core = core.core if hasattr(core, "core") else core
         if not isinstance(self.core, HipCore):
             raise TypeError("PreNormEncoder needs a Compute() backend or its HipCore")
-        if cfg.head_dim not in (32, 64, 128) or cfg.head_dim * cfg.heads != cfg.d_model:
-            raise ValueError("d_model must be heads*head_dim with head_dim 32, 64 or 128")
+        if cfg.head_dim * cfg.heads != cfg.d_model or cfg.head_dim % 2 or cfg.head_dim > 128:
+            raise ValueError("d_model must be heads*head_dim with an even head_dim up to 128 (rotary positions)")
         self.cfg, self.dtype, self.code = cfg, dtype, dtype_code(dtype)
         c = self.core
         self._keep = []
@@ -252,7 +252,8 @@ class PreNormEncoder:
         cfg, c = self.cfg, self.core
         es = 2 if self.code == L.GRL_BF16 else 4
         act = B * S * cfg.d_model * es
-        self.x, self.q, self.k, self.v, self.att, self.t = (c.alloc(act) for _ in range(6))
+        self.x, self.att, self.t = (c.alloc(act) for _ in range(3))
+        self.qkv = c.alloc(3 * act)                    # packed (M, 3d): Q, K, V are its three column blocks
         self.h = c.alloc(B * S * cfg.d_ff * es)
         self.ids = c.alloc(B * S * 4)
         self.mask = c.alloc(B * S * 4)
@@ -264,7 +265,7 @@ class PreNormEncoder:
 
     def release_activations(self):
         if self._shape is not None:
-            for b in (self.x, self.q, self.k, self.v, self.att, self.t, self.h, self.ids, self.mask, self.first, self.pooled):
+            for b in (self.x, self.qkv, self.att, self.t, self.h, self.ids, self.mask, self.first, self.pooled):
                 b.free()
             self._shape = None
 
@@ -296,11 +297,13 @@ class PreNormEncoder:
         L.check(lib.grl_layernorm(c.ctx, code, M, d, self.x.ptr, None, self.emb_g.ptr, self.emb_b.ptr, cfg.emb_eps,
                                   self.x.ptr), "embedding layernorm")
         for w in self.layers:
-            for i, dst in enumerate((self.q, self.k, self.v)):       # row blocks of the packed weight and bias
-                L.check(lib.grl_gemm_nt(c.ctx, code, code, M, d, d, self.x.ptr, w["w_qkv"].ptr + i * d * d * es,
-                                        w["b_qkv"].ptr + i * d * 4, dst.ptr, L.EPI_NONE), "q/k/v projection")
-            L.check(lib.grl_fa2_fwd(c.ctx, code, B, S, H, D, self.q.ptr, self.k.ptr, self.v.ptr, mask, self.att.ptr,
-                                    1.0 / float(np.sqrt(D)), 0, L.ROPE_HALF, cfg.rope_base, cfg.rope_scaling, None),
+            # one GEMM with the packed weight; attention reads Q, K, V as column blocks of its output and applies
+            # the rotation itself (queries as they are loaded, keys once per row from the cached table)
+            L.check(lib.grl_gemm_nt(c.ctx, code, code, M, 3 * d, d, self.x.ptr, w["w_qkv"].ptr, w["b_qkv"].ptr,
+                                    self.qkv.ptr, L.EPI_NONE), "q/k/v projection")
+            L.check(lib.grl_fa2_fwd_strided(c.ctx, code, B, S, H, D, self.qkv.ptr, self.qkv.ptr + d * es,
+                                            self.qkv.ptr + 2 * d * es, mask, self.att.ptr, 3 * d, 3 * d, 3 * d, d,
+                                            1.0 / float(np.sqrt(D)), 0, L.ROPE_HALF, cfg.rope_base, cfg.rope_scaling),
                     "attention")
             L.check(lib.grl_gemm_nt_res(c.ctx, code, code, M, d, d, self.att.ptr, w["w_o"].ptr, w["b_o"].ptr, self.x.ptr,
                                         self.x.ptr), "output projection + residual")

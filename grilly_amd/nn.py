@@ -241,9 +241,11 @@ class FlashAttention2(Module):
 
 
 class MultiheadAttention(Module):
-    """q/k/v/out projections around the fused attention kernel (reference nn/modules.py:1085-1222 builds
-    the same block from separate score / softmax / output shaders).  Self-attention shapes only
-    (query and key of the same length); `mask` is a (batch, seq) keep-mask.  Returns (output, None)."""
+    """q/k/v/out projections around attention (reference nn/modules.py:1085-1222 builds the block from separate
+    score / softmax / output steps).  Returns (output, attention_weights) with weights (batch, heads, query_len,
+    key_len) like the reference; key and value may be longer or shorter than the query.  `mask` is a
+    (batch, key_len) keep-mask (1 keep, 0 drop).  With need_weights=False the fused kernel runs (query and key
+    of the same length) and the second result is None."""
 
     def __init__(self, embed_dim, num_heads, dropout=0.0):
         super().__init__()
@@ -255,15 +257,19 @@ class MultiheadAttention(Module):
         self.v_proj = Linear(embed_dim, embed_dim)
         self.out_proj = Linear(embed_dim, embed_dim)
 
-    def forward(self, query, key, value, mask=None):
+    def forward(self, query, key, value, mask=None, need_weights=True):
         q, k, v = self.q_proj(query), self.k_proj(key), self.v_proj(value)
         B, S, _ = q.shape
-        if k.shape[1] != S or v.shape[1] != S:
-            raise ValueError("MultiheadAttention on this backend needs query, key and value of the same length")
-        shape = (B, S, self.num_heads, self.head_dim)
-        o = self._get_backend().attention.flash_attention2(q.reshape(shape), k.reshape(shape), v.reshape(shape),
-                                                           self.num_heads, self.head_dim, mask=mask)
-        return self.out_proj(o.reshape(B, S, self.embed_dim)), None
+        Sk = k.shape[1]
+        if v.shape[1] != Sk:
+            raise ValueError("key and value must have the same length")
+        qs, ks = (B, S, self.num_heads, self.head_dim), (B, Sk, self.num_heads, self.head_dim)
+        att = self._get_backend().attention
+        if need_weights or Sk != S:
+            o, w = att.attention_with_weights(q.reshape(qs), k.reshape(ks), v.reshape(ks), mask=mask)
+        else:
+            o, w = att.flash_attention2(q.reshape(qs), k.reshape(ks), v.reshape(ks), self.num_heads, self.head_dim, mask=mask), None
+        return self.out_proj(o.reshape(B, S, self.embed_dim)), w
 
     def __repr__(self):
         return f"MultiheadAttention(embed_dim={self.embed_dim}, num_heads={self.num_heads})"
@@ -294,7 +300,7 @@ class TransformerEncoderLayer(Module):
     def forward(self, src, src_mask=None, prosody=None):
         src = np.asarray(src, dtype=np.float32)
         src2 = self.norm1(src)
-        src2, _ = self.self_attn(src2, src2, src2, src_mask)
+        src2, _ = self.self_attn(src2, src2, src2, src_mask, need_weights=False)
         src = src + self.dropout1(src2)
         src2 = self.norm2(src)
         src2 = self.linear2(self.dropout2(self.activation(self.linear1(src2))))

@@ -178,8 +178,13 @@ int grl_swiglu_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t 
  * its docstring :374-395; constants of shaders/flash-attention2.glsl:95,152,214) and
  * shaders/flash-attention2-rope.glsl:73-148 (interleaved pairs, theta =
  * pos*base^(-2p/D)/scaling); causal rule of shaders/attention-mask.glsl:42-46.
- * D must be 32, 64 or 128.  GRL_ROPE_HALF uses the (d, d+D/2) pairing of
- * shaders/rope.glsl:74-125 and needs a workspace of 2*B*S*H*D elements (NULL = pool). */
+ * Any head dim D from 1 to 1024 (the reference reshapes with whatever head_dim it is given,
+ * backend/attention.py:403-410): 32, 64 and 128 with 16-byte granular operands run the MFMA kernels directly,
+ * other head dims up to 128 (or operands that are not 16-byte granular) run them on zero-padded copies taken
+ * from the pool, larger ones a one-wave-per-query kernel; RoPE needs an even D up to 128.
+ * GRL_ROPE_HALF uses the (d, d+D/2) pairing of shaders/rope.glsl:74-125 and, on the direct path, a workspace of
+ * 2*B*S*H*D elements (NULL = pool).  The cos/sin table of the rotation is built once per (D, base, scaling,
+ * pairing) and kept on the context. */
 int grl_fa2_fwd(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
                 const void* Q, const void* K, const void* V, const float* mask, void* O,
                 float scale, int causal, int rope, float rope_base, float rope_scaling,
@@ -224,6 +229,14 @@ int grl_gelu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
 int grl_silu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
 /* Replaces VulkanFNN.activation_relu (backend/fnn.py:232-283): max(0,x). */
 int grl_relu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
+/* Replaces VulkanFNN.activation_gcu (backend/fnn.py:393-440, shaders/activation-gcu.glsl:29-31): x*cos(x). */
+int grl_gcu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
+/* Replaces VulkanFNN.activation_roswish (backend/fnn.py:442-497, shaders/activation-roswish.glsl:30-46):
+ * (x+alpha)*sigmoid(beta*x) - alpha/2. */
+int grl_roswish(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y, float alpha, float beta);
+/* Softmax over the last dimension of x (rows, F).  Replaces VulkanFNN.activation_softmax
+ * (backend/fnn.py:574-700, shaders/activation-softmax.glsl:38-99: max from -1e10, sum of exp(x-max), quotient). */
+int grl_softmax(grl_ctx* ctx, int dtype, int64_t rows, int64_t F, const void* x, void* y);
 /* x (rows, 2h) -> y (rows, h): x1*(x2*sigmoid(x2)), x1 first half.
  * Replaces VulkanFNN.activation_swiglu (backend/fnn.py:499-572, shaders/activation-swiglu.glsl:21-52). */
 int grl_swiglu_act(grl_ctx* ctx, int dtype, int64_t rows, int64_t h, const void* x, void* y);

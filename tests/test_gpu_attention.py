@@ -131,7 +131,8 @@ def test_fa2_shapes_and_errors(backend):
     with pytest.raises(ValueError):
         backend.attention.flash_attention2(q, k, v, 2, 32, mask=np.ones((2, 39)))
     with pytest.raises(ValueError):
-        backend.attention.flash_attention2(q[..., :24], k[..., :24], v[..., :24], 2, 24)     # head_dim 24 unsupported
+        backend.attention.flash_attention2(np.zeros((1, 4, 1, 1100), np.float32), np.zeros((1, 4, 1, 1100), np.float32),
+                                           np.zeros((1, 4, 1, 1100), np.float32), 1, 1100)      # head_dim above 1024
     with pytest.raises(ValueError):
         backend.attention.flash_attention2(q, k[:, :10], v, 2, 32)
     # deterministic across runs (the reference shader is not)
@@ -178,3 +179,47 @@ def test_apply_rope_parity_table_and_pairwise_paths(backend, dtype, style, B, S,
     y2 = backend.attention.apply_rope(x, pid, 500.0, 1.5, rope_style=style, dtype=dtype)
     assert O.max_rel(y2, ref) < t
     assert O.max_rel(y2, y) < (1e-6 if dtype == "fp32" else 1e-2)      # same angles, same arithmetic
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("D", [8, 24, 40, 80, 96, 6, 1, 33, 130, 160, 320])
+@pytest.mark.parametrize("mode", ["dense", "causal_mask"])
+def test_fa2_any_head_dim(backend, dtype, D, mode):
+    """The reference reshapes with whatever head_dim it is given (backend/attention.py:403-410): head dims other
+    than 32 / 64 / 128 run on zero-padded copies (up to 128) or the one-wave-per-query kernel (above)."""
+    B, S, H = 2, 75, 3
+    rng = np.random.default_rng(D * 7 + len(mode))
+    q, k, v = qkv(rng, B, S, H, D, dtype)
+    causal = mode != "dense"
+    mask = None
+    if causal:
+        mask = np.ones((B, S), np.float32); mask[0, 50:] = 0; mask[1, :3] = 0
+    o = backend.attention.flash_attention2(q, k, v, H, D, mask=mask, causal=causal, dtype=dtype)
+    assert o.shape == (B, S, H, D)
+    assert O.max_rel(o, O.truth_attention(q, k, v, mask=mask, causal=causal)) < tol(dtype)
+    # (B,S,H*D) input with the head split given by the arguments
+    flat = [t.reshape(B, S, H * D) for t in (q, k, v)]
+    np.testing.assert_array_equal(backend.attention.flash_attention2(*flat, H, D, mask=mask, causal=causal, dtype=dtype), o)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("style", ["interleaved", "half"])
+@pytest.mark.parametrize("D", [8, 24, 96])
+def test_fa2_rope_any_head_dim(backend, dtype, style, D):
+    rng = np.random.default_rng(D + len(style))
+    q, k, v = qkv(rng, 1, 60, 2, D, dtype)
+    o = backend.attention.flash_attention2_rope(q, k, v, 2, D, causal=True, rope_style=style, dtype=dtype)
+    assert O.max_rel(o, O.truth_attention(q, k, v, causal=True, rope=style)) < tol(dtype)
+    with pytest.raises(ValueError):
+        backend.attention.flash_attention2_rope(q[..., :7], k[..., :7], v[..., :7], 2, 7, rope_style=style, dtype=dtype)
+
+
+def test_rope_table_is_reused_across_calls(backend):
+    """the cos/sin table of the fused rotation is built once per (head dim, base, scaling) and serves shorter sequences"""
+    rng = np.random.default_rng(77)
+    for S in (96, 40, 96, 130):
+        q, k, v = qkv(rng, 1, S, 2, 64, "bf16")
+        o = backend.attention.flash_attention2_rope(q, k, v, 2, 64, causal=True, dtype="bf16")
+        assert O.max_rel(o, O.truth_attention(q, k, v, causal=True, rope="interleaved")) < TOL_BF16
+    o2 = backend.attention.flash_attention2_rope(q, k, v, 2, 64, causal=True, rope_base=500.0, dtype="bf16")
+    assert O.max_rel(o2, O.truth_attention(q, k, v, causal=True, rope="interleaved", base=500.0)) < TOL_BF16

@@ -74,3 +74,33 @@ def test_transformer_encoder_layer(backend, act):
     ref = x1 + f @ P["linear2.weight"].T + P["linear2.bias"]
     assert y.shape == (B, S, d)
     assert O.max_rel(y, ref) < TOL_F32
+
+
+@pytest.mark.parametrize("Sq,Sk", [(30, 30), (17, 45), (40, 9)])
+def test_multihead_attention_weights_and_cross_length(backend, Sq, Sk):
+    """MultiheadAttention returns (output, weights (B,H,Sq,Sk)) like the reference (nn/modules.py:1123-1216), also
+    when key / value are longer or shorter than the query; with need_weights=False the fused kernel gives the
+    same output."""
+    np.random.seed(35)
+    rng = np.random.default_rng(35)
+    d, H, B = 96, 4, 2
+    mha = nn.MultiheadAttention(d, H).to_backend(backend)
+    for n, p in mha.named_parameters():
+        p.data[...] = rng.standard_normal(p.shape) * (0.1 if n.endswith("weight") else 0.05)
+    q = rng.standard_normal((B, Sq, d)).astype(np.float32)
+    kv = q if Sk == Sq else rng.standard_normal((B, Sk, d)).astype(np.float32)
+    mask = (np.arange(Sk)[None] < np.array([Sk, max(Sk // 2, 1)])[:, None]).astype(np.float32)
+    out, w = mha(q, kv, kv, mask)
+    P = {n: p.data.astype(np.float64) for n, p in mha.named_parameters()}
+    proj = lambda t, n: t @ P[f"{n}.weight"].T + P[f"{n}.bias"]
+    D = d // H
+    qh = proj(q, "q_proj").reshape(B, Sq, H, D); kh = proj(kv, "k_proj").reshape(B, Sk, H, D); vh = proj(kv, "v_proj").reshape(B, Sk, H, D)
+    sc = np.einsum("bqhd,bkhd->bhqk", qh, kh) / np.sqrt(D) + ((mask.astype(np.float64) - 1) * 1e9)[:, None, None, :]
+    pw = np.exp(sc - sc.max(-1, keepdims=True)); pw /= pw.sum(-1, keepdims=True)
+    ref = proj(np.einsum("bhqk,bkhd->bqhd", pw, vh).reshape(B, Sq, d), "out_proj")
+    assert out.shape == (B, Sq, d) and w.shape == (B, H, Sq, Sk)
+    assert O.max_rel(w, pw) < TOL_F32 and O.max_rel(out, ref) < TOL_F32
+    np.testing.assert_allclose(w.sum(-1), 1.0, atol=1e-5)
+    if Sq == Sk:
+        out2, none = mha(q, kv, kv, mask, need_weights=False)
+        assert none is None and O.max_rel(out2, ref) < TOL_F32

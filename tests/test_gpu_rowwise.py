@@ -159,7 +159,7 @@ def test_c_abi_argument_errors(backend):
     assert lib.grl_gemm_nt(c.ctx, 0, 0, 4, 4, 4, buf.ptr, buf.ptr, None, buf.ptr, 9) == L.ERR_ARG
     assert lib.grl_gemm_nt(c.ctx, 0, 0, -1, 4, 4, buf.ptr, buf.ptr, None, buf.ptr, 0) == L.ERR_SHAPE
     assert lib.grl_gemm_nt(c.ctx, 0, 0, 4, 4, 4, None, buf.ptr, None, buf.ptr, 0) == L.ERR_ARG
-    assert lib.grl_fa2_fwd(c.ctx, 0, 1, 8, 1, 48, buf.ptr, buf.ptr, buf.ptr, None, buf.ptr, 1.0, 0, 0, 1e4, 1.0, None) == L.ERR_SHAPE
+    assert lib.grl_fa2_fwd(c.ctx, 0, 1, 8, 1, 2048, buf.ptr, buf.ptr, buf.ptr, None, buf.ptr, 1.0, 0, 0, 1e4, 1.0, None) == L.ERR_SHAPE
     assert "head_dim" in L.last_error()
     assert lib.grl_layernorm(c.ctx, 0, 4, 0, buf.ptr, None, buf.ptr, buf.ptr, 1e-5, buf.ptr) == L.ERR_SHAPE
     assert lib.grl_free(c.ctx, ctypes.c_void_p(12345)) == L.ERR_ARG          # foreign pointer
@@ -168,3 +168,41 @@ def test_c_abi_argument_errors(backend):
     buf.free()
     info = backend.device_info()
     assert info["arch"].startswith("gfx950") and info["wavefront"] == 64 and info["compute_units"] > 0
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_gcu_roswish_softmax_activations(backend, dtype):
+    """activation_gcu / activation_roswish / activation_softmax (reference backend/fnn.py:393-497, :574-700) and
+    the reference's keyword name `input_data` on every activation."""
+    rng = np.random.default_rng(31)
+    x = (3 * rng.standard_normal((5, 7, 33))).astype(np.float32)
+    if dtype == "bf16":
+        x = O.bf16_round(x)
+    t = TOL_F32 if dtype == "fp32" else TOL_BF16
+    x64 = x.astype(np.float64)
+    assert O.max_rel(backend.fnn.activation_gcu(input_data=x, dtype=dtype), x64 * np.cos(x64)) < t
+    assert O.max_rel(backend.activation_roswish(x, alpha=0.7, beta=1.3, dtype=dtype), O.truth_roswish(x64, 0.7, 1.3)) < t
+    for axis in (-1, 1, 0):
+        e = np.exp(x64 - x64.max(axis=axis, keepdims=True))
+        sm = backend.fnn.activation_softmax(x, axis=axis, dtype=dtype)
+        assert sm.shape == x.shape and O.max_rel(sm, e / e.sum(axis=axis, keepdims=True)) < t
+    np.testing.assert_allclose(backend.activation_softmax(np.array([1.0, 1.0, 1.0, 1.0], np.float32)), 0.25, rtol=1e-6)
+    # keyword compatibility
+    np.testing.assert_array_equal(backend.fnn.activation_gelu(input_data=x, dtype=dtype), backend.fnn.activation_gelu(x, dtype=dtype))
+    np.testing.assert_array_equal(backend.fnn.activation_silu(input_data=x, dtype=dtype), backend.fnn.activation_silu(x, dtype=dtype))
+    np.testing.assert_array_equal(backend.fnn.activation_relu(input_data=x, dtype=dtype), np.maximum(x, 0))
+    x2 = x.reshape(5, 7 * 33)[:, :230]
+    np.testing.assert_array_equal(backend.fnn.activation_swiglu(input_data=x2, dtype=dtype), backend.fnn.activation_swiglu(x2, dtype=dtype))
+
+
+def test_gelu_epilogue_at_infinity_and_geglu_beyond_the_clip(backend):
+    """fused GELU at +-inf follows the shader's |x| > 50 rule (x, 0); the gated GELU keeps the unclipped
+    activation (the reference clips it at +-50, utils/vulkan_sentence_transformer.py:924-930: a documented deviation)."""
+    s = np.array([np.inf, -np.inf, 1e30, -1e30, 60.0, -60.0], np.float32)
+    x = np.zeros((len(s), 8), np.float32); x[:, 0] = s
+    W = np.zeros((4, 8), np.float32); W[:, 0] = 1
+    g = backend.fnn.fused_linear_gelu(np.nan_to_num(x, posinf=3e38, neginf=-3e38), W)[:, 0]
+    np.testing.assert_array_equal(g, np.array([3e38, 0, 1e30, 0, 60, 0], np.float32))
+    xg = np.zeros((2, 8), np.float32); xg[:, 0] = [60.0, 2.0]
+    out = backend.fnn.fused_geglu(xg, W, W)[:, 0]            # gate * gelu(up), both 60 / 2
+    np.testing.assert_allclose(out, [60.0 * 60.0, 2.0 * O.truth_gelu(np.array([2.0]))[0]], rtol=1e-5)
