@@ -96,3 +96,30 @@ def test_encoder_batch_independence_full_config(backend):
     assert np.isfinite(full).all()
     np.testing.assert_allclose(full[1:2], one, atol=2e-3)
     np.testing.assert_allclose(np.linalg.norm(full, axis=1), 1.0, atol=1e-4)
+
+
+def test_bench_shape_forward_b128(backend):
+    """The forward the benchmark times (BASELINE configs[2]: 12 layers, d=768, 12x64 heads, FFN 3072, batch 128 x seq 512,
+    bf16, M = 65536 rows per GEMM): sampled sequences equal their own batch-of-one runs through all 12 layers, and the
+    first layer at full batch width is checked against the float64 oracle of the same recipe with bf16 storage emulated."""
+    cfg = EncoderConfig()
+    w = random_bert_weights(cfg, seed=20260134)
+    rng = rng_for(3)
+    B, S = 128, 512
+    ids = rng.integers(0, cfg.vocab, (B, S))
+    enc = BertEncoder(backend, cfg, w, dtype="bf16")
+    h = enc.forward(ids, None, pool=False)
+    assert h.shape == (B, S, cfg.d_model) and np.isfinite(h).all()
+    for b in (0, 77, 127):
+        one = enc.forward(ids[b:b + 1], None, pool=False)
+        np.testing.assert_allclose(h[b:b + 1], one, atol=3e-2)          # same kernels, other tile walk: bf16 rounding only
+        assert O.max_rel(h[b:b + 1], one) < 5e-3
+    enc.release_activations()
+    cfg1 = EncoderConfig(layers=1)
+    w1 = dict(w, layers=w["layers"][:1])
+    enc1 = BertEncoder(backend, cfg1, w1, dtype="bf16")
+    h1 = enc1.forward(ids, None, pool=False)
+    for b in (3, 64, 126):
+        ref = truth_encoder(w1, cfg1, ids[b:b + 1], None, O.bf16_round)
+        assert O.max_rel(h1[b:b + 1], ref) < TOL_BF16, b
+    enc1.release_activations()
