@@ -66,6 +66,10 @@ SIGNATURES = {
     "grl_fa2_fwd": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64] + [c_void_p] * 5 + [c_float, c_int, c_int, c_float, c_float, c_void_p]),
     "grl_fa2_fwd_strided": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64] + [c_void_p] * 5 + [c_i64] * 4 + [c_float, c_int, c_int, c_float, c_float]),
     "grl_rope": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float]),
+    "grl_ln_fold": (c_int, [c_void_p, c_int, c_i64, c_i64] + [c_void_p] * 7),
+    "grl_ln_stats": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_float, c_void_p]),
+    "grl_ln_gemm_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 4 + [c_float, c_void_p, c_void_p]),
+    "grl_ln_glu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 7 + [c_float, c_void_p, c_void_p, c_int]),
     "grl_layernorm": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p]),
     "grl_add": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p, c_void_p]),
     "grl_gelu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),

@@ -140,8 +140,9 @@ class HipFNN:
 
     def fused_layernorm_linear(self, x, gamma, beta, weights, bias=None, eps=1e-5, dtype="fp32"):
         """Linear(LayerNorm(x)) (reference shaders/fused-layernorm-linear.glsl:67-128; the reference has no host
-        wrapper for it): the row-normalising kernel and the GEMM run back to back on the device, the
-        normalised rows never leave it (on the bf16 path they are rounded to bf16 between the two)."""
+        wrapper for it).  The normalised rows are never formed: gamma is folded into the weight, beta into the bias
+        (grl_ln_fold, once per call here, once per model in the encoder classes), one pass over x leaves
+        {rstd, rstd*mean} per row, and the GEMM on the raw rows applies them in its epilogue."""
         code = dtype_code(dtype)
         W = np.asarray(weights)
         if W.ndim != 2:
@@ -157,15 +158,18 @@ class HipFNN:
             raise ValueError(f"bias has {np.asarray(bias).size} elements, expected {N}")
         c = self.core
         es = 2 if code == L.GRL_BF16 else 4
+        if M == 0 or N == 0 or K == 0:
+            return self._fused_shape(x, np.zeros((M, N), np.float32))
         dx, dw, dg, dbt = c.upload(x2, code), c.upload(W, code), c.upload(g), c.upload(bt)
-        db = c.upload(np.asarray(bias).reshape(-1)) if bias is not None else None
-        dn, dy = c.alloc(max(M * K, 1) * es), c.alloc(max(M * N, 1) * es)
+        db = c.upload(np.asarray(bias, np.float32).reshape(-1)) if bias is not None else None
+        dws, dcs, dbf = c.alloc(N * K * es), c.alloc(N * 4), c.alloc(N * 4)
+        dst, dy = c.alloc(M * 8), c.alloc(M * N * es)
         try:
-            L.check(c.lib.grl_layernorm(c.ctx, code, M, K, dx.ptr, None, dg.ptr, dbt.ptr, float(eps), dn.ptr), "layernorm")
-            L.check(c.lib.grl_gemm_nt(c.ctx, code, code, M, N, K, dn.ptr, dw.ptr, db.ptr if db else None, dy.ptr, L.EPI_NONE), "gemm_nt")
+            L.check(c.lib.grl_ln_fold(c.ctx, code, N, K, dw.ptr, dg.ptr, dbt.ptr, db.ptr if db else None, dws.ptr, dcs.ptr, dbf.ptr), "ln_fold")
+            L.check(c.lib.grl_ln_gemm_nt(c.ctx, code, code, M, N, K, dx.ptr, dws.ptr, dcs.ptr, dbf.ptr, float(eps), dst.ptr, dy.ptr), "ln_gemm_nt")
             return self._fused_shape(x, c.download(dy, (M, N), code))
         finally:
-            for t in (dx, dw, dg, dbt, db, dn, dy):
+            for t in (dx, dw, dg, dbt, db, dws, dcs, dbf, dst, dy):
                 if t is not None:
                     t.free()
 

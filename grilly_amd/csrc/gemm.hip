@@ -17,6 +17,20 @@ static int dispatch_types(grl_ctx* c, GemmArgs& a, int in_dtype, int out_dtype, 
     return GRL_ERR_ARG;
 }
 
+extern template int dispatch_epi_ln<float, float>(grl_ctx*, GemmArgs&, int);
+extern template int dispatch_epi_ln<uint16_t, uint16_t>(grl_ctx*, GemmArgs&, int);
+extern template int dispatch_epi_ln<uint16_t, float>(grl_ctx*, GemmArgs&, int);
+extern template int dispatch_epi_ln<float, uint16_t>(grl_ctx*, GemmArgs&, int);
+
+static int dispatch_types_ln(grl_ctx* c, GemmArgs& a, int in_dtype, int out_dtype, int epi) {
+    if (in_dtype == GRL_F32 && out_dtype == GRL_F32) return dispatch_epi_ln<float, float>(c, a, epi);
+    if (in_dtype == GRL_BF16 && out_dtype == GRL_BF16) return dispatch_epi_ln<uint16_t, uint16_t>(c, a, epi);
+    if (in_dtype == GRL_BF16 && out_dtype == GRL_F32) return dispatch_epi_ln<uint16_t, float>(c, a, epi);
+    if (in_dtype == GRL_F32 && out_dtype == GRL_BF16) return dispatch_epi_ln<float, uint16_t>(c, a, epi);
+    grl_set_error("gemm: bad dtype in=%d out=%d", in_dtype, out_dtype);
+    return GRL_ERR_ARG;
+}
+
 static int check_dims(const char* who, int64_t M, int64_t N, int64_t K) {
     GRL_REQUIRE(M >= 0 && N >= 0 && K >= 0, GRL_ERR_SHAPE, "%s: negative dimension", who);
     GRL_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31), GRL_ERR_SHAPE, "%s: dimension exceeds 2^31-1", who);
@@ -113,6 +127,52 @@ extern "C" int grl_glu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, in
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     a.act = activation;
     return dispatch_types(c, a, in_dtype, out_dtype, EPI_GLU);
+}
+
+int grl_ln_stats(grl_ctx* c, int dtype, int64_t rows, int64_t F, const void* x, float eps, float* stats);
+
+// LayerNorm folded into the GEMM: row statistics of x (one pass over x, 8 bytes per row out), then the GEMM on the
+// raw rows with the scaled weight; the normalised rows are never formed.
+extern "C" int grl_ln_gemm_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                              const void* W_scaled, const float* colsum, const float* bias_folded, float eps,
+                              float* stats, void* out) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_ln_gemm_nt: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_ln_gemm_nt: bad dtype");
+    int rc = check_dims("grl_ln_gemm_nt", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    GRL_REQUIRE(out && K > 0 && x && W_scaled && colsum && stats, GRL_ERR_ARG, "grl_ln_gemm_nt: null argument or K == 0");
+    rc = grl_ln_stats(c, in_dtype, M, K, x, eps, stats);
+    if (rc) return rc;
+    GemmArgs a{};
+    a.A = x; a.W = W_scaled; a.bias = bias_folded; a.C = out;
+    a.ln_stats = stats; a.ln_c = colsum;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    return dispatch_types_ln(c, a, in_dtype, out_dtype, EPI_NONE);
+}
+
+extern "C" int grl_ln_glu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                             const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
+                             const float* bias_gate_folded, const float* bias_up_folded, float eps, float* stats,
+                             void* out, int activation) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_ln_glu_nt: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_ln_glu_nt: bad dtype");
+    GRL_REQUIRE(activation == GRL_EPI_SILU || activation == GRL_EPI_RELU || activation == GRL_EPI_GELU, GRL_ERR_ARG,
+                "grl_ln_glu_nt: activation must be GRL_EPI_SILU, GRL_EPI_RELU or GRL_EPI_GELU (got %d)", activation);
+    int rc = check_dims("grl_ln_glu_nt", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    GRL_REQUIRE(out && K > 0 && x && Wg_scaled && Wu_scaled && colsum_gate && colsum_up && bias_gate_folded && bias_up_folded && stats,
+                GRL_ERR_ARG, "grl_ln_glu_nt: null argument or K == 0");
+    rc = grl_ln_stats(c, in_dtype, M, K, x, eps, stats);
+    if (rc) return rc;
+    GemmArgs a{};
+    a.A = x; a.W = Wg_scaled; a.W2 = Wu_scaled; a.C = out;
+    a.bias = bias_gate_folded; a.bias2 = bias_up_folded;
+    a.ln_stats = stats; a.ln_c = colsum_gate; a.ln_c2 = colsum_up;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.act = activation;
+    return dispatch_types_ln(c, a, in_dtype, out_dtype, EPI_GLU);
 }
 
 extern "C" int grl_swiglu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,

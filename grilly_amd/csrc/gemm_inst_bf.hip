@@ -2,3 +2,4 @@
 #include "gemm_kernels.hpp"
 
 template int dispatch_epi<uint16_t, float>(grl_ctx*, GemmArgs&, int);
+template int dispatch_epi_ln<uint16_t, float>(grl_ctx*, GemmArgs&, int);

@@ -2,3 +2,4 @@
 #include "gemm_kernels.hpp"
 
 template int dispatch_epi<float, uint16_t>(grl_ctx*, GemmArgs&, int);
+template int dispatch_epi_ln<float, uint16_t>(grl_ctx*, GemmArgs&, int);

@@ -2,3 +2,4 @@
 #include "gemm_kernels.hpp"
 
 template int dispatch_epi<float, float>(grl_ctx*, GemmArgs&, int);
+template int dispatch_epi_ln<float, float>(grl_ctx*, GemmArgs&, int);

@@ -42,6 +42,11 @@ struct GemmArgs {
     int act;             // run-time activation code of the EPI_RT / dual epilogues (a GRL_EPI_* value)
     float alpha, beta;   // RoSwish parameters
     const void* residual; // (M,N) of the output type, added to the result (EPI_RES), else null
+    // LayerNorm folded into the GEMM (template flag LN): A holds the raw rows, W the weight scaled by gamma;
+    // sum_k LN(x)[m,k] W0[n,k] = rstd_m * (acc[m,n] - mean_m * c[n]) + sum_k beta[k] W0[n,k], c[n] = sum_k W[n,k]
+    const float* ln_stats; // (M,2): {rstd, rstd*mean} per row
+    const float* ln_c;     // (N) column sums of the scaled weight W
+    const float* ln_c2;    // (N) the same for W2, else null
 };
 
 // Epilogue template codes.  NONE / GELU / SILU are compiled in (the encoder's hot shapes); EPI_RT picks
@@ -144,13 +149,15 @@ template <> __device__ __forceinline__ u32x4 add_chunk<uint16_t>(u32x4 c, u32x4 
 // (8- or 16-byte stores).  Every index into the accumulators is a compile-time constant so
 // they stay in registers.  Used for ragged N, for the SwiGLU pre-activation outputs and by the
 // staged kernel.
-template <typename OutT, int TM, int TN, int TNO, int WM, int WNO, int EPI, bool DUAL>
+template <typename OutT, int TM, int TN, int TNO, int WM, int WNO, int EPI, bool DUAL, bool LN = false>
 __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const GemmArgs& p, int m0, int n0, int wm, int wn, int li, int lg) {
     OutT* C = (OutT*)p.C;
     const bool vec_ok = (p.N & 3) == 0;
     static_for<TM>([&](auto ia) {
         constexpr int a = decltype(ia)::value;
         const int m = m0 + wm * WM + a * 32 + li;
+        float rs = 1.f, rsm = 0.f;
+        if (LN && m < p.M) { rs = p.ln_stats[2 * (int64_t)m]; rsm = p.ln_stats[2 * (int64_t)m + 1]; }
         static_for<TNO>([&](auto ib) {
             constexpr int b = decltype(ib)::value;
             static_for<4>([&](auto iq) {
@@ -162,6 +169,10 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
                     for (int e = 0; e < 4; ++e) {
                         v[e] = acc[a][b][4 * q + e];
                         u[e] = DUAL ? acc[a][DUAL ? b + TNO : b][4 * q + e] : 0.f;
+                        if (LN && n + e < p.N) {
+                            v[e] = v[e] * rs - rsm * p.ln_c[n + e];
+                            if (DUAL) u[e] = u[e] * rs - rsm * p.ln_c2[n + e];
+                        }
                     }
                     const int64_t o = (int64_t)m * p.N + n;
                     if (vec_ok) {
@@ -212,7 +223,7 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
 
 // BN counts LDS rows of the weight tile; with DUAL it is 2x the output-column count of the
 // tile (first half gate rows, second half up rows).
-template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL>
+template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL, bool LN = false>
 __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
     constexpr int NT = WGM * WGN * 64;
     constexpr int EPC = 16 / (int)sizeof(T);     // elements per 16-byte chunk
@@ -340,7 +351,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
         __syncthreads();
     }
 
-    epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
+    epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL, LN>(acc, p, m0, n0, wm, wn, li, lg);
 }
 
 // =====================================================================================
@@ -365,7 +376,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
 //   swizzled by row) -> 16-byte row-contiguous global stores, 32 output rows per wave-row
 //   per pass, two staging regions used alternately so a pass costs one barrier.
 // =====================================================================================
-template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL>
+template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL, bool LN = false>
 __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p) {
     constexpr int NW = WGM * WGN, NT = NW * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -383,7 +394,11 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     constexpr int RG = WGM * 32 * CROWB;                    // one staging region
     constexpr int NREG = 2 * RG <= STAGE ? 2 : 1;
     static_assert(RG <= STAGE && (CPR & (CPR - 1)) == 0, "output staging must fit in LDS stage 1");
-    constexpr int BIASB = BN * 4;                           // one tile's bias slice(s), fp32
+    // one tile's per-column vectors, fp32: bias slice(s); with LN also the column sums c (c2) behind them and the
+    // tile's BM row-statistics pairs
+    constexpr int COLB = BN * 4;
+    constexpr int BIASB = LN ? 2 * COLB + BM * 8 : COLB;
+    static_assert(!LN || NW >= 4, "the per-tile vectors are fetched by distinct waves");
     __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + 2 * BIASB];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -460,6 +475,30 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + 2 * STAGE + buf * BIASB + (w2 ? BNO * 4 : 0)),
                                                      16, lane * 16, 0, 0, 0);
         }
+        if constexpr (LN) {
+            // wave 1: c[n0 .. n0+BNO), the second wave of the upper half: c2
+            const bool w3 = wave == 1, w4 = DUAL && wave == NW / 2 + 1;
+            if ((w3 || w4) && lane < BNO / 4) {
+                const float* src = (w4 ? p.ln_c2 : p.ln_c) + n0t;
+                int left = (p.N - n0t) * 4;
+                __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, left > 0 ? left : 0, 0x00020000);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + 2 * STAGE + buf * BIASB + COLB + (w4 ? BNO * 4 : 0)),
+                                                         16, lane * 16, 0, 0, 0);
+            }
+        }
+    };
+    // rows m0t .. m0t+BM of the statistics (rows past M read zero), fetched by the last wave
+    auto issue_stats = [&](int m0t, int buf) {
+        if constexpr (LN) {
+            if (wave == NW - 1) {
+                int left = (p.M - m0t) * 8;
+                __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)(p.ln_stats + 2 * (int64_t)m0t), 0, left > 0 ? left : 0, 0x00020000);
+#pragma unroll
+                for (int j = 0; j < BM * 8 / 1024; ++j)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + 2 * STAGE + buf * BIASB + 2 * COLB + j * 1024),
+                                                             16, j * 1024 + lane * 16, 0, 0, 0);
+            }
+        }
     };
 
     int rowX[TM], rowW[TN];
@@ -485,6 +524,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     issue(rsA, rsW, 0);
     int bbuf = 0;
     issue_bias(n0, bbuf);
+    issue_stats(m0, bbuf);
 
     for (;;) {
         // not zeroed: the first slab's multiplications start every accumulator from a constant zero
@@ -543,6 +583,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
         if (has_next) {
             issue(rsAn, rsWn, 0);
             issue_bias(n0n, bbuf ^ 1);
+            issue_stats(m0n, bbuf ^ 1);
         }
 
         if (staged) {
@@ -551,15 +592,19 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             char* stg = lds + STAGE;
             const char* bias_lds = lds + 2 * STAGE + bbuf * BIASB;
             // bias of this lane's 4-column groups, once per tile (columns past N hold zero)
-            f32x4 bv1[TNO][4], bv2[TNO][4];
+            // (with the folded LayerNorm every per-column vector is read from LDS where it is used instead: the
+            // epilogue then keeps nothing more in registers across its bands than the plain one)
+            f32x4 bv1[LN ? 1 : TNO][4], bv2[LN ? 1 : TNO][4];
+            if constexpr (!LN) {
 #pragma unroll
-            for (int b = 0; b < TNO; ++b)
+                for (int b = 0; b < TNO; ++b)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
-                    bv1[b][q] = p.bias ? *(const f32x4*)(bias_lds + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
-                    if (DUAL) bv2[b][q] = p.bias2 ? *(const f32x4*)(bias_lds + BNO * 4 + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
-                }
+                    for (int q = 0; q < 4; ++q) {
+                        const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
+                        bv1[b][q] = p.bias ? *(const f32x4*)(bias_lds + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                        if (DUAL) bv2[b][q] = p.bias2 ? *(const f32x4*)(bias_lds + BNO * 4 + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                    }
+            }
             constexpr int TOTAL = WGM * 32 * CPR;
             static_assert(TOTAL % NT == 0, "staged chunks divide over the threads");
             constexpr int PER = TOTAL / NT;
@@ -570,6 +615,13 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             auto stage_band = [&](auto ia) {
                 constexpr int a = decltype(ia)::value;
                 char* crow = stg + (NREG == 2 ? (a & 1) * RG : 0) + r_w * CROWB;
+                // LN: this row's {rstd, rstd*mean} once per band, the column sums from LDS where they are used:
+                // nothing more stays live across the bands than without the folded LayerNorm
+                float rs = 1.f, rsm = 0.f;
+                if constexpr (LN) {
+                    const float* st = (const float*)(bias_lds + 2 * COLB) + 2 * (wm * WM + a * 32 + li);
+                    rs = st[0]; rsm = st[1];
+                }
                 static_for<TNO>([&](auto ib) {
                     constexpr int b = decltype(ib)::value;
                     static_for<4>([&](auto iq) {
@@ -577,10 +629,27 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                         const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
                         float v[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] + bv1[b][q][e];
+                        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] + (LN ? 0.f : bv1[LN ? 0 : b][q][e]);
+                        f32x4 c2 = {0.f, 0.f, 0.f, 0.f}, b2 = {0.f, 0.f, 0.f, 0.f};
+                        if constexpr (LN) {
+                            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                            const f32x4 c1 = *(const f32x4*)(bias_lds + COLB + nl * 4);
+                            const f32x4 b1 = p.bias ? *(const f32x4*)(bias_lds + nl * 4) : zero;
+                            if constexpr (DUAL) {
+                                c2 = *(const f32x4*)(bias_lds + COLB + BNO * 4 + nl * 4);
+                                b2 = p.bias2 ? *(const f32x4*)(bias_lds + BNO * 4 + nl * 4) : zero;
+                            }
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] * rs + (b1[e] - rsm * c1[e]);
+                        }
                         if (DUAL) {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = glu_apply(v[e], acc[a][DUAL ? b + TNO : b][4 * q + e] + bv2[b][q][e], p);
+                            for (int e = 0; e < 4; ++e) {
+                                float up = acc[a][DUAL ? b + TNO : b][4 * q + e];
+                                if constexpr (LN) up = up * rs + (b2[e] - rsm * c2[e]);
+                                else up += bv2[LN ? 0 : b][q][e];
+                                v[e] = glu_apply(v[e], up, p);
+                            }
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
@@ -687,7 +756,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                 });
             }
         } else {
-            epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL>(acc, p, m0, n0, wm, wn, li, lg);
+            epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL, LN>(acc, p, m0, n0, wm, wn, li, lg);
         }
         if (!has_next) break;
         pid = npid; m0 = m0n; n0 = n0n; rsA = rsAn; rsW = rsWn; rsWp = rsWpn; bbuf ^= 1;
@@ -696,7 +765,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
 
 // ---- any shape / any alignment: one thread per output, ascending-k fp32 sum (the summation
 // order of shaders/fnn-linear.glsl:45-49).  Used only when rows are not 16-byte aligned.
-template <typename T, typename OutT, int EPI, bool DUAL>
+template <typename T, typename OutT, int EPI, bool DUAL, bool LN = false>
 __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmArgs p) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (int64_t)p.M * p.N) return;
@@ -705,11 +774,14 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmArgs p) {
     const T* w = (const T*)p.W + (int64_t)n * p.K;
     float s = 0.f;
     for (int k = 0; k < p.K; ++k) s += elem<T>::ld(a + k) * elem<T>::ld(w + k);
+    float rs = 1.f, rsm = 0.f;
+    if (LN) { rs = p.ln_stats[2 * (int64_t)m]; rsm = p.ln_stats[2 * (int64_t)m + 1]; s = s * rs - rsm * p.ln_c[n]; }
     if (p.bias) s += p.bias[n];
     if (DUAL) {
         const T* w2 = (const T*)p.W2 + (int64_t)n * p.K;
         float u = 0.f;
         for (int k = 0; k < p.K; ++k) u += elem<T>::ld(a + k) * elem<T>::ld(w2 + k);
+        if (LN) u = u * rs - rsm * p.ln_c2[n];
         if (p.bias2) u += p.bias2[n];
         if (p.cache1) p.cache1[idx] = s;
         if (p.cache2) p.cache2[idx] = u;
@@ -722,15 +794,16 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmArgs p) {
 }
 
 // ------------------------------------------------------------------ host dispatch
-template <typename T, typename OutT, int EPI, bool DUAL>
+template <typename T, typename OutT, int EPI, bool DUAL, bool LN = false>
 static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     const int64_t epc = 16 / (int64_t)sizeof(T);
     const bool aligned = (a.K % epc == 0) && ((((uintptr_t)a.A) | ((uintptr_t)a.W) | ((uintptr_t)a.W2)) & 15u) == 0 &&
-                         ((((uintptr_t)a.C) | ((uintptr_t)a.bias) | ((uintptr_t)a.bias2) | ((uintptr_t)a.cache1) | ((uintptr_t)a.cache2) | ((uintptr_t)a.residual)) & 15u) == 0;
+                         ((((uintptr_t)a.C) | ((uintptr_t)a.bias) | ((uintptr_t)a.bias2) | ((uintptr_t)a.cache1) | ((uintptr_t)a.cache2) | ((uintptr_t)a.residual) |
+                           ((uintptr_t)a.ln_stats) | ((uintptr_t)a.ln_c) | ((uintptr_t)a.ln_c2)) & 15u) == 0;
     if (!aligned) {
         int64_t total = (int64_t)a.M * a.N;
         GRL_REQUIRE((total + 255) / 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: unaligned problem too large for the scalar kernel");
-        hipLaunchKernelGGL((gemm_nt_scalar_kernel<T, OutT, EPI, DUAL>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, a);
+        hipLaunchKernelGGL((gemm_nt_scalar_kernel<T, OutT, EPI, DUAL, LN>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, c->stream, a);
         GRL_CHECK_LAUNCH();
         return GRL_OK;
     }
@@ -754,19 +827,19 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     switch (variant) {
         case 1:
             a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
-            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 256, 256, 2, 2, EPI, DUAL>), dim3((unsigned)(big_m * big_n)), dim3(256), 0, c->stream, a);
+            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 256, 256, 2, 2, EPI, DUAL, LN>), dim3((unsigned)(big_m * big_n)), dim3(256), 0, c->stream, a);
             break;
         case 2:
             a.tiles_m = (int)sm; a.tiles_n = (int)sn;
-            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)(sm * sn)), dim3(256), 0, c->stream, a);
+            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL, LN>), dim3((unsigned)(sm * sn)), dim3(256), 0, c->stream, a);
             break;
         case 3:
             a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
-            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 256, 256, 2, 4, EPI, DUAL>), dim3((unsigned)std::min<int64_t>(big_m * big_n, cus)), dim3(512), 0, c->stream, a);
+            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 256, 256, 2, 4, EPI, DUAL, LN>), dim3((unsigned)std::min<int64_t>(big_m * big_n, cus)), dim3(512), 0, c->stream, a);
             break;
         default:
             a.tiles_m = (int)sm; a.tiles_n = (int)sn;
-            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL>), dim3((unsigned)std::min<int64_t>(sm * sn, 2 * cus)), dim3(256), 0, c->stream, a);
+            hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 128, 128, 2, 2, EPI, DUAL, LN>), dim3((unsigned)std::min<int64_t>(sm * sn, 2 * cus)), dim3(256), 0, c->stream, a);
             break;
     }
     GRL_CHECK_LAUNCH();
@@ -784,6 +857,17 @@ int dispatch_epi(grl_ctx* c, GemmArgs& a, int epi) {
         case EPI_RES: return launch_gemm<T, OutT, EPI_RES, false>(c, a);
     }
     grl_set_error("gemm: bad epilogue %d", epi);
+    return GRL_ERR_ARG;
+}
+
+// the LayerNorm-folded forms: plain (bias only) and the gated dual-weight epilogue
+template <typename T, typename OutT>
+int dispatch_epi_ln(grl_ctx* c, GemmArgs& a, int epi) {
+    switch (epi) {
+        case EPI_NONE: return launch_gemm<T, OutT, EPI_NONE, false, true>(c, a);
+        case EPI_GLU: return launch_gemm<T, OutT, EPI_GLU, true, true>(c, a);
+    }
+    grl_set_error("gemm: epilogue %d has no LayerNorm-folded form", epi);
     return GRL_ERR_ARG;
 }
 

@@ -42,7 +42,8 @@ __device__ __forceinline__ float wave_sum(float v) { return group_sum<64>(v); } 
 // between the mean pass, the variance pass and the normalise pass, so the row is read
 // from HBM exactly once (the reference makes three dispatches over it,
 // shaders/fnn-layernorm.glsl:44-103).
-template <typename T, int MAXC, bool HAS_RES>
+// STATS: instead of the normalised row, {1/sd, mean/sd} goes to ((float*)y)[2*row ..] (what the LayerNorm-folded GEMM reads).
+template <typename T, int MAXC, bool HAS_RES, bool STATS = false>
 __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     const T* x, const T* res, const float* __restrict__ gamma,
     const float* __restrict__ beta, T* y, int64_t rows, int F, float eps) {
@@ -85,6 +86,10 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     }
     const float var = wave_sum(q) / (float)F;
     const float sd = sqrtf(var + eps);
+    if constexpr (STATS) {
+        if (lane == 0) { float2 o = {1.0f / sd, mean / sd}; ((float2*)y)[row] = o; }
+        return;
+    }
     T* yr = y + row * (int64_t)F;
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
@@ -102,7 +107,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
 
 // bf16 rows with F % 8 == 0: 16-byte streaming accesses (8 values), LPR lanes per row, i.e. 64/LPR rows per
 // wave (two rows per wave for F <= 1024 keeps 96 B of loads in flight per lane at F = 768 instead of 48).
-template <int MAXC, bool HAS_RES, int LPR>
+template <int MAXC, bool HAS_RES, int LPR, bool STATS = false>
 __global__ __launch_bounds__(256) void layernorm_bf16x8_kernel(
     const uint16_t* x, const uint16_t* res, const float* __restrict__ gamma,
     const float* __restrict__ beta, uint16_t* y, int64_t rows, int F, float eps) {
@@ -146,6 +151,10 @@ __global__ __launch_bounds__(256) void layernorm_bf16x8_kernel(
     }
     q = group_sum<LPR>(q);
     const float sd = sqrtf(q / (float)F + eps);
+    if constexpr (STATS) {
+        if (sub == 0) { float2 o = {1.0f / sd, mean / sd}; ((float2*)y)[row] = o; }
+        return;
+    }
     uint16_t* yr = y + row * (int64_t)F;
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
@@ -168,7 +177,7 @@ __global__ __launch_bounds__(256) void layernorm_bf16x8_kernel(
 }
 
 // Any F: three passes over the row from global memory (the second and third hit L2).
-template <typename T, bool HAS_RES>
+template <typename T, bool HAS_RES, bool STATS = false>
 __global__ __launch_bounds__(256) void layernorm_rows_generic_kernel(
     const T* x, const T* res, const float* __restrict__ gamma,
     const float* __restrict__ beta, T* y, int64_t rows, int F, float eps) {
@@ -186,6 +195,10 @@ __global__ __launch_bounds__(256) void layernorm_rows_generic_kernel(
         q += d * d;
     }
     const float sd = sqrtf(wave_sum(q) / (float)F + eps);
+    if constexpr (STATS) {
+        if (lane == 0) { float2 o = {1.0f / sd, mean / sd}; ((float2*)y)[row] = o; }
+        return;
+    }
     T* yr = y + row * (int64_t)F;
     for (int f = lane; f < F; f += 64) {
         float v = elem<T>::ld(xr + f) + (HAS_RES ? elem<T>::ld(rr + f) : 0.f);
@@ -249,6 +262,90 @@ extern "C" int grl_layernorm(grl_ctx* c, int dtype, int64_t rows, int64_t F, con
     if (rows == 0) return GRL_OK;
     return dtype == GRL_F32 ? launch_layernorm<float>(c, rows, F, x, residual, gamma, beta, eps, y)
                             : launch_layernorm<uint16_t>(c, rows, F, x, residual, gamma, beta, eps, y);
+}
+
+// Row statistics for the LayerNorm-folded GEMM: stats[2*row] = 1/sd, stats[2*row+1] = mean/sd with the same two-pass
+// mean / variance as grl_layernorm (one read of x, 8 bytes per row written).
+template <typename T>
+static int launch_ln_stats(grl_ctx* c, int64_t rows, int64_t F, const void* x, float eps, float* stats) {
+    dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    const T* X = (const T*)x; T* Y = (T*)stats;
+    const float* nil = nullptr;
+    const bool fast = (F % 4 == 0) && F <= 64 * 4 * 8 && aligned16(x) && ((F * sizeof(T)) % 8 == 0);
+    if constexpr (sizeof(T) == 2) {
+        if (fast && F % 8 == 0 && F <= 4096) {
+            const int nch8 = (int)(F / 8);
+#define LNS16_LAUNCH(MAXC, LPR)                                                                              \
+    do {                                                                                                     \
+        dim3 g16((unsigned)((rows + 4 * (64 / LPR) - 1) / (4 * (64 / LPR))));                                \
+        hipLaunchKernelGGL((layernorm_bf16x8_kernel<MAXC, false, LPR, true>), g16, block, 0, c->stream, X, X, nil, nil, Y, rows, (int)F, eps); \
+    } while (0)
+            if (nch8 <= 32 * 2) LNS16_LAUNCH(2, 32);
+            else if (nch8 <= 32 * 4) LNS16_LAUNCH(4, 32);
+            else if (nch8 <= 64 * 4) LNS16_LAUNCH(4, 64);
+            else LNS16_LAUNCH(8, 64);
+#undef LNS16_LAUNCH
+            GRL_CHECK_LAUNCH();
+            return GRL_OK;
+        }
+    }
+    if (fast) {
+        const int nch = (int)(F / 4), maxc = (nch + 63) / 64;
+        if (maxc <= 2) hipLaunchKernelGGL((layernorm_rows_kernel<T, 2, false, true>), grid, block, 0, c->stream, X, X, nil, nil, Y, rows, (int)F, eps);
+        else if (maxc <= 3) hipLaunchKernelGGL((layernorm_rows_kernel<T, 3, false, true>), grid, block, 0, c->stream, X, X, nil, nil, Y, rows, (int)F, eps);
+        else if (maxc <= 4) hipLaunchKernelGGL((layernorm_rows_kernel<T, 4, false, true>), grid, block, 0, c->stream, X, X, nil, nil, Y, rows, (int)F, eps);
+        else hipLaunchKernelGGL((layernorm_rows_kernel<T, 8, false, true>), grid, block, 0, c->stream, X, X, nil, nil, Y, rows, (int)F, eps);
+    } else {
+        hipLaunchKernelGGL((layernorm_rows_generic_kernel<T, false, true>), grid, block, 0, c->stream, X, X, nil, nil, Y, rows, (int)F, eps);
+    }
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+extern "C" int grl_ln_stats(grl_ctx* c, int dtype, int64_t rows, int64_t F, const void* x, float eps, float* stats) {
+    GRL_REQUIRE(c && x && stats, GRL_ERR_ARG, "grl_ln_stats: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_ln_stats: bad dtype %d", dtype);
+    GRL_REQUIRE(rows >= 0 && F > 0 && F < (1 << 30), GRL_ERR_SHAPE, "grl_ln_stats: bad shape rows=%lld F=%lld", (long long)rows, (long long)F);
+    GRL_REQUIRE(rows < ((int64_t)1 << 33), GRL_ERR_SHAPE, "grl_ln_stats: too many rows");
+    GRL_REQUIRE((((uintptr_t)stats) & 15u) == 0, GRL_ERR_ARG, "grl_ln_stats: stats must be 16-byte aligned");
+    if (rows == 0) return GRL_OK;
+    return dtype == GRL_F32 ? launch_ln_stats<float>(c, rows, F, x, eps, stats) : launch_ln_stats<uint16_t>(c, rows, F, x, eps, stats);
+}
+
+// Weight side of the LayerNorm-folded GEMM, once per weight: W_scaled[n,k] = gamma[k]*W[n,k] (rounded to the storage
+// type), colsum[n] = sum_k W_scaled[n,k] (of the rounded values, which is what the GEMM multiplies), bias_folded[n] =
+// bias[n] + sum_k beta[k]*W[n,k].  One wave per weight row.
+template <typename T>
+__global__ __launch_bounds__(256) void ln_fold_kernel(const T* W, const float* gamma, const float* beta, const float* bias,
+                                                      T* Ws, float* colsum, float* bias_folded, int64_t N, int K) {
+    const int lane = threadIdx.x & 63;
+    const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    const T* w = W + n * (int64_t)K;
+    T* ws = Ws + n * (int64_t)K;
+    float cs = 0.f, ds = 0.f;
+    for (int k = lane; k < K; k += 64) {
+        const float wv = elem<T>::ld(w + k);
+        elem<T>::st(ws + k, gamma[k] * wv);
+        cs += elem<T>::ld(ws + k);          // the value as stored
+        ds += beta[k] * wv;
+    }
+    cs = wave_sum(cs); ds = wave_sum(ds);
+    if (lane == 0) { colsum[n] = cs; bias_folded[n] = ds + (bias ? bias[n] : 0.f); }
+}
+
+extern "C" int grl_ln_fold(grl_ctx* c, int dtype, int64_t N, int64_t K, const void* W, const float* gamma, const float* beta,
+                           const float* bias, void* W_scaled, float* colsum, float* bias_folded) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_ln_fold: null context");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_ln_fold: bad dtype %d", dtype);
+    GRL_REQUIRE(N >= 0 && K > 0 && K < (1LL << 31) && N < (1LL << 31), GRL_ERR_SHAPE, "grl_ln_fold: bad shape N=%lld K=%lld", (long long)N, (long long)K);
+    if (N == 0) return GRL_OK;
+    GRL_REQUIRE(W && gamma && beta && W_scaled && colsum && bias_folded, GRL_ERR_ARG, "grl_ln_fold: null argument");
+    dim3 grid((unsigned)((N + 3) / 4)), block(256);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(ln_fold_kernel<float>, grid, block, 0, c->stream, (const float*)W, gamma, beta, bias, (float*)W_scaled, colsum, bias_folded, N, (int)K);
+    else hipLaunchKernelGGL(ln_fold_kernel<uint16_t>, grid, block, 0, c->stream, (const uint16_t*)W, gamma, beta, bias, (uint16_t*)W_scaled, colsum, bias_folded, N, (int)K);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
 }
 
 // ------------------------------------------------------------------ elementwise

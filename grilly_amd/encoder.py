@@ -210,13 +210,12 @@ class PreNormEncoder:
         pooled = x[:, 0, :] (first token), L2-normalised                       (:1179-1183, :1194-1201)
 
     Built from the same entry points as the post-LN encoder: the projection GEMMs, attention with the
-    rotate-half rotation fused, LayerNorm, the dual GEMM with the GELU gate, and the GEMM that adds the
-    residual stream in place.
+    rotate-half rotation fused, the dual GEMM with the GELU gate, and the GEMM that adds the residual stream in
+    place.  The LayerNorm in front of the MLP is folded into that dual GEMM (gamma into the two weights, beta into
+    the biases, once at construction; the GEMM reads the residual stream itself and applies each row's mean and
+    1/sd in its epilogue), so the normalised rows are never written.
     The packed Wqkv is one GEMM; attention reads its three column blocks in place.  The +-50 / +-1e6 clips the
     reference puts around the gate (:924-930) are not applied: they only act beyond those magnitudes."""
-
-    _MATS = ("w_qkv", "w_o", "w_ff_in", "w_ff_gate", "w_ff2")
-    _VECS = ("b_qkv", "b_o", "ffn_ln_g", "ffn_ln_b", "b_ff_in", "b_ff_gate", "b_ff2")
 
     def __init__(self, core, cfg, weights, dtype="fp32"):
         self.core = core.core if hasattr(core, "core") else core
@@ -235,9 +234,20 @@ class PreNormEncoder:
         if weights.get("final_ln_g") is not None:
             self.final = (vec(weights["final_ln_g"]), vec(weights["final_ln_b"]))
         self.layers = []
+        es = 2 if self.code == L.GRL_BF16 else 4
+        d, ff = cfg.d_model, cfg.d_ff
         for lw in weights["layers"]:
-            entry = {k: up(lw[k], self.code) for k in self._MATS}
-            entry.update({k: vec(lw[k]) for k in self._VECS})
+            entry = {k: up(lw[k], self.code) for k in ("w_qkv", "w_o", "w_ff2")}
+            entry.update({k: vec(lw[k]) for k in ("b_qkv", "b_o", "b_ff2")})
+            g, bt = c.upload(np.asarray(lw["ffn_ln_g"], np.float32).reshape(-1)), c.upload(np.asarray(lw["ffn_ln_b"], np.float32).reshape(-1))
+            for name in ("gate", "in"):
+                raw = c.upload(lw["w_ff_" + name], self.code)
+                b = c.upload(np.asarray(lw["b_ff_" + name], np.float32).reshape(-1))
+                ws, cs, bf = self._own(c.alloc(ff * d * es)), self._own(c.alloc(ff * 4)), self._own(c.alloc(ff * 4))
+                L.check(c.lib.grl_ln_fold(c.ctx, self.code, ff, d, raw.ptr, g.ptr, bt.ptr, b.ptr, ws.ptr, cs.ptr, bf.ptr), "fold mlp layernorm")
+                entry["ws_" + name], entry["cs_" + name], entry["bf_" + name] = ws, cs, bf
+                raw.free(); b.free()
+            g.free(); bt.free()
             self.layers.append(entry)
         self._shape = None
 
@@ -252,7 +262,8 @@ class PreNormEncoder:
         cfg, c = self.cfg, self.core
         es = 2 if self.code == L.GRL_BF16 else 4
         act = B * S * cfg.d_model * es
-        self.x, self.att, self.t = (c.alloc(act) for _ in range(3))
+        self.x, self.att = (c.alloc(act) for _ in range(2))
+        self.stats = c.alloc(B * S * 8)                # {1/sd, mean/sd} per row, for the GEMM that carries the MLP's LayerNorm
         self.qkv = c.alloc(3 * act)                    # packed (M, 3d): Q, K, V are its three column blocks
         self.h = c.alloc(B * S * cfg.d_ff * es)
         self.ids = c.alloc(B * S * 4)
@@ -265,7 +276,7 @@ class PreNormEncoder:
 
     def release_activations(self):
         if self._shape is not None:
-            for b in (self.x, self.qkv, self.att, self.t, self.h, self.ids, self.mask, self.first, self.pooled):
+            for b in (self.x, self.qkv, self.att, self.stats, self.h, self.ids, self.mask, self.first, self.pooled):
                 b.free()
             self._shape = None
 
@@ -307,11 +318,10 @@ class PreNormEncoder:
                     "attention")
             L.check(lib.grl_gemm_nt_res(c.ctx, code, code, M, d, d, self.att.ptr, w["w_o"].ptr, w["b_o"].ptr, self.x.ptr,
                                         self.x.ptr), "output projection + residual")
-            L.check(lib.grl_layernorm(c.ctx, code, M, d, self.x.ptr, None, w["ffn_ln_g"].ptr, w["ffn_ln_b"].ptr, cfg.eps,
-                                      self.t.ptr), "mlp layernorm")
-            # the dual GEMM activates its second ("up") operand: that is the first half of Wi here
-            L.check(lib.grl_glu_nt(c.ctx, code, code, M, ff, d, self.t.ptr, w["w_ff_gate"].ptr, w["w_ff_in"].ptr,
-                                   w["b_ff_gate"].ptr, w["b_ff_in"].ptr, self.h.ptr, None, None, L.EPI_GELU), "geglu")
+            # LayerNorm + dual GEMM; the dual GEMM activates its second ("up") operand: that is the first half of Wi here
+            L.check(lib.grl_ln_glu_nt(c.ctx, code, code, M, ff, d, self.x.ptr, w["ws_gate"].ptr, w["ws_in"].ptr,
+                                      w["cs_gate"].ptr, w["cs_in"].ptr, w["bf_gate"].ptr, w["bf_in"].ptr, cfg.eps,
+                                      self.stats.ptr, self.h.ptr, L.EPI_GELU), "mlp layernorm + geglu")
             L.check(lib.grl_gemm_nt_res(c.ctx, code, code, M, d, ff, self.h.ptr, w["w_ff2"].ptr, w["b_ff2"].ptr, self.x.ptr,
                                         self.x.ptr), "mlp output + residual")
         if self.final is not None:

@@ -218,6 +218,26 @@ int grl_rope(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D
 int grl_layernorm(grl_ctx* ctx, int dtype, int64_t rows, int64_t F, const void* x,
                   const void* residual, const float* gamma, const float* beta, float eps, void* y);
 
+/* ---- Linear(LayerNorm(x)) without forming the normalised rows --------------------------
+ * Replaces the shader shaders/fused-layernorm-linear.glsl:67-128 (per-row mean / variance, then the GEMM on the
+ * normalised row inside one dispatch).  Here the normalisation moves into the GEMM epilogue:
+ *     sum_k LN(x)[m,k] W[n,k] = rstd_m * (sum_k x[m,k] Ws[n,k] - mean_m * c[n]) + b'[n]
+ * with Ws[n,k] = gamma[k] W[n,k], c[n] = sum_k Ws[n,k], b'[n] = bias[n] + sum_k beta[k] W[n,k].
+ * grl_ln_fold builds Ws (storage type), c and b' once per weight; grl_ln_stats writes {rstd, rstd*mean} per row
+ * (one read of x, 8 bytes out per row); grl_ln_gemm_nt runs grl_ln_stats into `stats` (2*M floats, 16-byte aligned,
+ * caller-owned) and then the GEMM on the raw x.  grl_ln_glu_nt is the gated form act(up)*gate of grl_glu_nt on
+ * LN(x), both weights folded with the same gamma / beta.  Statistics as grl_layernorm (biased variance, two passes). */
+int grl_ln_fold(grl_ctx* ctx, int dtype, int64_t N, int64_t K, const void* W, const float* gamma, const float* beta,
+                const float* bias /* (N) or NULL */, void* W_scaled, float* colsum, float* bias_folded);
+int grl_ln_stats(grl_ctx* ctx, int dtype, int64_t rows, int64_t F, const void* x, float eps, float* stats);
+int grl_ln_gemm_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                   const void* W_scaled, const float* colsum, const float* bias_folded /* (N) or NULL */, float eps,
+                   float* stats, void* out);
+int grl_ln_glu_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                  const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
+                  const float* bias_gate_folded, const float* bias_up_folded, float eps, float* stats,
+                  void* out, int activation);
+
 /* out = a + b.  Replaces VulkanFNN.residual (shaders/fnn-residual.glsl:25-34).
  * grl_add, grl_gelu, grl_silu and grl_relu may run in place (out == a, out == b, y == x).
  * Every other entry point of this header needs its outputs distinct from its inputs unless its own

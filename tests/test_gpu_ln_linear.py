@@ -1,0 +1,181 @@
+"""GPU parity of Linear(LayerNorm(x)) with the normalisation folded into the GEMM (reference shader
+shaders/fused-layernorm-linear.glsl:67-128: per-row mean / variance, then the product with the normalised row) and of its
+gated form on the pre-norm MLP (gate * act(up) of LN(x), the ModernBERT branch of
+utils/vulkan_sentence_transformer.py:799-970).  Truth: float64 LayerNorm followed by the float64 linear / gated
+linear of the oracle on the same (bf16-rounded, for the bf16 path) x and W.  Shapes select every kernel that carries
+the folded epilogue: the persistent 256x256 and 128x128 tile kernels (staged and direct stores), the register-staged
+kernels (K rows that are not whole 128-byte slabs) and the scalar kernel (rows not 16-byte aligned).
+Tolerances: max|y-ref|/max|ref| <= 1e-4 (fp32), <= 2e-2 (bf16)."""
+import numpy as np
+import pytest
+
+from conftest import TOL_F32, TOL_BF16
+from oracle import oracle_np as O
+from grilly_amd import _lib as L
+
+pytestmark = pytest.mark.gpu
+
+
+def tol(dtype):
+    return TOL_F32 if dtype == "fp32" else TOL_BF16
+
+
+def q(dtype, a):
+    return O.bf16_round(a) if dtype == "bf16" else a
+
+
+def ln_linear(backend, dtype, x, g, bt, W, b, eps):
+    """grl_ln_fold + grl_ln_gemm_nt through the C ABI; returns (y, stats, W_scaled, colsum, bias_folded)"""
+    c = backend.core
+    code = L.GRL_BF16 if dtype == "bf16" else L.GRL_F32
+    es = 2 if dtype == "bf16" else 4
+    M, K = x.shape
+    N = W.shape[0]
+    dx, dw, dg, dbt = c.upload(x, code), c.upload(W, code), c.upload(g), c.upload(bt)
+    db = c.upload(b) if b is not None else None
+    dws, dcs, dbf, dst, dy = c.alloc(N * K * es), c.alloc(N * 4), c.alloc(N * 4), c.alloc(M * 8), c.alloc(M * N * es)
+    try:
+        L.check(c.lib.grl_ln_fold(c.ctx, code, N, K, dw.ptr, dg.ptr, dbt.ptr, db.ptr if db else None, dws.ptr, dcs.ptr, dbf.ptr), "fold")
+        L.check(c.lib.grl_ln_gemm_nt(c.ctx, code, code, M, N, K, dx.ptr, dws.ptr, dcs.ptr, dbf.ptr, float(eps), dst.ptr, dy.ptr), "gemm")
+        return (c.download(dy, (M, N), code), c.download(dst, (M, 2)), c.download(dws, (N, K), code), c.download(dcs, (N,)),
+                c.download(dbf, (N,)))
+    finally:
+        for t in (dx, dw, dg, dbt, db, dws, dcs, dbf, dst, dy):
+            if t is not None:
+                t.free()
+
+
+def ln_glu(backend, dtype, x, g, bt, Wg, Wu, bg, bu, eps, act):
+    c = backend.core
+    code = L.GRL_BF16 if dtype == "bf16" else L.GRL_F32
+    es = 2 if dtype == "bf16" else 4
+    M, K = x.shape
+    N = Wg.shape[0]
+    bufs = [c.upload(x, code), c.upload(Wg, code), c.upload(Wu, code), c.upload(g), c.upload(bt), c.upload(bg), c.upload(bu)]
+    dx, dwg, dwu, dg, dbt, dbg, dbu = bufs
+    outs = [c.alloc(N * K * es), c.alloc(N * K * es), c.alloc(N * 4), c.alloc(N * 4), c.alloc(N * 4), c.alloc(N * 4), c.alloc(M * 8),
+            c.alloc(M * N * es)]
+    wgs, wus, cg, cu, dgf, duf, dst, dy = outs
+    try:
+        L.check(c.lib.grl_ln_fold(c.ctx, code, N, K, dwg.ptr, dg.ptr, dbt.ptr, dbg.ptr, wgs.ptr, cg.ptr, dgf.ptr), "fold gate")
+        L.check(c.lib.grl_ln_fold(c.ctx, code, N, K, dwu.ptr, dg.ptr, dbt.ptr, dbu.ptr, wus.ptr, cu.ptr, duf.ptr), "fold up")
+        L.check(c.lib.grl_ln_glu_nt(c.ctx, code, code, M, N, K, dx.ptr, wgs.ptr, wus.ptr, cg.ptr, cu.ptr, dgf.ptr, duf.ptr, float(eps),
+                                    dst.ptr, dy.ptr, {"silu": L.EPI_SILU, "relu": L.EPI_RELU, "gelu": L.EPI_GELU}[act]), "ln_glu")
+        return c.download(dy, (M, N), code)
+    finally:
+        for t in bufs + outs:
+            t.free()
+
+
+def make(rng, M, K, N, mean=0.0, scale=1.0):
+    x = (rng.standard_normal((M, K)) * scale + mean).astype(np.float32)
+    # rows with their own offset and spread, so that the statistics matter
+    x = x * (0.5 + rng.random((M, 1))).astype(np.float32) + rng.standard_normal((M, 1)).astype(np.float32)
+    W = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    g = (1.0 + 0.3 * rng.standard_normal(K)).astype(np.float32)
+    bt = (0.3 * rng.standard_normal(K)).astype(np.float32)
+    return x, W, b, g, bt
+
+
+# (M, K, N, what it selects)
+SHAPES = [
+    (16384, 768, 768, "256x256 persistent tiles (192 of them), staged stores"),
+    (16384 + 37, 768, 776, "256x256 tiles with a ragged row band and an 8-column edge tile"),
+    (1000, 768, 2304, "128x128 persistent tiles"),
+    (515, 768, 300, "128x128 tiles, rows of 600 / 1200 bytes: direct stores"),
+    (300, 776, 200, "K rows that are not whole 128-byte slabs: register-staged kernel"),
+    (16384, 776, 3072, "register-staged 256x256 kernel"),
+    (70, 13, 9, "rows not 16-byte aligned: scalar kernel"),
+    (5, 64, 1, "single output column"),
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("M,K,N,what", SHAPES)
+def test_ln_linear_parity(backend, dtype, M, K, N, what):
+    rng = np.random.default_rng(M * 7 + K * 3 + N)
+    x, W, b, g, bt = make(rng, M, K, N)
+    x, W = q(dtype, x), q(dtype, W)
+    eps = 1e-5
+    y, stats, Ws, cs, bf = ln_linear(backend, dtype, x, g, bt, W, b, eps)
+    rows = np.unique(np.concatenate([np.arange(0, M, max(1, M // 64)), [M - 1], rng.integers(0, M, 32)]))
+    ref = O.truth_linear(O.truth_layernorm(x[rows], g, bt, eps), W, b)
+    assert O.max_rel(y[rows], ref) < tol(dtype), what
+    assert np.isfinite(y).all()
+    # the pieces: statistics, scaled weight, column sums, folded bias
+    x64 = x.astype(np.float64)
+    mean = x64.mean(1)
+    rstd = 1.0 / np.sqrt(x64.var(1) + eps)
+    np.testing.assert_allclose(stats[:, 0], rstd, rtol=2e-5)
+    np.testing.assert_allclose(stats[:, 1], rstd * mean, rtol=2e-5, atol=1e-5)
+    Ws_ref = q(dtype, (g[None, :] * W).astype(np.float32))
+    np.testing.assert_allclose(Ws, Ws_ref, rtol=1e-6 if dtype == "fp32" else 8e-3, atol=1e-7)
+    np.testing.assert_allclose(cs, Ws.astype(np.float64).sum(1), rtol=1e-4, atol=2e-5)       # of the values as stored
+    np.testing.assert_allclose(bf, b + W.astype(np.float64) @ bt.astype(np.float64), rtol=1e-4, atol=2e-5)
+    # without bias
+    y0 = ln_linear(backend, dtype, x, g, bt, W, None, eps)[0]
+    ref0 = O.truth_linear(O.truth_layernorm(x[rows], g, bt, eps), W, None)
+    assert O.max_rel(y0[rows], ref0) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_ln_linear_rows_far_from_zero(backend, dtype):
+    """Row mean several spreads away from zero: the epilogue subtracts mean * column sum from the raw product, which
+    must not cost the result its accuracy (fp32 accumulation; bf16 inputs already carry the offset's rounding)."""
+    rng = np.random.default_rng(5)
+    M, K, N = 777, 1024, 512
+    x, W, b, g, bt = make(rng, M, K, N, mean=6.0, scale=1.0)
+    x, W = q(dtype, x), q(dtype, W)
+    y = ln_linear(backend, dtype, x, g, bt, W, b, 1e-5)[0]
+    ref = O.truth_linear(O.truth_layernorm(x, g, bt, 1e-5), W, b)
+    assert O.max_rel(y, ref) < (5e-4 if dtype == "fp32" else TOL_BF16)
+
+
+def test_ln_linear_closed_forms(backend):
+    # constant rows: variance 0, normalised row 0 -> out = bias + W.beta whatever gamma is.  The epilogue forms
+    # rstd * (x.Ws - mean * c) with rstd = 1/sqrt(eps) = 316 here, so the fp32 rounding of the two products
+    # (about 2^-23 * |mean| * sum|Ws| = 2e-5) comes back multiplied by 316: the bound below.
+    K, N = 64, 8
+    x = np.full((4, K), 3.25, np.float32)
+    rng = np.random.default_rng(1)
+    W = rng.standard_normal((N, K)).astype(np.float32)
+    g, bt, b = rng.standard_normal(K).astype(np.float32), rng.standard_normal(K).astype(np.float32), rng.standard_normal(N).astype(np.float32)
+    y = ln_linear(backend, "fp32", x, g, bt, W, b, 1e-5)[0]
+    np.testing.assert_allclose(y, np.tile(b + W.astype(np.float64) @ bt, (4, 1)), rtol=1e-4, atol=1e-2)
+    # gamma = 1, beta = 0, W = identity rows: out = the normalised row itself
+    x = rng.standard_normal((6, K)).astype(np.float32)
+    y = ln_linear(backend, "fp32", x, np.ones(K, np.float32), np.zeros(K, np.float32), np.eye(K, dtype=np.float32), None, 1e-5)[0]
+    np.testing.assert_allclose(y, O.truth_layernorm(x, None, None, 1e-5), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(y.mean(1), 0, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("act", ["gelu", "silu", "relu"])
+@pytest.mark.parametrize("M,K,N", [(16384, 768, 1152), (700, 768, 1152), (130, 776, 72), (33, 10, 5)])
+def test_ln_glu_parity(backend, dtype, act, M, K, N):
+    if M == 16384 and act != "gelu":
+        pytest.skip("the large shape runs with the activation the pre-norm encoder uses")
+    rng = np.random.default_rng(M + K + N + len(act))
+    x, Wg, bg, g, bt = make(rng, M, K, N)
+    Wu = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+    bu = rng.standard_normal(N).astype(np.float32)
+    x, Wg, Wu = q(dtype, x), q(dtype, Wg), q(dtype, Wu)
+    y = ln_glu(backend, dtype, x, g, bt, Wg, Wu, bg, bu, 1e-5, act)
+    rows = np.unique(np.concatenate([np.arange(0, M, max(1, M // 48)), [M - 1]]))
+    xn = O.truth_layernorm(x[rows], g, bt, 1e-5)
+    ref = O.truth_fused_glu(xn, Wg, Wu, bg, bu, act)[0]
+    assert O.max_rel(y[rows], ref) < tol(dtype)
+
+
+def test_ln_linear_argument_errors(backend):
+    c = backend.core
+    with pytest.raises(ValueError):
+        L.check(c.lib.grl_ln_gemm_nt(c.ctx, 0, 0, 4, 4, 8, None, None, None, None, 1e-5, None, None))
+    with pytest.raises(ValueError):
+        L.check(c.lib.grl_ln_stats(c.ctx, 7, 4, 8, None, 1e-5, None))
+    with pytest.raises(ValueError):
+        L.check(c.lib.grl_ln_fold(c.ctx, 0, 4, 0, None, None, None, None, None, None, None))
+    # empty problems are no-ops
+    L.check(c.lib.grl_ln_gemm_nt(c.ctx, 0, 0, 0, 4, 8, None, None, None, None, 1e-5, None, None))
+    L.check(c.lib.grl_ln_fold(c.ctx, 0, 0, 8, None, None, None, None, None, None, None))
