@@ -33,6 +33,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16 = 2.5e15      # MI355X dense bf16 MFMA, FLOP/s
 PEAK_FP32 = 157.3e12
 PEAK_HBM = 8.0e12       # B/s
+NOMINAL_GHZ = 2.4        # engine clock the MFMA peaks are quoted at (256 CUs x 4 SIMDs x 1024 bf16 FLOP/cycle x 2.4 GHz = 2.5 PFLOP/s)
 TOL = {"bf16": 2e-2, "fp32": 1e-4}
 
 WARM = 5
@@ -136,6 +137,14 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
             continue
         ms = time_launches(c, fn, reps)
         rec = {"ms": round(ms, 4), "group": group, "flops": flops, "bytes": nbytes}
+        # the shader clock these launches run at: a one-wave probe on a second stream lives for 70 % of a repeat of the
+        # same launch sequence (the clock is one domain for the whole GPU)
+        c.sync()
+        c.clock_probe_begin(max(0.7 * ms * reps, 0.05))
+        for _ in range(reps):
+            fn()
+        rec["shader_clock_ghz"] = round(c.clock_probe_end(), 3)
+        c.sync()
         if flops:
             rec["tflops"] = round(flops / ms / 1e9, 1)
             rec["frac_mfma"] = round(flops / (ms * 1e-3) / peak, 4)
@@ -401,6 +410,12 @@ def main():
 
     wall, ev_ms = timed_forward(backend, enc, a.steps, a.warmup)
     ms_per_step = wall * 1e3 / a.steps
+    # shader clock during the forward: probe beside three more (untimed) steps
+    backend.core.clock_probe_begin(max(2.0 * ms_per_step, 0.05))
+    for _ in range(3):
+        enc.launch(pool=True)
+    fwd_clock = backend.core.clock_probe_end()
+    backend.core.sync()
     tokens_per_s = B * S * a.steps / wall
     flops = enc.flops_per_forward(B, S)
     peak = PEAK_BF16 if a.dtype == "bf16" else PEAK_FP32
@@ -415,6 +430,7 @@ def main():
         "event_ms_per_step": round(ev_ms / a.steps, 3),
         "model_tflops": round(flops / (ms_per_step * 1e-3) / 1e12, 1),
         "model_frac_mfma": round(flops / (ms_per_step * 1e-3) / peak, 4),
+        "shader_clock_ghz_during_forward": round(fwd_clock, 3),
         "device": info,
     }
     nseq = min(a.cpu_sequences, B)
@@ -436,7 +452,12 @@ def main():
                            "traffic": traffic, "traffic_measured_at_commit": at_commit,
                            "algorithmic_bytes": sum(r["bytes"] for r in g) / 3,
                            "avg_launch_ms": round(avg_ms, 4), "flops_per_launch": avg_flops,
+                           "shader_clock_ghz": round(sum(r["shader_clock_ghz"] for r in g) / 3, 3), "nominal_clock_ghz": NOMINAL_GHZ,
+                           "frac_at_measured_clock": round(ach * 1e12 / (peak * (sum(r["shader_clock_ghz"] for r in g) / 3) / NOMINAL_GHZ), 4),
                            "launches_per_step": 3 * cfg.layers,
+                           "clock_note": "peak = 256 CUs x 4 SIMDs x 1024 bf16 FLOP per cycle (fp32: 64) x the nominal 2.4 GHz; under the board's "
+                                         "power limit the timed launches run at shader_clock_ghz (probe kernel beside them), and "
+                                         "frac_at_measured_clock is the same achieved rate against the peak at that clock",
                            "note": "launches timed back to back on the layer's real operands; inside the forward the same launches "
                                    "run about 10 % longer (operands come from HBM): see profiles/encoder_forward_bert_base_bf16_kernel_stats.md"}
     extra = {}

@@ -54,6 +54,8 @@ SIGNATURES = {
     "grl_sync": (c_int, [c_void_p]),
     "grl_timer_start": (c_int, [c_void_p]),
     "grl_timer_stop": (c_int, [c_void_p, ctypes.POINTER(c_float)]),
+    "grl_clock_probe_begin": (c_int, [c_void_p, c_float]),
+    "grl_clock_probe_end": (c_int, [c_void_p, ctypes.POINTER(c_float)]),
     "grl_cast": (c_int, [c_void_p, c_int, c_int, c_i64, c_void_p, c_void_p]),
     "grl_gemm_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
     "grl_gemm_nn": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p]),

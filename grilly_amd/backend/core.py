@@ -137,3 +137,13 @@ class HipCore:
         ms = ctypes.c_float()
         L.check(self.lib.grl_timer_stop(self.ctx, ctypes.byref(ms)), "timer_stop")
         return float(ms.value)
+
+    def clock_probe_begin(self, millis):
+        """start the shader-clock probe: it runs for `millis` beside whatever is enqueued next"""
+        L.check(self.lib.grl_clock_probe_begin(self.ctx, float(millis)), "clock_probe_begin")
+
+    def clock_probe_end(self):
+        """wait for the probe; average shader clock in GHz while it ran"""
+        ghz = ctypes.c_float()
+        L.check(self.lib.grl_clock_probe_end(self.ctx, ctypes.byref(ghz)), "clock_probe_end")
+        return float(ghz.value)

@@ -27,6 +27,9 @@ struct grl_ctx {
     struct rope_table { int S, D, style; float base, scaling; void* dev; };
     std::mutex tab_mu;
     std::vector<rope_table> rope_tables;
+    // shader-clock probe (grl_clock_probe_begin / _end): its own stream, so that it runs beside the work it observes
+    hipStream_t probe_stream = nullptr;
+    uint64_t* probe_out = nullptr;      // device: {shader cycles, 100 MHz ticks}
 };
 
 // device pointer to a (>= S, D/2) table of {cos, sin}; builds it on first use (on the context stream)

@@ -60,6 +60,8 @@ extern "C" void grl_destroy(grl_ctx* c) {
     for (auto& kv : c->live) hipFree(kv.first);
     hipEventDestroy(c->ev0);
     hipEventDestroy(c->ev1);
+    if (c->probe_stream) { hipStreamSynchronize(c->probe_stream); hipStreamDestroy(c->probe_stream); }
+    if (c->probe_out) hipFree(c->probe_out);
     hipStreamDestroy(c->stream);
     delete c;
 }
@@ -214,5 +216,45 @@ extern "C" int grl_timer_stop(grl_ctx* c, float* ms) {
     GRL_CHECK_HIP(hipEventRecord(c->ev1, c->stream));
     GRL_CHECK_HIP(hipEventSynchronize(c->ev1));
     GRL_CHECK_HIP(hipEventElapsedTime(ms, c->ev0, c->ev1));
+    return GRL_OK;
+}
+
+// ---- shader-clock probe ---------------------------------------------------------------------------------------
+// One wave that sleeps in short naps until `ticks` of the 100 MHz reference counter have passed and reports how many
+// shader-clock cycles went by meanwhile.  The shader clock is one domain for the whole GPU, so a probe that runs
+// beside a kernel (on its own stream) reads the clock that kernel runs at: under a power limit that is well below
+// the nominal frequency the peak figures are quoted for.
+__global__ __launch_bounds__(64) void clock_probe_kernel(uint64_t* out, uint64_t ticks) {
+    const uint64_t r0 = __builtin_amdgcn_s_memrealtime();
+    const uint64_t c0 = __builtin_amdgcn_s_memtime();
+    uint64_t r;
+    do {
+        __builtin_amdgcn_s_sleep(32);
+        r = __builtin_amdgcn_s_memrealtime();
+    } while (r - r0 < ticks);             // the reference counter only moves forward: the loop ends
+    const uint64_t c1 = __builtin_amdgcn_s_memtime();
+    if (threadIdx.x == 0) { out[0] = c1 - c0; out[1] = r - r0; }
+}
+
+extern "C" int grl_clock_probe_begin(grl_ctx* c, float millis) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_clock_probe_begin: null context");
+    GRL_REQUIRE(millis > 0.f && millis <= 500.f, GRL_ERR_ARG, "grl_clock_probe_begin: duration must be in (0, 500] ms");
+    std::lock_guard<std::mutex> lk(c->timer_mu);
+    GRL_CHECK_HIP(hipSetDevice(c->device));
+    if (!c->probe_stream) GRL_CHECK_HIP(hipStreamCreateWithFlags(&c->probe_stream, hipStreamNonBlocking));
+    if (!c->probe_out) GRL_CHECK_HIP(hipMalloc((void**)&c->probe_out, 2 * sizeof(uint64_t)));
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, c->probe_stream, c->probe_out, (uint64_t)((double)millis * 1e5));
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
+extern "C" int grl_clock_probe_end(grl_ctx* c, float* ghz) {
+    GRL_REQUIRE(c && ghz, GRL_ERR_ARG, "grl_clock_probe_end: null argument");
+    std::lock_guard<std::mutex> lk(c->timer_mu);
+    GRL_REQUIRE(c->probe_stream && c->probe_out, GRL_ERR_ARG, "grl_clock_probe_end: no probe was started");
+    GRL_CHECK_HIP(hipStreamSynchronize(c->probe_stream));
+    uint64_t h[2] = {0, 0};
+    GRL_CHECK_HIP(hipMemcpy(h, c->probe_out, sizeof(h), hipMemcpyDeviceToHost));
+    *ghz = h[1] ? (float)((double)h[0] / (double)h[1] * 0.1) : 0.f;
     return GRL_OK;
 }

@@ -104,6 +104,13 @@ int grl_sync(grl_ctx* ctx);
  * each other's start. */
 int grl_timer_start(grl_ctx* ctx);
 int grl_timer_stop(grl_ctx* ctx, float* elapsed_ms);   /* synchronises */
+/* Shader-clock probe, a measurement aid with no counterpart in the reference: _begin starts a one-wave kernel on a
+ * second stream of the context that runs for `millis` of wall time beside whatever the caller enqueues next; _end
+ * waits for it and returns the average shader clock in GHz over that time (shader cycles over 100 MHz reference
+ * ticks).  Peak MFMA rates are quoted at the nominal clock; under a power limit the GPU runs a loaded kernel below
+ * it, and this is how the benchmark reads the clock its timed launches really ran at. */
+int grl_clock_probe_begin(grl_ctx* ctx, float millis);
+int grl_clock_probe_end(grl_ctx* ctx, float* ghz);
 
 /* fp32 <-> bf16 conversion on the device (RNE).  No reference counterpart: the
  * reference is fp32 only. */

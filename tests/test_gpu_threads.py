@@ -49,3 +49,40 @@ def test_concurrent_calls_share_one_context(backend):
     before = backend.core.pool_stats()["bytes_in_use"]
     backend.fnn.linear(np.ones((4, 8), np.float32), np.ones((3, 8), np.float32))
     assert backend.core.pool_stats()["bytes_in_use"] == before
+
+
+def test_shader_clock_probe(backend):
+    """The probe kernel runs on its own stream beside the context's work and reports shader cycles over 100 MHz reference
+    ticks: a plausible clock for this GPU, idle and beside a GEMM; bad durations are refused."""
+    from grilly_amd import _lib as L
+    c = backend.core
+    c.sync()
+    c.clock_probe_begin(2.0)
+    idle = c.clock_probe_end()
+    assert 0.05 < idle < 3.5, idle
+    rng = np.random.default_rng(0)
+    x = O.bf16_round(rng.standard_normal((8192, 1024)).astype(np.float32))
+    w = O.bf16_round((rng.standard_normal((4096, 1024)) * 0.03).astype(np.float32))
+    dx, dw = c.upload(x, L.GRL_BF16), c.upload(w, L.GRL_BF16)
+    dy = c.alloc(8192 * 4096 * 2)
+    try:
+        run = lambda: L.check(c.lib.grl_gemm_nt(c.ctx, L.GRL_BF16, L.GRL_BF16, 8192, 4096, 1024, dx.ptr, dw.ptr, None, dy.ptr, L.EPI_NONE))
+        run()
+        c.sync()
+        c.clock_probe_begin(3.0)
+        for _ in range(60):
+            run()
+        busy = c.clock_probe_end()
+        c.sync()
+        assert 0.3 < busy < 3.5, busy
+        # the GEMM beside the probe still computes what it should
+        y = c.download(dy, (8192, 4096), L.GRL_BF16)
+        rows = [0, 4097, 8191]
+        assert O.max_rel(y[rows], O.truth_linear(x[rows], w, None)) < 2e-2
+    finally:
+        for t in (dx, dw, dy):
+            t.free()
+    with pytest.raises(ValueError):
+        c.clock_probe_begin(0.0)
+    with pytest.raises(ValueError):
+        c.clock_probe_begin(1e6)
