@@ -252,9 +252,10 @@ extern "C" int grl_clock_probe_end(grl_ctx* c, float* ghz) {
     GRL_REQUIRE(c && ghz, GRL_ERR_ARG, "grl_clock_probe_end: null argument");
     std::lock_guard<std::mutex> lk(c->timer_mu);
     GRL_REQUIRE(c->probe_stream && c->probe_out, GRL_ERR_ARG, "grl_clock_probe_end: no probe was started");
-    GRL_CHECK_HIP(hipStreamSynchronize(c->probe_stream));
     uint64_t h[2] = {0, 0};
-    GRL_CHECK_HIP(hipMemcpy(h, c->probe_out, sizeof(h), hipMemcpyDeviceToHost));
+    // copied on the probe's own stream: a copy on the null stream would serialise with the work being observed
+    GRL_CHECK_HIP(hipMemcpyAsync(h, c->probe_out, sizeof(h), hipMemcpyDeviceToHost, c->probe_stream));
+    GRL_CHECK_HIP(hipStreamSynchronize(c->probe_stream));
     *ghz = h[1] ? (float)((double)h[0] / (double)h[1] * 0.1) : 0.f;
     return GRL_OK;
 }
