@@ -445,15 +445,16 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     // every wave requests its own share (and a mask row, so that all waves count the same number of
     // transfers per tile)
     auto issue = [&](int kt) { issue_share(kt, wave); issue_mask(kt); };
-    // lacc: row sums of P, accumulated by the matrix core against an all-ones operand (every
-    // register of a lane then holds the full sum for that lane's query); only register 0 is kept exact
-    f32x16 oacc[QT][DT], lacc[QT];
+    // lsum: this lane's share of the row sum of P (its 8 of the 16 keys of every slab; the other half sits in lane ^ 32),
+    // summed from the bf16-rounded values that also enter the PV product, two per v_dot2c_f32_bf16.  (Row sums by one more
+    // MFMA against an all-ones operand cost a fifth of the PV matrix work for head dim 64 and were 6-8 % slower.)
+    f32x16 oacc[QT][DT];
+    float lsum[QT];
     float m_run[QT];
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
         m_run[t] = -1.4426950408889634e10f;      // -1e10 in the base-2 domain
-#pragma unroll
-        for (int r = 0; r < 16; ++r) lacc[t][r] = 0.f;
+        lsum[t] = 0.f;
 #pragma unroll
         for (int d = 0; d < DT; ++d)
 #pragma unroll
@@ -611,7 +612,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
                 // rescale the running output and sum only when some row of the wave raised its maximum
                 // (never for the first tile: there is nothing accumulated yet)
                 if (kt > 0 && __builtin_amdgcn_ballot_w64(mx != m_run[u]) != 0) {
-                    lacc[u][0] *= alpha;
+                    lsum[u] *= alpha;
                     sfor<DT>([&](auto idt) {
                         constexpr int dt = decltype(idt)::value;
 #pragma unroll
@@ -625,7 +626,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
                 pneg[u] = -delta;
                 if (__builtin_amdgcn_ballot_w64(delta != 0.f) != 0) {
                     const float alpha = __builtin_amdgcn_exp2f(-delta);
-                    lacc[u][0] *= alpha;
+                    lsum[u] *= alpha;
                     sfor<DT>([&](auto idt) {
                         constexpr int dt = decltype(idt)::value;
 #pragma unroll
@@ -657,9 +658,18 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
                         const float p1 = __builtin_amdgcn_exp2f(FAST ? sacc[u][t][8 * hh + 2 * e + 1] : sacc[u][t][8 * hh + 2 * e + 1] + pneg[u]);
                         pf[u][e] = pack_bf16x2(p0, p1);
                     }
-                // row sums: P^T against an all-ones (bf16 1.0) operand
-                const u32x4 ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
-                sfor<QT>([&](auto iu) { Slab<uint16_t>::run(ones, pf[decltype(iu)::value], lacc[decltype(iu)::value]); });
+                // row sums of the rounded values
+                {
+                    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2v;
+                    const bf16x2v one2 = __builtin_bit_cast(bf16x2v, 0x3f803f80u);
+#pragma unroll
+                    for (int u = 0; u < QT; ++u)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t w = pf[u][e];
+                            lsum[u] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2v, w), one2, lsum[u], false);
+                        }
+                }
                 // keys of MFMA k-index (g, e): 32t + 16hh + 8*(e/4) + 4g + e%4, g = lane/32
                 const int kA = 32 * t + 16 * hh + 4 * (grp >> 1) + (j16 >> 2);
                 sfor<DT>([&](auto idt) {
@@ -705,7 +715,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
 #pragma unroll
     for (int u = 0; u < QT; ++u) {
         const int qi = qw0 + 32 * u + li;
-        const float inv = 1.0f / fmaxf(lacc[u][0], 1e-10f);
+        const float inv = 1.0f / fmaxf(halves_sum(lsum[u]), 1e-10f);
         if (qi < S) {
             uint16_t* Og = p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
 #pragma unroll
