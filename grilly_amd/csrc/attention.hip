@@ -351,47 +351,68 @@ template <int IPT, int MAXT> __device__ __forceinline__ void wait_tiles_outstand
     }
 }
 
+template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
+    __builtin_amdgcn_s_waitcnt(15 | (3 << 14) | (7 << 4) | ((N & 15) << 8));
+}
+// a wave-uniform value, said so to the compiler (it then lives in a scalar register and branches on it are scalar)
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// The PV accumulates of one 16-key slab as in-place instructions the register allocator cannot untie (with the builtin
+// it moves the 32-register accumulator to another place and back around every tile).  The compiler does not know that
+// these are matrix instructions and adds no hazard wait states for them:
+//   * the s_nop in front keeps two wait states between whatever VALU instruction last wrote an operand register (the
+//     accumulators' zero fill, which the compiler sinks to their first use; a conversion; a register move or reload the
+//     compiler puts in front of the statement) and the MFMA that reads it;
+//   * mfma_drain() before any VALU / memory instruction reads or writes the accumulators.
+template <int DT> __device__ __forceinline__ void mfma_inplace(const u32x4 (&a)[DT], const u32x4& b, f32x16 (&acc)[DT]) {
+    static_assert(DT == 1 || DT == 2 || DT == 4, "head dims 32, 64, 128");
+    if constexpr (DT == 1)
+        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[0]) : "v"(a[0]), "v"(b));
+    else if constexpr (DT == 2)
+        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %2, %4, %0\n\tv_mfma_f32_32x32x16_bf16 %1, %3, %4, %1"
+                     : "+v"(acc[0]), "+v"(acc[1]) : "v"(a[0]), "v"(a[1]), "v"(b));
+    else
+        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %4, %8, %0\n\tv_mfma_f32_32x32x16_bf16 %1, %5, %8, %1\n\t"
+                     "v_mfma_f32_32x32x16_bf16 %2, %6, %8, %2\n\tv_mfma_f32_32x32x16_bf16 %3, %7, %8, %3"
+                     : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]) : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b));
+}
+__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory"); }
+
 // ROPE_Q: rotation applied to the query rows as they are loaded: 0 none, 1 interleaved pairs (2p, 2p+1), 2 the
 // (d, d+D/2) pairing (both halves of a pair sit in chunks this lane loads itself)
+// QT = 32-query MFMA tiles per wave, NW waves per workgroup, NSTG-deep ring of KT-key (64 or 128) K/V tiles in LDS
+// (NSTG-1 tiles in flight), OCC workgroups per CU the registers are budgeted for.
 template <int D, int ROPE_Q, int QT, int NW, int NSTG, bool HAS_MASK, int KT, int OCC = (NW == 4 ? 2 : 1)>
 __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
-    // QT = 32-query MFMA tiles per wave (every K / V fragment read from LDS feeds QT MFMAs),
-    // NW waves per workgroup, NSTG-deep ring of 64-key K/V tiles in LDS (NSTG-1 tiles in flight).
     constexpr int RB = D * 2, NCH = RB / 16, NS = D / 16;
-    constexpr int NKB = KT / 32, DT = D / 32;     // KT keys per tile (64 or 128)
+    constexpr int NKB = KT / 32, DT = D / 32;
     constexpr int TILE = KT * RB;
     constexpr int NT = NW * 64;
-    constexpr int TPO = TILE / 1024;              // 1 KiB transfers per tile and operand
-    constexpr int IPT = 2 * TPO / NW + (HAS_MASK ? 1 : 0);   // transfers per wave per tile (K, V, mask)
-    constexpr int RPI = 1024 / RB;                // tile rows per transfer
-    constexpr int QW = 32 * QT, QB = NW * QW;     // queries per wave / per workgroup
+    constexpr int TPO = TILE / 1024;
+    constexpr int IPT = 2 * TPO / NW + (HAS_MASK ? 1 : 0);
+    constexpr int RPI = 1024 / RB;
+    constexpr int QW = 32 * QT, QB = NW * QW;
     static_assert((2 * TPO) % NW == 0 && 2 * TPO >= NW, "transfers must divide over the waves");
     static_assert(NSTG >= 2 && IPT * (NSTG - 1) < 64, "ring of at least two stages; vmcnt is a 6-bit counter");
-    // ONE LDS array with manual offsets: with several __shared__ objects the compiler tracks the
-    // LDS-DMA transfers per object and puts a full vmcnt(0) in front of every LDS read of a ring
-    // that has a transfer in flight, which would serialise the prefetch.
     constexpr int OFF_V = NSTG * TILE, OFF_M = 2 * NSTG * TILE;
-    __shared__ __attribute__((aligned(1024))) char lds[2 * NSTG * TILE + NSTG * 1024];
+    __shared__ __attribute__((aligned(1024))) char lds[2 * NSTG * TILE + (HAS_MASK ? NSTG * 1024 : 0)];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Everything that steers control flow or addresses a transfer is wave-uniform and is told so to the compiler
+    // (readfirstlane): the loop then branches on scalar conditions and keeps its counters in scalar registers.
+    const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6);
     const int li = lane & 31, lg = lane >> 5;
-    // 1-D grid; p.order picks the workgroup -> (batch*head, query block) map: bit 0 renumbers the ids per XCD,
-    // bit 1 puts the heaviest query blocks of all heads first (causal), else heads are walked one by one
-    // (causal: each head's heavy blocks first) so that neighbours share that head's K/V in L2.
     const int S = p.S;
     const int nqb = (S + QB - 1) / QB, nbh = p.B * p.H;
-    // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2: `lin` renumbers them so
-    // that every XCD walks one contiguous run, and workgroups that run side by side on an XCD are
-    // neighbours in `lin`.
     const int nwg = (int)gridDim.x, per = nwg >> 3, rem = nwg & 7, xcd = (int)blockIdx.x & 7, loc = (int)blockIdx.x >> 3;
     const int lin = (p.order & 1) ? xcd * per + (xcd < rem ? xcd : rem) + loc : (int)blockIdx.x;
     int qb, bh;
-    if (p.order & 2) { qb = nqb - 1 - lin / nbh; bh = lin % nbh; }            // heaviest query blocks of all heads first
-    else if (p.causal) { bh = lin / nqb; qb = nqb - 1 - lin % nqb; }          // head by head, heavy blocks first
-    else { qb = lin % nqb; bh = lin / nqb; }                                  // head by head
-    const int b = bh / p.H, h = bh % p.H;
+    if (p.order & 2) { qb = nqb - 1 - lin / nbh; bh = lin % nbh; }
+    else if (p.causal) { bh = lin / nqb; qb = nqb - 1 - lin % nqb; }
+    else { qb = lin % nqb; bh = lin / nqb; }
+    qb = uni(qb); bh = uni(bh);
+    const int b = uni(bh / p.H), h = uni(bh % p.H);
     const int q0 = qb * QB;
-    const int qw0 = q0 + wave * QW;               // first query of this wave
+    const int qw0 = q0 + wave * QW;
     const uint16_t* Qg = p.Q + (int64_t)b * S * p.q_stride + h * D;
 
     int nkt = (S + KT - 1) / KT;
@@ -399,61 +420,52 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
         int last = (q0 + QB - 1 < S - 1 ? q0 + QB - 1 : S - 1) / KT + 1;
         nkt = nkt < last ? nkt : last;
     }
+    nkt = uni(nkt);
 
-    // buffer resources cover this (batch, head)'s rows 0..S-1; rows >= S are out of range
-    auto make_rsrc = [&](const uint16_t* base, int64_t stride) {
+    auto make_rsrc = [&](const uint16_t* base, int64_t stride) __attribute__((always_inline)) {
         int64_t bytes = (int64_t)(S - 1) * stride * 2 + RB;
         uint32_t nrec = bytes > 0xffffffffLL ? 0xffffffffu : (uint32_t)bytes;
         return make_rsrc_words(base + (int64_t)b * S * stride + h * D, nrec);
     };
-    const rsrc_words rsK = make_rsrc(p.K, p.k_stride);
-    const rsrc_words rsV = make_rsrc(p.V, p.v_stride);
-    const rsrc_words rsM = make_rsrc_words(p.mask ? (const void*)(p.mask + (int64_t)b * S) : (const void*)p.Q, HAS_MASK ? (uint32_t)S * 4u : 0u);
-    const int kstride_b = (int)p.k_stride * 2, vstride_b = (int)p.v_stride * 2;
-    // lane -> (row, slot) inside one 1 KiB transfer; the slot holds chunk slot ^ swizzle(row)
-    const int t_row = lane / NCH, t_slot = lane % NCH;
-
-    // Transfer addresses: the per-lane part (row inside the transfer x row stride + swizzled chunk) does not
-    // change from tile to tile and has KVAR variants for K (the swizzle looks at row bits the transfer index
-    // supplies) and one for V; the tile and transfer index are wave-uniform and travel in the scalar offset.
+    // A wave's share of a tile's transfers is all K or all V (K transfers first, then V): which one is a
+    // wave-uniform choice made once, so the loop issues its transfers without a branch.
     constexpr int TPW = 2 * TPO / NW;
     constexpr int KVAR = NCH >= 16 ? 4 : (NCH == 8 ? 2 : 1);
+    static_assert(TPO % TPW == 0, "a wave's share does not straddle K and V");
     static_assert(TPW % KVAR == 0 && TPO % KVAR == 0 && (RPI * KVAR) % 16 == 0, "swizzle period must divide the transfer split");
-    int voffK[KVAR];
+    const bool isv = wave * TPW >= TPO;
+    const rsrc_words rsT = isv ? make_rsrc(p.V, p.v_stride) : make_rsrc(p.K, p.k_stride);
+    const rsrc_words rsM = make_rsrc_words(p.mask ? (const void*)(p.mask + (int64_t)b * S) : (const void*)p.Q, HAS_MASK ? (uint32_t)S * 4u : 0u);
+    const int stride_b = uni((int)(isv ? p.v_stride : p.k_stride) * 2);
+    const int inst0 = wave * TPW - (isv ? TPO : 0);
+    const int t_row = lane / NCH, t_slot = lane % NCH;
+    // per-lane part of a transfer address: row inside the transfer x row stride + swizzled chunk (K: KVAR variants,
+    // the swizzle looks at row bits the transfer index supplies; V: one)
+    int voffT[KVAR];
 #pragma unroll
-    for (int i = 0; i < KVAR; ++i) voffK[i] = t_row * kstride_b + ((t_slot ^ lds_swz<NCH>(i * RPI + t_row)) << 4);
-    const int voffV = t_row * vstride_b + ((t_slot ^ lds_swz_v<NCH>(t_row)) << 4);
-    // wave v's share of the K / V transfers of tile kt (v is wave-uniform)
-    auto issue_share = [&](int kt, int v) {
-        const int st = kt % NSTG, k0 = kt * KT;
-        const bool isv = v * TPW >= TPO;                             // K transfers first, then V: a share is all K or all V
-        static_assert(TPO % TPW == 0, "a wave's share does not straddle K and V");
-        const int inst0 = v * TPW - (isv ? TPO : 0);
+    for (int i = 0; i < KVAR; ++i)
+        voffT[i] = t_row * stride_b + ((t_slot ^ (isv ? lds_swz_v<NCH>(t_row) : lds_swz<NCH>(i * RPI + t_row))) << 4);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+    const uint32_t lds_t = lds0 + (isv ? OFF_V : 0) + inst0 * 1024;
+    const int soff_w = inst0 * RPI * stride_b, soff_step = RPI * stride_b, soff_tile = KT * stride_b;
+    auto issue = [&](int kt, int ST) __attribute__((always_inline)) {
+        const int so = kt * soff_tile + soff_w;
 #pragma unroll
-        for (int j = 0; j < TPW; ++j) {
-            const int inst = inst0 + j;
-            const int rowg = k0 + inst * RPI;
-            if (isv) dma16s(rsV, lds + OFF_V + st * TILE + inst * 1024, voffV, rowg * vstride_b);
-            else dma16s(rsK, lds + st * TILE + inst * 1024, voffK[j % KVAR], rowg * kstride_b);
-        }
+        for (int j = 0; j < TPW; ++j)
+            asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         ::"s"(lds_t + ST * TILE + j * 1024), "v"(voffT[j % KVAR]), "s"(rsT), "s"(so + j * soff_step) : "memory");
+        if constexpr (HAS_MASK)
+            asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         ::"s"(lds0 + OFF_M + ST * 1024), "v"(lane * 16), "s"(rsM), "s"(kt * KT * 4) : "memory");
     };
-    // raw mask values of the tile's keys (the transfer unit is 1 KiB per wave, lanes past the tile read
-    // further mask entries or out of range, which nobody uses)
-    auto issue_mask = [&](int kt) {
-        if (HAS_MASK) dma16(rsM, lds + OFF_M + (kt % NSTG) * 1024, (kt * KT + lane * 4) * 4);
-    };
-    // every wave requests its own share (and a mask row, so that all waves count the same number of
-    // transfers per tile)
-    auto issue = [&](int kt) { issue_share(kt, wave); issue_mask(kt); };
-    // lsum: this lane's share of the row sum of P (its 8 of the 16 keys of every slab; the other half sits in lane ^ 32),
-    // summed from the bf16-rounded values that also enter the PV product, two per v_dot2c_f32_bf16.  (Row sums by one more
-    // MFMA against an all-ones operand cost a fifth of the PV matrix work for head dim 64 and were 6-8 % slower.)
+    // the stage a runtime tile index lives in (prologue only; the loop knows its stage at compile time)
+    auto issue_rt = [&](int kt) __attribute__((always_inline)) { issue(kt, kt % NSTG); };
+
     f32x16 oacc[QT][DT];
-    float lsum[QT];
-    float m_run[QT];
+    float lsum[QT], m_run[QT];
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
-        m_run[t] = -1.4426950408889634e10f;      // -1e10 in the base-2 domain
+        m_run[t] = -1.4426950408889634e10f;
         lsum[t] = 0.f;
 #pragma unroll
         for (int d = 0; d < DT; ++d)
@@ -462,12 +474,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     }
     const float c2 = p.scale * 1.4426950408889634f;
 
-    issue(0);
+    issue(0, 0);
 
-    // this wave's queries as MFMA "B" operand: slab s holds dims (2s+lg)*8 .. +7 of query li.
-    // Loaded right after the first tile was requested and before the rest of the ring, so the
-    // counted wait below (transfers return in order) retires tile 0 and these loads together while
-    // the later tiles are still in flight; inside the loop only tile transfers remain to be counted.
     u32x4 qf[QT][NS];
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
@@ -510,223 +518,380 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
         }
     }
 
+
     f32x16 sacc[QT][NKB];
-    // a wave whose queries all precede tile kt has nothing to add (causal): it only keeps the barriers
-    auto skip_tile = [&](int kt) { return p.causal && kt * KT > qw0 + QW - 1; };
-    // last, partial tile: rows >= S hold whatever the out-of-range transfer left; clear them (all threads)
-    auto zero_tail = [&](int kt) {
-        const int k0 = kt * KT;
-        if (k0 + KT > S) {
-            const int st = kt % NSTG, first = S - k0;
-            for (int i = tid; i < (KT - first) * NCH; i += NT) {
-                const u32x4 zero = {0u, 0u, 0u, 0u};
-                *(u32x4*)(lds + st * TILE + first * RB + i * 16) = zero;
-                *(u32x4*)(lds + OFF_V + st * TILE + first * RB + i * 16) = zero;
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        }
-    };
-
-    // A tile without mask, diagonal or ragged end, other than the first one, is a "lazy" tile: its score
-    // accumulators start at -m_run, so the matrix core hands back s - m_run and the exponentials need no
-    // further arithmetic; m_run is raised (with the usual rescale) only when a score exceeds it by more
-    // than 2^LAZY.  m_run is then a reference point at most LAZY below the true running maximum, which
-    // the softmax quotient does not depend on.
     constexpr float LAZY = 6.0f;
-    auto is_lazy = [&](int kt) {
-        const int k0 = kt * KT;
-        return kt > 0 && !HAS_MASK && !(k0 + KT > S) && !(p.causal && (k0 + KT - 1 > qw0));
-    };
+    const u32x4 kone = {lg == 0 ? 0x3f803f80u : 0u, lg == 0 ? 0x3f80u : 0u, 0u, 0u};   // key side of the reference slab: 1 at k-indices 0, 1, 2
+    u32x4 mq[QT];                                                 // query side: -m_run in three parts there
+#pragma unroll
+    for (int u = 0; u < QT; ++u) mq[u] = u32x4{0u, 0u, 0u, 0u};
 
-    // ---- score phase: S^T = K . Q'^T for tile kt into sacc (Q' = Q * scale * log2 e)
-    auto phase_S = [&](int kt) {
-        const char* Kb = lds + (kt % NSTG) * TILE;
-        const bool lazy = is_lazy(kt);
-        sfor<NKB>([&](auto it) {
-            constexpr int t = decltype(it)::value;
+    // ---- fragment addresses.  K: row li of a 32-key block, chunk 2s+lg, swizzled by the row (the swizzle has period 16,
+    // so block and stage offsets are immediates).  V (transposing read): see phase_PV.
+    typedef __attribute__((address_space(3))) char lds_char;
+    const lds_char* const ldsp = (const lds_char*)lds;
+    const lds_char* kbase[NS];
 #pragma unroll
-            for (int u = 0; u < QT; ++u) {
-                const float init = lazy ? -m_run[u] : 0.f;
+    for (int s = 0; s < NS; ++s) kbase[s] = ldsp + li * RB + (((2 * s + lg) ^ lds_swz<NCH>(li)) << 4);
+    const int j16 = lane & 15, grp = lane >> 4;
+    const lds_char* vbase[DT];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[u][t][r] = init;
-            }
-            const int key = 32 * t + li;
+    for (int dt = 0; dt < DT; ++dt) {
+        const int key = 4 * (grp >> 1) + (j16 >> 2);                    // + 32t + 16hh (+ 8): multiples of 8 leave the swizzle alone
+        const int dcol = 32 * dt + 16 * (grp & 1) + 4 * (j16 & 3);
+        const int ch = dcol >> 3, sub = (dcol & 7) * 2;
+        vbase[dt] = ldsp + OFF_V + key * RB + ((ch ^ lds_swz_v<NCH>(key)) << 4) + sub;
+    }
+
+    // ---- score phase: S^T = K . Q'^T for the tile in stage ST; accumulators start from C0 (zero, or -m_run for a lazy tile)
+    constexpr int KB = 1;                                    // fragment buffers (2 = next group's reads in flight during a group's MFMAs: measured, no gain)
+    constexpr int KG = NS < 4 ? NS : 4;                      // fragments per read group
+    constexpr int NFR = NKB * NS, NG = NFR / KG;
+    static_assert(NFR % KG == 0 && NS % KG == 0, "read groups stay inside a key block");
+    auto phase_S = [&](int ST, auto ilazy) __attribute__((always_inline)) {
+        constexpr bool LZ = decltype(ilazy)::value;
+        const lds_char* kb[NS];
 #pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                const int c = 2 * s + lg;
-                const int slot = c ^ lds_swz<NCH>(key);
-                u32x4 kf = *(const u32x4*)(Kb + key * RB + slot * 16);
-                sfor<QT>([&](auto iu) { Slab<uint16_t>::run(kf, qf[decltype(iu)::value][s], sacc[decltype(iu)::value][t]); });
-            }
+        for (int s = 0; s < NS; ++s) kb[s] = kbase[s] + ST * TILE;
+        u32x4 kf[KB][KG];
+        auto kread = [&](auto ig) __attribute__((always_inline)) {
+            constexpr int G = decltype(ig)::value;
+            sfor<KG>([&](auto ii) __attribute__((always_inline)) {
+                constexpr int i = decltype(ii)::value, f = G * KG + i, t = f / NS, s = f % NS;
+                kf[G % KB][i] = *(const __attribute__((address_space(3))) u32x4*)(kb[s] + t * 32 * RB);
+            });
+        };
+        if constexpr (KB == 2) kread(std::integral_constant<int, 0>{});
+        if constexpr (LZ) {
+            // scores relative to m_run: one more k-slab whose key side is 1 and whose query side is -m_run puts -m_run
+            // into every accumulator while the first fragments are on their way
+            sfor<NKB>([&](auto it) __attribute__((always_inline)) {
+                sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+                    constexpr int t = decltype(it)::value, u = decltype(iu)::value;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sacc[u][t][r] = 0.f;
+                    Slab<uint16_t>::run(kone, mq[u], sacc[u][t]);
+                });
+            });
+        }
+        sfor<NG>([&](auto ig) __attribute__((always_inline)) {
+            constexpr int G = decltype(ig)::value;
+            if constexpr (KB == 1) kread(ig);
+            else if constexpr (G + 1 < NG) kread(std::integral_constant<int, G + 1>{});
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (KB == 2 && G + 1 < NG) wait_lgkmcnt<KG>(); else wait_lgkmcnt<0>();
+            sfor<KG>([&](auto ii) __attribute__((always_inline)) {
+                constexpr int i = decltype(ii)::value, f = G * KG + i, t = f / NS, s = f % NS;
+                sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+                    constexpr int u = decltype(iu)::value;
+                    if constexpr (s == 0 && !LZ) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) sacc[u][t][r] = 0.f;
+                    }
+                    Slab<uint16_t>::run(kf[G % KB][i], qf[u][s], sacc[u][t]);
+                });
+            });
+            __builtin_amdgcn_sched_barrier(0);
         });
-
     };
 
-    // ---- softmax in the base-2 domain, p = exp2(s*c2 + bias - m), and O^T += V^T . P^T for tile kt
-    auto phase_PV = [&](int kt) {
-        const int st = kt % NSTG, k0 = kt * KT;
-        const char* Vb = lds + OFF_V + st * TILE;
-        const float* Mb = (const float*)(lds + OFF_M + st * 1024);
-        const bool diag = p.causal && (k0 + KT - 1 > qw0);
-        const bool tail = k0 + KT > S;
-        const bool biased = HAS_MASK || tail;
-        const bool lazy = is_lazy(kt);
-        float pneg[QT];               // p = exp2(score + pneg); all zero on the fast path
-        bool fast = lazy;             // wave-uniform
-        sfor<QT>([&](auto iu) {
+    // maximum over this lane's scores of the tile, then over the two halves of the wave (one query = lanes l and l+32)
+    auto tile_max = [&](auto iu) __attribute__((always_inline)) {
+        constexpr int u = decltype(iu)::value;
+        float m0 = -__builtin_inff(), m1 = -__builtin_inff();
+#pragma unroll
+        for (int t = 0; t < NKB; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; r += 4) {
+                m0 = __builtin_fmaxf(__builtin_fmaxf(m0, sacc[u][t][r]), sacc[u][t][r + 1]);
+                m1 = __builtin_fmaxf(__builtin_fmaxf(m1, sacc[u][t][r + 2]), sacc[u][t][r + 3]);
+            }
+        return halves_max(__builtin_fmaxf(m0, m1));
+    };
+    // multiply what has been accumulated for query tile u by alpha (per lane = per query)
+    auto rescale = [&](auto iu, float alpha) __attribute__((always_inline)) {
+        constexpr int u = decltype(iu)::value;
+        lsum[u] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[u][dt][r] *= alpha;
+    };
+    // move the scores of the tile and the reference of later lazy tiles by -d (per lane)
+    auto shift = [&](auto iu, float d) __attribute__((always_inline)) {
+        constexpr int u = decltype(iu)::value;
+#pragma unroll
+        for (int t = 0; t < NKB; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[u][t][r] -= d;
+    };
+    // -m_run as the sum of three bf16 numbers (exact for any float: 3 x 8 significant bits), at k-indices 0, 1, 2 of the
+    // query side of the reference slab
+    auto set_negm = [&](auto iu) __attribute__((always_inline)) {
+        constexpr int u = decltype(iu)::value;
+        const float x = -m_run[u];
+        const uint32_t h1 = f2u(x) & 0xffff0000u;
+        const float r1 = x - u2f(h1);
+        const uint32_t h2 = f2u(r1) & 0xffff0000u;
+        const float r2 = r1 - u2f(h2);
+        mq[u][0] = lg == 0 ? ((h1 >> 16) | h2) : 0u;
+        mq[u][1] = lg == 0 ? (f2u(r2) >> 16) : 0u;
+    };
+
+    // key mask, diagonal and ragged end on the scores of the tile in stage ST (absolute or relative alike: the mask bias
+    // is additive, excluded keys become -inf)
+    auto mask_apply = [&](int kt, int ST, bool diag, bool tail) __attribute__((always_inline)) {
+        const int k0 = kt * KT;
+        const __attribute__((address_space(3))) float* Mb = (const __attribute__((address_space(3))) float*)(ldsp + OFF_M + ST * 1024);
+        sfor<QT>([&](auto iu) __attribute__((always_inline)) {
             constexpr int u = decltype(iu)::value;
             const int qi = qw0 + 32 * u + li;
-            float mx = -__builtin_inff();
-            if (biased || diag) {
-                sfor<NKB>([&](auto it) {
-                    constexpr int t = decltype(it)::value;
 #pragma unroll
-                    for (int qd = 0; qd < 4; ++qd) {
-                        const int kl = 32 * t + 8 * qd + 4 * lg;
-                        f32x4 mk = {1.f, 1.f, 1.f, 1.f};
-                        if (HAS_MASK) mk = *(const f32x4*)(Mb + kl);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            // (mask-1)*1e9 as the shader forms it, then into the base-2 domain
-                            float sv = sacc[u][t][4 * qd + e];
-                            if (HAS_MASK) sv += ((mk[e] - 1.0f) * 1e9f) * 1.4426950408889634f;
-                            if ((diag && (k0 + kl + e > qi)) || (tail && (k0 + kl + e >= S))) sv = -__builtin_inff();
-                            sacc[u][t][4 * qd + e] = sv;
-                            mx = __builtin_fmaxf(mx, sv);
-                        }
-                    }
-                });
-            } else {
-                sfor<NKB>([&](auto it) {
-                    constexpr int t = decltype(it)::value;
-#pragma unroll
-                    for (int r = 0; r < 16; r += 2) mx = __builtin_fmaxf(mx, __builtin_fmaxf(sacc[u][t][r], sacc[u][t][r + 1]));
-                });
-            }
-            mx = halves_max(mx);
-            if (!lazy) {
-                // absolute scores: the classic running maximum
-                mx = fmaxf(m_run[u], mx);
-                pneg[u] = -mx;
-                const float alpha = __builtin_amdgcn_exp2f(m_run[u] - mx);
-                // rescale the running output and sum only when some row of the wave raised its maximum
-                // (never for the first tile: there is nothing accumulated yet)
-                if (kt > 0 && __builtin_amdgcn_ballot_w64(mx != m_run[u]) != 0) {
-                    lsum[u] *= alpha;
-                    sfor<DT>([&](auto idt) {
-                        constexpr int dt = decltype(idt)::value;
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) oacc[u][dt][r] *= alpha;
-                    });
-                }
-                m_run[u] = mx;
-            } else {
-                // scores relative to m_run: move the reference only for rows that overshoot it by 2^LAZY
-                const float delta = mx > LAZY ? mx : 0.f;
-                pneg[u] = -delta;
-                if (__builtin_amdgcn_ballot_w64(delta != 0.f) != 0) {
-                    const float alpha = __builtin_amdgcn_exp2f(-delta);
-                    lsum[u] *= alpha;
-                    sfor<DT>([&](auto idt) {
-                        constexpr int dt = decltype(idt)::value;
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) oacc[u][dt][r] *= alpha;
-                    });
-                    m_run[u] += delta;
-                    fast = false;
-                }
-            }
-        });
-
-        // ---- O^T += V^T . P^T; V operand through the transposing LDS read
-        // source role of this lane inside its 16-lane group: key row j/4, 4 dims at 4*(j%4)
-        const int j16 = lane & 15, grp = lane >> 4;
-        auto pv_loop = [&](auto ifast) {
-        constexpr bool FAST = decltype(ifast)::value;
-        sfor<NKB>([&](auto it) {
-            constexpr int t = decltype(it)::value;
-#pragma unroll
-            for (int hh = 0; hh < 2; ++hh) {
-                // exponentials of this 16-key slab only: they are independent of the MFMAs of the previous
-                // slab, which lets the VALU work run under the matrix work instead of ahead of it
-                u32x4 pf[QT];
-#pragma unroll
-                for (int u = 0; u < QT; ++u)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float p0 = __builtin_amdgcn_exp2f(FAST ? sacc[u][t][8 * hh + 2 * e] : sacc[u][t][8 * hh + 2 * e] + pneg[u]);
-                        const float p1 = __builtin_amdgcn_exp2f(FAST ? sacc[u][t][8 * hh + 2 * e + 1] : sacc[u][t][8 * hh + 2 * e + 1] + pneg[u]);
-                        pf[u][e] = pack_bf16x2(p0, p1);
-                    }
-                // row sums of the rounded values
-                {
-                    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2v;
-                    const bf16x2v one2 = __builtin_bit_cast(bf16x2v, 0x3f803f80u);
-#pragma unroll
-                    for (int u = 0; u < QT; ++u)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint32_t w = pf[u][e];
-                            lsum[u] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2v, w), one2, lsum[u], false);
-                        }
-                }
-                // keys of MFMA k-index (g, e): 32t + 16hh + 8*(e/4) + 4g + e%4, g = lane/32
-                const int kA = 32 * t + 16 * hh + 4 * (grp >> 1) + (j16 >> 2);
-                sfor<DT>([&](auto idt) {
-                    constexpr int dt = decltype(idt)::value;
-                    const int dcol = 32 * dt + 16 * (grp & 1) + 4 * (j16 & 3);     // first of 4 dims this lane points at
-                    const int ch = dcol >> 3, sub = (dcol & 7) * 2;
-                    auto addr = [&](int key) {
-                        const int slot = ch ^ lds_swz_v<NCH>(key);
-                        return (__attribute__((address_space(3))) s16x4_t*)(Vb + key * RB + slot * 16 + sub);
-                    };
-                    s16x4_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16(addr(kA));
-                    s16x4_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16(addr(kA + 8));
-                    u32x2 wa = __builtin_bit_cast(u32x2, va), wb = __builtin_bit_cast(u32x2, vb);
-                    u32x4 vf = {wa[0], wa[1], wb[0], wb[1]};
-                    sfor<QT>([&](auto iu) { Slab<uint16_t>::run(vf, pf[decltype(iu)::value], oacc[decltype(iu)::value][dt]); });
-                });
-            }
-        });
-        };
-        if (fast) pv_loop(std::true_type{}); else pv_loop(std::false_type{});
-    };
-
-    // (A "ping-pong" schedule -- the two waves of a SIMD half a tile apart, one in the score phase while the
-    // other is in the softmax + PV phase, one barrier per half tile -- was built and measured: correct, 6-10 %
-    // slower; inside the PV phase the two waves already overlap each other's VALU and matrix work.)
-    for (int t = 1; t < NSTG - 1 && t < nkt; ++t) issue(t);
-    wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1);
-    for (int kt = 0; kt < nkt; ++kt) {
-        // tiles kt+1 .. kt+NSTG-2 may still be in flight; tile kt (this wave's part) must have landed
-        wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1 - kt);
-        // barrier without a memory fence (a fence would wait for every transfer in flight): LDS
-        // writes of this wave are drained by lgkmcnt(0), its tile transfers by the wait above
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        // into the stage tile kt-1 has just left.  (Letting only one wave of each SIMD pair request the tile, as
-        // the GEMM does, was measured here too: no gain.)
-        if (kt + NSTG - 1 < nkt) issue(kt + NSTG - 1);
-        zero_tail(kt);
-        if (skip_tile(kt)) continue;
-        phase_S(kt);
-        phase_PV(kt);
-    }
-
-#pragma unroll
-    for (int u = 0; u < QT; ++u) {
-        const int qi = qw0 + 32 * u + li;
-        const float inv = 1.0f / fmaxf(halves_sum(lsum[u]), 1e-10f);
-        if (qi < S) {
-            uint16_t* Og = p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+            for (int t = 0; t < NKB; ++t)
 #pragma unroll
                 for (int qd = 0; qd < 4; ++qd) {
-                    const int d = 32 * dt + 8 * qd + 4 * lg;
-                    fa_store4<uint16_t>(Og + d, oacc[u][dt][4 * qd] * inv, oacc[u][dt][4 * qd + 1] * inv, oacc[u][dt][4 * qd + 2] * inv, oacc[u][dt][4 * qd + 3] * inv);
+                    const int kl = 32 * t + 8 * qd + 4 * lg;
+                    f32x4 mk = {1.f, 1.f, 1.f, 1.f};
+                    if (HAS_MASK) mk = *(const __attribute__((address_space(3))) f32x4*)(Mb + kl);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        // (mask-1)*1e9 as the shader forms it, then into the base-2 domain
+                        float sv = sacc[u][t][4 * qd + e];
+                        if (HAS_MASK) sv += ((mk[e] - 1.0f) * 1e9f) * 1.4426950408889634f;
+                        if ((diag && (k0 + kl + e > qi)) || (tail && (k0 + kl + e >= S))) sv = -__builtin_inff();
+                        sacc[u][t][4 * qd + e] = sv;
+                    }
                 }
+        });
+    };
+    // ---- softmax reference.  The first tile sets the reference m_run to its row maxima.  Every later tile is computed
+    // relative to m_run (the reference slab puts -m_run into its score accumulators, so the exponentials need no further
+    // arithmetic); m_run moves, with the usual rescale of what has been accumulated, only for rows that overshoot it by
+    // more than 2^LAZY, and the tile's scores are then computed again against the new reference.  m_run is thus a
+    // reference point at most LAZY below the true running maximum, which the softmax quotient does not depend on.
+    // overshoot(): does any row of the wave exceed the reference by more than 2^LAZY?  raise(): move those rows' reference.
+    float mx_tile[QT];
+    auto overshoot = [&]() __attribute__((always_inline)) {
+        bool any = false;
+        sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+            constexpr int u = decltype(iu)::value;
+            mx_tile[u] = tile_max(iu);
+            any = any || __builtin_amdgcn_ballot_w64(mx_tile[u] > LAZY) != 0;
+        });
+        return any;
+    };
+    // mx_tile holds the tile's ABSOLUTE row maxima: rows that exceed their reference by more than 2^LAZY take the maximum
+    // as their new reference, and what they have accumulated is rescaled
+    auto raise = [&]() __attribute__((always_inline)) {
+        mfma_drain();
+        sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+            constexpr int u = decltype(iu)::value;
+            const float m_new = mx_tile[u] > m_run[u] + LAZY ? mx_tile[u] : m_run[u];
+            rescale(iu, __builtin_amdgcn_exp2f(m_run[u] - m_new));
+            m_run[u] = m_new;
+            set_negm(iu);
+        });
+    };
+
+    // ---- p = exp2(score), O^T += V^T . P^T; V operand through the transposing LDS read: inside a 16-lane group source
+    // lane j points at key j/4, 4 dims at 4*(j%4); keys of MFMA k-index (g, e): 32t + 16hh + 8*(e/4) + 4g + e%4, g = lane/32
+    constexpr int VB = 1;                                    // the same choice for the V fragments of a 16-key slab
+    constexpr int NSL = 2 * NKB;                             // 16-key slabs per tile
+    auto phase_PV = [&](int ST, auto iinplace) __attribute__((always_inline)) {
+        // INPLACE: the accumulate through mfma_inplace (first loop); else the builtin, whose hazards and spills the compiler
+        // manages itself (tile 0 and the second loop, where register moves do not matter)
+        constexpr bool INPLACE = decltype(iinplace)::value;
+        const lds_char* vb[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vb[dt] = vbase[dt] + ST * TILE;
+        u32x2 vf[VB][DT][2];
+        auto vread = [&](auto isl) __attribute__((always_inline)) {
+            constexpr int SL = decltype(isl)::value;
+            sfor<DT>([&](auto idt) __attribute__((always_inline)) {
+                constexpr int dt = decltype(idt)::value;
+                sfor<2>([&](auto ihb) __attribute__((always_inline)) {
+                    constexpr int hb = decltype(ihb)::value;
+                    const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4_t*)(vb[dt] + (16 * SL + 8 * hb) * RB));
+                    vf[SL % VB][dt][hb] = __builtin_bit_cast(u32x2, v);
+                });
+            });
+        };
+        if constexpr (VB == 2) vread(std::integral_constant<int, 0>{});
+        sfor<NSL>([&](auto isl) __attribute__((always_inline)) {
+            constexpr int SL = decltype(isl)::value, t = SL / 2, hh = SL % 2;
+            if constexpr (VB == 1) vread(isl);
+            else if constexpr (SL + 1 < NSL) vread(std::integral_constant<int, SL + 1>{});
+            u32x4 pf[QT];
+            typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2v;
+            const bf16x2v one2 = __builtin_bit_cast(bf16x2v, 0x3f803f80u);
+#pragma unroll
+            for (int u = 0; u < QT; ++u)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float p0 = __builtin_amdgcn_exp2f(sacc[u][t][8 * hh + 2 * e]);
+                    const float p1 = __builtin_amdgcn_exp2f(sacc[u][t][8 * hh + 2 * e + 1]);
+                    pf[u][e] = pack_bf16x2(p0, p1);
+                }
+            if constexpr (VB == 2 && SL + 1 < NSL) wait_lgkmcnt<2 * DT>(); else wait_lgkmcnt<0>();
+            u32x4 v4[DT];
+            sfor<DT>([&](auto idt) __attribute__((always_inline)) {
+                constexpr int dt = decltype(idt)::value;
+                v4[dt] = u32x4{vf[SL % VB][dt][0][0], vf[SL % VB][dt][0][1], vf[SL % VB][dt][1][0], vf[SL % VB][dt][1][1]};
+            });
+            __builtin_amdgcn_sched_barrier(0);
+            // row sums of the rounded values
+#pragma unroll
+            for (int u = 0; u < QT; ++u)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t w = pf[u][e];
+                    lsum[u] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2v, w), one2, lsum[u], false);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+            sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+                constexpr int u = decltype(iu)::value;
+                if constexpr (INPLACE) mfma_inplace<DT>(v4, pf[u], oacc[u]);
+                else sfor<DT>([&](auto idt) __attribute__((always_inline)) { Slab<uint16_t>::run(v4[decltype(idt)::value], pf[u], oacc[u][decltype(idt)::value]); });
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    // last, partial tile: rows >= S hold whatever the out-of-range transfer left; clear them (all threads)
+    auto zero_tail = [&](int kt, int ST) __attribute__((always_inline)) {
+        const int first = S - kt * KT;
+        for (int i = tid; i < (KT - first) * NCH; i += NT) {
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            *(u32x4*)(lds + ST * TILE + first * RB + i * 16) = zero;
+            *(u32x4*)(lds + OFF_V + ST * TILE + first * RB + i * 16) = zero;
         }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+
+    // tile kt's turn: its transfers have landed for everybody, the stage tile kt-1 has left takes the next transfer
+    auto enter_tile = [&](int kt, int ST) __attribute__((always_inline)) {
+        // tiles kt+1 .. kt+NSTG-2 may still be in flight; tile kt (this wave's part) must have landed.  Barrier without a
+        // memory fence (a fence would wait for every transfer in flight): this wave's LDS accesses are drained by
+        // lgkmcnt(0), its tile transfers by the counted wait.
+        if constexpr (NSTG == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else {
+            wait_tiles_outstanding<IPT, NSTG - 2>(nkt - 1 - kt);
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        }
+        if (kt + NSTG - 1 < nkt) issue(kt + NSTG - 1, ST == 0 ? NSTG - 1 : ST - 1);
+        if (__builtin_expect(kt * KT + KT > S, 0)) zero_tail(kt, ST);
+    };
+    auto is_diag = [&](int kt) __attribute__((always_inline)) { return p.causal && (kt * KT + KT - 1 > qw0); };
+    auto is_tail = [&](int kt) __attribute__((always_inline)) { return kt * KT + KT > S; };
+    auto relative_scores = [&](int kt, int ST) __attribute__((always_inline)) {
+        phase_S(ST, std::true_type{});
+        const bool diag = is_diag(kt), tail = is_tail(kt);
+        if (HAS_MASK || diag || tail) mask_apply(kt, ST, diag, tail);
+    };
+    auto absolute_scores = [&](int kt, int ST) __attribute__((always_inline)) {
+        phase_S(ST, std::false_type{});
+        const bool diag = is_diag(kt), tail = is_tail(kt);
+        if (HAS_MASK || diag || tail) mask_apply(kt, ST, diag, tail);
+    };
+    auto next_stage = [&](int st) __attribute__((always_inline)) { return st + 1 == NSTG ? 0 : st + 1; };
+
+    for (int t = 1; t < NSTG - 1 && t < nkt; ++t) issue_rt(t);
+    // ---- tile 0 sets the softmax reference: absolute scores, exact row maxima (rounded to bf16)
+    {
+        enter_tile(0, 0);
+        absolute_scores(0, 0);
+        sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+            constexpr int u = decltype(iu)::value;
+            m_run[u] = tile_max(iu);
+            shift(iu, m_run[u]);
+            set_negm(iu);
+        });
+        phase_PV(0, std::false_type{});
     }
+    // normalise and store this wave's rows
+    auto finish = [&]() __attribute__((always_inline)) {
+    mfma_drain();
+#pragma unroll
+        for (int u = 0; u < QT; ++u) {
+            const int qi = qw0 + 32 * u + li;
+            const float inv = 1.0f / fmaxf(halves_sum(lsum[u]), 1e-10f);
+            if (qi < S) {
+                uint16_t* Og = p.O + ((int64_t)b * S + qi) * p.o_stride + h * D;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int qd = 0; qd < 4; ++qd) {
+                        const int d = 32 * dt + 8 * qd + 4 * lg;
+                        fa_store4<uint16_t>(Og + d, oacc[u][dt][4 * qd] * inv, oacc[u][dt][4 * qd + 1] * inv, oacc[u][dt][4 * qd + 2] * inv, oacc[u][dt][4 * qd + 3] * inv);
+                    }
+            }
+        }
+    };
+    // ---- all later tiles.  The first loop is the common case, and nothing in it rewrites the accumulators except the PV
+    // matrix products themselves (in place).  A tile whose scores overshoot the reference leaves it for the second loop,
+    // which finishes the sequence with the reference raised (and the accumulated output rescaled) wherever needed; it is
+    // not entered again from there, so the first loop has no path that joins it with rescaled accumulators.
+    int kt = 1, st = 1 % NSTG;
+    int over = 0;
+    for (; kt < nkt; ++kt, st = next_stage(st)) {
+        enter_tile(kt, st);
+        // a wave whose queries all precede the tile has nothing to add (causal): it only keeps the barriers
+        if (p.causal && kt * KT > qw0 + QW - 1) continue;
+        relative_scores(kt, st);
+        if (__builtin_expect(overshoot(), 0)) { over = 1; break; }
+        phase_PV(st, std::true_type{});
+    }
+    // (the flag passes through an opaque statement: the first loop then has one exit block, and the register allocator keeps
+    // the accumulators in place inside it; with the overshoot exit wired straight to the second loop it gives them a second
+    // home and moves all 32 registers there and back in every pass)
+    asm volatile("" : "+s"(over));
+    if (__builtin_expect(over != 0, 0)) {
+        // The accumulators enter this loop through private memory: handed over in registers, the two loops' accumulators
+        // become one value for the register allocator, which then moves all 32 registers to a second home and back in
+        // every pass of the first loop.
+        mfma_drain();
+        {
+            volatile float stash[QT * DT * 16];
+            sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+                sfor<DT>([&](auto idt) __attribute__((always_inline)) {
+                    constexpr int u = decltype(iu)::value, dt = decltype(idt)::value;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) stash[(u * DT + dt) * 16 + r] = oacc[u][dt][r];
+                });
+            });
+            sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+                sfor<DT>([&](auto idt) __attribute__((always_inline)) {
+                    constexpr int u = decltype(iu)::value, dt = decltype(idt)::value;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[u][dt][r] = stash[(u * DT + dt) * 16 + r];
+                });
+            });
+        }
+        for (;;) {
+            // tile kt has been entered and its scores stand in sacc, relative to the present reference.  Where they overshoot
+            // it, the new reference comes from the tile's absolute scores (exact whatever the old reference was: relative
+            // scores lose their low bits against a reference like the -1.4e9 of a fully masked tile).
+            if (overshoot()) {
+                absolute_scores(kt, st);
+                sfor<QT>([&](auto iu) __attribute__((always_inline)) { mx_tile[decltype(iu)::value] = tile_max(iu); });
+                raise();
+                relative_scores(kt, st);
+            }
+            phase_PV(st, std::false_type{});
+            do {
+                ++kt; st = next_stage(st);
+                if (kt < nkt) enter_tile(kt, st);
+            } while (kt < nkt && p.causal && kt * KT > qw0 + QW - 1);
+            if (kt >= nkt) break;
+            relative_scores(kt, st);
+        }
+        // (a store sequence of its own: the two loops' accumulators never meet)
+        finish();
+        return;
+    }
+
+    finish();
 }
 
 template <int D, int QT, int NW, int NSTG, int KT, int OCC = (NW == 4 ? 2 : 1)>
@@ -760,14 +925,17 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, int rope_q) {
     f.order = order_env >= 0 ? order_env : ((a.causal || a.S <= 1024) ? 1 : 0);
     f.q_stride = a.q_stride; f.k_stride = a.k_stride; f.v_stride = a.v_stride; f.o_stride = a.o_stride;
     // GRL_FA_CFG forces a configuration, for tuning runs:
-    //   1: 8 waves, 64-key tiles, deep ring   2: 8 waves, 128-key tiles   3: 4 waves, 64-key tiles, 4 stages
+    //   1: 8 waves, 64-key tiles, deep ring   2: 8 waves, 128-key tiles   3: 4 waves, 64-key tiles, 4 stages (head dims up to 64)
     //   4: 4 waves, 128-key tiles, half-size ring (two workgroups per CU)
     //   5: 4 waves, 64-key tiles, two stages, three workgroups per CU (head dims up to 64)
     static const int forced = [] { const char* e = getenv("GRL_FA_CFG"); return e ? atoi(e) : 0; }();
     // short sequences are bound by per-workgroup latency (first-tile wait, output stores): two or, where the
     // registers allow it (head dims up to 64), three small workgroups per CU hide each other's; long ones: one
     // 8-wave workgroup with the full ring
-    int cfg = forced >= 1 && forced <= 5 ? forced : (a.S > 1024 ? 2 : (D <= 64 ? 5 : (a.S > 128 ? 4 : 3)));
+    int cfg = forced >= 1 && forced <= 5 ? forced : (a.S > 1024 ? 2 : (D <= 64 ? 5 : 4));
+    // (head dim 128 has no 4-stage instantiation: it does not fit the 256 registers of two waves per SIMD, and the
+    // accumulators must not move to AGPRs next to the in-place MFMAs; the build turns a missed register budget into an error)
+    if (D == 128 && cfg == 3) cfg = 4;
     constexpr int DEEP = D == 128 ? 4 : 8;        // 128 KiB of K/V tiles: D=128 -> 4 x 32 KiB, else 8 x 16 (8) KiB
     switch (cfg) {
         case 1: return launch_fa16_cfg<D, 1, 8, DEEP, 64>(c, f, rope_q);
@@ -776,7 +944,8 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, int rope_q) {
         case 5: if constexpr (D <= 64) return launch_fa16_cfg<D, 1, 4, 2, 64, 3>(c, f, rope_q); else break;
         default: break;
     }
-    return launch_fa16_cfg<D, 1, 4, 4, 64>(c, f, rope_q);
+    if constexpr (D <= 64) return launch_fa16_cfg<D, 1, 4, 4, 64>(c, f, rope_q);
+    else return launch_fa16_cfg<D, 1, 4, 2, 64>(c, f, rope_q);
 }
 
 template <typename T, int D>
