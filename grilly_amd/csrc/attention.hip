@@ -313,17 +313,23 @@ __global__ __launch_bounds__(256) void fa2_fwd_kernel(FaArgs p) {
 }
 
 // =====================================================================================
-// bf16 kernel, second generation.
+// bf16 kernel.
 //
-//   K and V tiles (64 keys) go HBM -> LDS by buffer_load ... lds (no staging registers), both
-//   row-major [key][d] with the 16-byte chunks XOR-swizzled by key, double buffered.
+//   K and V tiles (64 or 128 keys) go HBM -> LDS by buffer_load ... lds (no staging registers), both
+//   row-major [key][d] with the 16-byte chunks XOR-swizzled by key, in a ring of 2-8 stages.
 //   S^T = K.Q^T reads K with ds_read_b128; O^T += V^T.P^T reads V with the transposing
 //   ds_read_b64_tr_b16: inside a 16-lane group, source lane j points at
 //   V[k0 + j/4][d0 + 4*(j%4) ..] and result lane i receives V[k0 .. k0+3][d0 + i], i.e. four
 //   consecutive keys of ONE head dimension -- the MFMA operand -- without any shuffling.
-//   Softmax works in the base-2 domain: p = exp2(s*scale*log2e - m), one v_exp_f32 per score.
-//   About 130-190 VGPRs, so 2-3 workgroups share a CU and one wave's softmax VALU work
-//   overlaps another's MFMAs.
+//   Softmax works in the base-2 domain, p = exp2(s*scale*log2e - m), one v_exp_f32 per score, and the
+//   subtraction of m is done by the matrix core (one more k-slab, see the kernel).
+//   The kernel is bound by instruction issue, not by any one pipeline (SQ counters: a SIMD issues one
+//   instruction of any kind per four cycles, and the sum of its waves' active cycles fills the kernel
+//   time), so the tile loop is kept to the instructions the algorithm needs: per 32 queries x 64 keys
+//   at head dim 64, 17 MFMA + 32 v_exp + 16 v_cvt_pk + 16 v_dot2c + 17 v_max3 + 24 LDS reads, about
+//   45 scalar and 10 wait instructions.  What that takes: wave-uniform values are declared so
+//   (readfirstlane), transfers are addressed through scalar registers, the common tile has a loop of its
+//   own that nothing else joins, and the PV accumulates are tied in place.
 //   RoPE: each Q row is rotated once as it is loaded; K is rotated once per row by the host
 //   wrapper into a workspace (rotating K inside the kernel would redo it for every query block).
 // =====================================================================================
@@ -828,69 +834,52 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
             }
         }
     };
-    // ---- all later tiles.  The first loop is the common case, and nothing in it rewrites the accumulators except the PV
-    // matrix products themselves (in place).  A tile whose scores overshoot the reference leaves it for the second loop,
-    // which finishes the sequence with the reference raised (and the accumulated output rescaled) wherever needed; it is
-    // not entered again from there, so the first loop has no path that joins it with rescaled accumulators.
+    // ---- all later tiles.  The inner loop is the common case, and nothing in it rewrites the accumulators except the PV
+    // matrix products themselves (in place).  A tile whose scores overshoot the reference leaves it, is handled below
+    // (reference raised from the tile's absolute scores, accumulated output rescaled, scores formed again), and the inner
+    // loop is entered again.  The accumulators come back to it through opaque register moves: handed back as they are, the
+    // handler's and the loop's accumulators become one value for the register allocator, which then gives them a second home
+    // and moves all of them there and back in every pass of the inner loop.
+    auto hand_back = [&]() __attribute__((always_inline)) {
+        mfma_drain();      // the moves below are inline asm too: the compiler adds no wait states between the PV MFMAs and them
+        sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+            sfor<DT>([&](auto idt) __attribute__((always_inline)) {
+                constexpr int u = decltype(iu)::value, dt = decltype(idt)::value;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float t;
+                    asm volatile("v_mov_b32 %0, %1" : "=v"(t) : "v"(oacc[u][dt][r]));
+                    oacc[u][dt][r] = t;
+                }
+            });
+        });
+    };
     int kt = 1, st = 1 % NSTG;
-    int over = 0;
-    for (; kt < nkt; ++kt, st = next_stage(st)) {
-        enter_tile(kt, st);
-        // a wave whose queries all precede the tile has nothing to add (causal): it only keeps the barriers
-        if (p.causal && kt * KT > qw0 + QW - 1) continue;
-        relative_scores(kt, st);
-        if (__builtin_expect(overshoot(), 0)) { over = 1; break; }
-        phase_PV(st, std::true_type{});
-    }
-    // (the flag passes through an opaque statement: the first loop then has one exit block, and the register allocator keeps
-    // the accumulators in place inside it; with the overshoot exit wired straight to the second loop it gives them a second
-    // home and moves all 32 registers there and back in every pass)
-    asm volatile("" : "+s"(over));
-    if (__builtin_expect(over != 0, 0)) {
-        // The accumulators enter this loop through private memory: handed over in registers, the two loops' accumulators
-        // become one value for the register allocator, which then moves all 32 registers to a second home and back in
-        // every pass of the first loop.
-        mfma_drain();
-        {
-            volatile float stash[QT * DT * 16];
-            sfor<QT>([&](auto iu) __attribute__((always_inline)) {
-                sfor<DT>([&](auto idt) __attribute__((always_inline)) {
-                    constexpr int u = decltype(iu)::value, dt = decltype(idt)::value;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) stash[(u * DT + dt) * 16 + r] = oacc[u][dt][r];
-                });
-            });
-            sfor<QT>([&](auto iu) __attribute__((always_inline)) {
-                sfor<DT>([&](auto idt) __attribute__((always_inline)) {
-                    constexpr int u = decltype(iu)::value, dt = decltype(idt)::value;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[u][dt][r] = stash[(u * DT + dt) * 16 + r];
-                });
-            });
-        }
-        for (;;) {
-            // tile kt has been entered and its scores stand in sacc, relative to the present reference.  Where they overshoot
-            // it, the new reference comes from the tile's absolute scores (exact whatever the old reference was: relative
-            // scores lose their low bits against a reference like the -1.4e9 of a fully masked tile).
-            if (overshoot()) {
-                absolute_scores(kt, st);
-                sfor<QT>([&](auto iu) __attribute__((always_inline)) { mx_tile[decltype(iu)::value] = tile_max(iu); });
-                raise();
-                relative_scores(kt, st);
-            }
-            phase_PV(st, std::false_type{});
-            do {
-                ++kt; st = next_stage(st);
-                if (kt < nkt) enter_tile(kt, st);
-            } while (kt < nkt && p.causal && kt * KT > qw0 + QW - 1);
-            if (kt >= nkt) break;
+    for (;;) {
+        int over = 0;
+        for (; kt < nkt; ++kt, st = next_stage(st)) {
+            enter_tile(kt, st);
+            // a wave whose queries all precede the tile has nothing to add (causal): it only keeps the barriers
+            if (p.causal && kt * KT > qw0 + QW - 1) continue;
             relative_scores(kt, st);
+            if (__builtin_expect(overshoot(), 0)) { over = 1; break; }
+            phase_PV(st, std::true_type{});
         }
-        // (a store sequence of its own: the two loops' accumulators never meet)
-        finish();
-        return;
+        // (the flag passes through an opaque statement: the inner loop then has one exit block)
+        asm volatile("" : "+s"(over));
+        if (__builtin_expect(over == 0, 1)) break;
+        // tile kt has been entered and its scores stand in sacc, relative to the present reference, which some row exceeds
+        // by more than 2^LAZY.  The new reference comes from the tile's absolute scores (exact whatever the old reference
+        // was: relative scores lose their low bits against a reference like the -1.4e9 of a fully masked tile).
+        mfma_drain();
+        absolute_scores(kt, st);
+        sfor<QT>([&](auto iu) __attribute__((always_inline)) { mx_tile[decltype(iu)::value] = tile_max(iu); });
+        raise();
+        relative_scores(kt, st);
+        phase_PV(st, std::false_type{});
+        ++kt; st = next_stage(st);
+        hand_back();
     }
-
     finish();
 }
 

@@ -90,3 +90,24 @@ def test_fa2_running_maximum_rescale(backend, dtype, D, S, shape):
         ref = O.truth_attention(q, k, v, causal=causal)
         assert np.isfinite(o).all()
         assert O.max_rel(o, ref) < tol(dtype), (shape, causal)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("S,D", [(200, 64), (512, 64), (512, 32), (300, 128), (1300, 64), (1300, 128)])
+def test_fa2_mask_layouts(backend, dtype, S, D):
+    """Key masks other than right padding: whole leading tiles masked out (left padding of 70 and of 130 keys: the
+    softmax reference of those rows starts at the -1e9 of masked scores and has to come up to the first real
+    key's), holes inside the sequence, and a single visible key (the output is that key's value row)."""
+    B, H = 4, 2
+    rng = np.random.default_rng(S * 3 + D)
+    q, k, v = qkv(rng, B, S, H, D, dtype)
+    mask = np.ones((B, S), np.float32)
+    mask[0, :70] = 0
+    mask[1, :130] = 0; mask[1, S - 9:] = 0
+    mask[2, 40:110] = 0; mask[2, 150:170] = 0
+    mask[3, :] = 0; mask[3, 137] = 1
+    o = backend.attention.flash_attention2(q, k, v, H, D, mask=mask, dtype=dtype)
+    assert np.isfinite(o).all()
+    ref = O.truth_attention(q, k, v, mask=mask)
+    assert O.max_rel(o, ref) < tol(dtype)
+    np.testing.assert_allclose(o[3], np.broadcast_to(v[3, 137], o[3].shape), atol=1e-6 if dtype == "fp32" else 1e-2)
