@@ -883,16 +883,18 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     finish();
 }
 
-template <int D, int QT, int NW, int NSTG, int KT, int OCC = (NW == 4 ? 2 : 1)>
+// OCC / OCCM: workgroups per CU the registers are budgeted for, without / with a key mask (applying the mask takes about
+// 40 more registers)
+template <int D, int QT, int NW, int NSTG, int KT, int OCC = (NW == 4 ? 2 : 1), int OCCM = OCC>
 static int launch_fa16_cfg(grl_ctx* c, const Fa16Args& f, int rope_q) {
     const int qb = 32 * QT * NW;
     const int64_t nwg = (int64_t)((f.S + qb - 1) / qb) * f.H * f.B;
     GRL_REQUIRE(nwg < (1LL << 31), GRL_ERR_SHAPE, "attention: %lld workgroups exceed the grid limit", (long long)nwg);
     dim3 grid((unsigned)nwg), block(NW * 64);
     if (f.mask) {
-        if (rope_q == 2) hipLaunchKernelGGL((fa2_bf16_kernel<D, 2, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
-        else if (rope_q == 1) hipLaunchKernelGGL((fa2_bf16_kernel<D, 1, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
-        else hipLaunchKernelGGL((fa2_bf16_kernel<D, 0, QT, NW, NSTG, true, KT, OCC>), grid, block, 0, c->stream, f);
+        if (rope_q == 2) hipLaunchKernelGGL((fa2_bf16_kernel<D, 2, QT, NW, NSTG, true, KT, OCCM>), grid, block, 0, c->stream, f);
+        else if (rope_q == 1) hipLaunchKernelGGL((fa2_bf16_kernel<D, 1, QT, NW, NSTG, true, KT, OCCM>), grid, block, 0, c->stream, f);
+        else hipLaunchKernelGGL((fa2_bf16_kernel<D, 0, QT, NW, NSTG, true, KT, OCCM>), grid, block, 0, c->stream, f);
     } else {
         if (rope_q == 2) hipLaunchKernelGGL((fa2_bf16_kernel<D, 2, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
         else if (rope_q == 1) hipLaunchKernelGGL((fa2_bf16_kernel<D, 1, QT, NW, NSTG, false, KT, OCC>), grid, block, 0, c->stream, f);
@@ -916,11 +918,11 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, int rope_q) {
     // GRL_FA_CFG forces a configuration, for tuning runs:
     //   1: 8 waves, 64-key tiles, deep ring   2: 8 waves, 128-key tiles   3: 4 waves, 64-key tiles, 4 stages (head dims up to 64)
     //   4: 4 waves, 128-key tiles, half-size ring (two workgroups per CU)
-    //   5: 4 waves, 64-key tiles, two stages, three workgroups per CU (head dims up to 64)
+    //   5: 4 waves, 64-key tiles, two stages, four workgroups per CU, three with a key mask (head dims up to 64)
     static const int forced = [] { const char* e = getenv("GRL_FA_CFG"); return e ? atoi(e) : 0; }();
     // short sequences are bound by per-workgroup latency (first-tile wait, output stores): two or, where the
-    // registers allow it (head dims up to 64), three small workgroups per CU hide each other's; long ones: one
-    // 8-wave workgroup with the full ring
+    // registers allow it (head dims up to 64), three to four small workgroups per CU hide each other's; long ones:
+    // one 8-wave workgroup with the full ring
     int cfg = forced >= 1 && forced <= 5 ? forced : (a.S > 1024 ? 2 : (D <= 64 ? 5 : 4));
     // (head dim 128 has no 4-stage instantiation: it does not fit the 256 registers of two waves per SIMD, and the
     // accumulators must not move to AGPRs next to the in-place MFMAs; the build turns a missed register budget into an error)
@@ -930,7 +932,7 @@ static int launch_fa16(grl_ctx* c, const FaArgs& a, int rope_q) {
         case 1: return launch_fa16_cfg<D, 1, 8, DEEP, 64>(c, f, rope_q);
         case 2: return launch_fa16_cfg<D, 1, 8, DEEP / 2, 128>(c, f, rope_q);
         case 4: return launch_fa16_cfg<D, 1, 4, 2, (D == 128 ? 64 : 128)>(c, f, rope_q);
-        case 5: if constexpr (D <= 64) return launch_fa16_cfg<D, 1, 4, 2, 64, 3>(c, f, rope_q); else break;
+        case 5: if constexpr (D <= 64) return launch_fa16_cfg<D, 1, 4, 2, 64, 4, 3>(c, f, rope_q); else break;
         default: break;
     }
     if constexpr (D <= 64) return launch_fa16_cfg<D, 1, 4, 4, 64>(c, f, rope_q);
