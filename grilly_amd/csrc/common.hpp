@@ -223,14 +223,31 @@ __device__ __forceinline__ float silu_clamped(float x) {
 __device__ __forceinline__ float silu_plain(float x) {
     return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
 }
+// v_mul_legacy_f32 (0 times anything, infinities and NaN included, is 0); the intrinsic has no clang builtin
+extern "C" __device__ float fmul_legacy(float, float) __asm("llvm.amdgcn.fmul.legacy");
 // shaders/fused-linear-gelu.glsl:45-63 rewritten with tanh(u) = 2/(1+exp(-2u)) - 1:
 //   0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (c + 0.044715 c^3), c = clamp(x, +-50).
 // The +-50 clamp needs no instruction of its own: beyond |x| = 50 (already from |x| > 7) the exponential saturates
-// to 0 / +inf, also when x*x overflows, which yields x and (-)0: the shader's rule for |x| > 50.  Only x = -inf
-// would give (-inf)*0; the lower bound keeps that at -0 (the shader returns 0 there), +inf stays +inf.
+// to 0 / +inf, also when x*x overflows, which yields x and (-)0: the shader's rule for |x| > 50.  x = -inf would give
+// (-inf)*0 = NaN with an IEEE multiply; the last product is v_mul_legacy_f32 (0 times anything is 0), which returns the
+// shader's 0 there and is the same product everywhere else; +inf stays +inf.
 __device__ __forceinline__ float gelu_fast(float x) {
-    x = fmaxf(x, -3.0e38f);
     float e = x * (-2.302208198f + -0.10294324f * (x * x));     // -2u*log2(e)
-    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e));
+    return fmul_legacy(x, __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e)));
+}
+// four values stage by stage: the result of an exponential or reciprocal is then never needed by the very next
+// instruction (one s_nop per value otherwise, in epilogues that are bound by instruction issue)
+__device__ __forceinline__ void gelu_fast4(float (&v)[4]) {
+    float e[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = v[i] * (-2.302208198f + -0.10294324f * (v[i] * v[i]));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = __builtin_amdgcn_exp2f(e[i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = 1.0f + e[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = __builtin_amdgcn_rcpf(e[i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = fmul_legacy(v[i], e[i]);
 }
 #endif

@@ -192,6 +192,8 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = glu_apply(v[e], u[e], p);
                         } else {
+                            if constexpr (EPI == EPI_GELU) gelu_fast4(v);
+                            else
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
                             if constexpr (EPI == EPI_RES) add4<OutT>((const OutT*)p.residual + o, v);
@@ -651,6 +653,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                                 v[e] = glu_apply(v[e], up, p);
                             }
                         } else {
+                            if constexpr (EPI == EPI_GELU) gelu_fast4(v);
+                            else
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
                         }
