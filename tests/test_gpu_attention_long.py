@@ -111,3 +111,44 @@ def test_fa2_mask_layouts(backend, dtype, S, D):
     ref = O.truth_attention(q, k, v, mask=mask)
     assert O.max_rel(o, ref) < tol(dtype)
     np.testing.assert_allclose(o[3], np.broadcast_to(v[3, 137], o[3].shape), atol=1e-6 if dtype == "fp32" else 1e-2)
+
+
+def test_fa2_randomized_configurations(backend):
+    """Seeded sweep over what steers the bf16 kernel's paths: sequence length (whole and ragged tiles, below and above
+    the 1024-key switch to eight-wave workgroups), head dim, causal, key masks with random holes and padding on either
+    side, and score profiles that raise the row maximum at random keys (the rare path of the tile loop, possibly several
+    times per row and next to masked or diagonal tiles).  Every case against the float64 closed form."""
+    rng = np.random.default_rng(20240611)
+    worst = 0.0
+    for case in range(36):
+        D = int(rng.choice([32, 64, 128]))
+        S = int(rng.choice([65, 128, 191, 256, 448, 512, 777, 1024, 1100, 1536]))
+        B, H = 2, int(rng.choice([1, 3]))
+        causal = bool(rng.integers(0, 2))
+        q = rng.standard_normal((B, S, H, D)).astype(np.float32)
+        k = rng.standard_normal((B, S, H, D)).astype(np.float32)
+        v = rng.standard_normal((B, S, H, D)).astype(np.float32)
+        kind = case % 3
+        if kind == 1:          # a few keys line up with every query: jumps of the running maximum at random places
+            qdir = np.abs(rng.standard_normal((1, 1, H, D))).astype(np.float32)
+            q = np.abs(q) * 0.5 + qdir
+            jumps = np.cumsum(np.where(rng.random(S) < 0.02, rng.uniform(4.0, 30.0, S), 0.0))
+            k = 0.05 * k + (jumps[None, :, None, None] / np.sqrt(D) / max(float(qdir.mean()), 0.5)).astype(np.float32)
+        mask = None
+        if kind == 2 or case % 4 == 0:
+            mask = (rng.random((B, S)) > 0.15).astype(np.float32)
+            left, right = int(rng.integers(0, S // 2)), int(rng.integers(0, S // 3))
+            mask[0, :left] = 0
+            if right:
+                mask[1, S - right:] = 0
+            mask[:, S // 2] = 1            # at least one visible key per row (not causal-safe for early rows: see below)
+            if causal:
+                mask[:, 0] = 1             # every causal row sees key 0
+        q, k, v = (O.bf16_round(t) for t in (q, k, v))
+        o = backend.attention.flash_attention2(q, k, v, H, D, mask=mask, causal=causal, dtype="bf16")
+        assert np.isfinite(o).all(), (case, S, D, causal, kind)
+        ref = O.truth_attention(q, k, v, mask=mask, causal=causal)
+        err = O.max_rel(o, ref)
+        worst = max(worst, err)
+        assert err < TOL_BF16, (case, S, D, causal, kind, err)
+    assert worst < TOL_BF16
