@@ -653,7 +653,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
             constexpr int u = decltype(iu)::value;
             const int qi = qw0 + 32 * u + li;
 #pragma unroll
-            for (int t = 0; t < NKB; ++t)
+            for (int t = 0; t < NKB; ++t) {
 #pragma unroll
                 for (int qd = 0; qd < 4; ++qd) {
                     const int kl = 32 * t + 8 * qd + 4 * lg;
@@ -661,13 +661,21 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
                     if (HAS_MASK) mk = *(const __attribute__((address_space(3))) f32x4*)(Mb + kl);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        // (mask-1)*1e9 as the shader forms it, then into the base-2 domain
+                        // (mask-1)*1e9 as the shader forms it, then into the base-2 domain.  The bias has to be one float
+                        // that is then ADDED: contracted into a fused multiply-add, the unrounded product would meet the
+                        // rounded one inside a reference taken from masked keys, and keys masked alike would no longer
+                        // weigh alike (the mean over all keys that a fully masked row stands for).
+#pragma clang fp contract(off)
                         float sv = sacc[u][t][4 * qd + e];
-                        if (HAS_MASK) sv += ((mk[e] - 1.0f) * 1e9f) * 1.4426950408889634f;
+                        if (HAS_MASK) {
+                            const float bias = ((mk[e] - 1.0f) * 1e9f) * 1.4426950408889634f;
+                            sv = sv + bias;
+                        }
                         if ((diag && (k0 + kl + e > qi)) || (tail && (k0 + kl + e >= S))) sv = -__builtin_inff();
                         sacc[u][t][4 * qd + e] = sv;
                     }
                 }
+            }
         });
     };
     // ---- softmax reference.  The first tile sets the reference m_run to its row maxima.  Every later tile is computed
@@ -790,15 +798,43 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     };
     auto is_diag = [&](int kt) __attribute__((always_inline)) { return p.causal && (kt * KT + KT - 1 > qw0); };
     auto is_tail = [&](int kt) __attribute__((always_inline)) { return kt * KT + KT > S; };
-    auto relative_scores = [&](int kt, int ST) __attribute__((always_inline)) {
+    // What the key mask does to the tile in stage ST, as two wave-uniform answers (each lane looks at KT/64 keys):
+    //   biased  - some key's mask differs from 1, so the tile's scores need the bias (most tiles of a padded batch do not,
+    //             and run exactly as without a mask);
+    //   dark    - every key's mask is at most 0.5: a bias of -5e8 or lower on every score.  For a row whose reference
+    //             stands at an ordinary score level, every exponential of such a tile is exactly zero in float.
+    auto mask_look = [&](int ST, bool& biased, bool& dark) __attribute__((always_inline)) {
+        if constexpr (HAS_MASK) {
+            const __attribute__((address_space(3))) float* Mb = (const __attribute__((address_space(3))) float*)(ldsp + OFF_M + ST * 1024);
+            bool ne = false, lit = false;
+#pragma unroll
+            for (int i = 0; i < KT / 64; ++i) {
+                const float mk = Mb[lane + 64 * i];
+                ne = ne || mk != 1.0f;
+                lit = lit || !(mk <= 0.5f);
+            }
+            biased = __builtin_amdgcn_ballot_w64(ne) != 0;
+            dark = __builtin_amdgcn_ballot_w64(lit) == 0;
+        } else {
+            biased = false; dark = false;
+        }
+    };
+    // no row of this wave still has a reference from masked keys only (around -1.4e9; an ordinary one is a score)
+    auto references_lit = [&]() __attribute__((always_inline)) {
+        bool low = false;
+#pragma unroll
+        for (int u = 0; u < QT; ++u) low = low || !(m_run[u] > -1.0e8f);
+        return __builtin_amdgcn_ballot_w64(low) == 0;
+    };
+    auto relative_scores = [&](int kt, int ST, bool biased) __attribute__((always_inline)) {
         phase_S(ST, std::true_type{});
         const bool diag = is_diag(kt), tail = is_tail(kt);
-        if (HAS_MASK || diag || tail) mask_apply(kt, ST, diag, tail);
+        if (biased || diag || tail) mask_apply(kt, ST, diag, tail);
     };
-    auto absolute_scores = [&](int kt, int ST) __attribute__((always_inline)) {
+    auto absolute_scores = [&](int kt, int ST, bool biased) __attribute__((always_inline)) {
         phase_S(ST, std::false_type{});
         const bool diag = is_diag(kt), tail = is_tail(kt);
-        if (HAS_MASK || diag || tail) mask_apply(kt, ST, diag, tail);
+        if (biased || diag || tail) mask_apply(kt, ST, diag, tail);
     };
     auto next_stage = [&](int st) __attribute__((always_inline)) { return st + 1 == NSTG ? 0 : st + 1; };
 
@@ -806,7 +842,9 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
     // ---- tile 0 sets the softmax reference: absolute scores, exact row maxima (rounded to bf16)
     {
         enter_tile(0, 0);
-        absolute_scores(0, 0);
+        bool biased, dark;
+        mask_look(0, biased, dark);
+        absolute_scores(0, 0, biased);
         sfor<QT>([&](auto iu) __attribute__((always_inline)) {
             constexpr int u = decltype(iu)::value;
             m_run[u] = tile_max(iu);
@@ -861,7 +899,12 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
             enter_tile(kt, st);
             // a wave whose queries all precede the tile has nothing to add (causal): it only keeps the barriers
             if (p.causal && kt * KT > qw0 + QW - 1) continue;
-            relative_scores(kt, st);
+            bool biased, dark;
+            mask_look(st, biased, dark);
+            // nor has a tile whose keys are all masked out, once every row has seen a key that is not (the padding of a
+            // batch): its exponentials are exact zeros
+            if (HAS_MASK && dark && references_lit()) continue;
+            relative_scores(kt, st, biased);
             if (__builtin_expect(overshoot(), 0)) { over = 1; break; }
             phase_PV(st, std::true_type{});
         }
@@ -872,10 +915,10 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
         // by more than 2^LAZY.  The new reference comes from the tile's absolute scores (exact whatever the old reference
         // was: relative scores lose their low bits against a reference like the -1.4e9 of a fully masked tile).
         mfma_drain();
-        absolute_scores(kt, st);
+        absolute_scores(kt, st, HAS_MASK);
         sfor<QT>([&](auto iu) __attribute__((always_inline)) { mx_tile[decltype(iu)::value] = tile_max(iu); });
         raise();
-        relative_scores(kt, st);
+        relative_scores(kt, st, HAS_MASK);
         phase_PV(st, std::false_type{});
         ++kt; st = next_stage(st);
         hand_back();
