@@ -113,9 +113,10 @@ def test_fa2_mask_layouts(backend, dtype, S, D):
     np.testing.assert_allclose(o[3], np.broadcast_to(v[3, 137], o[3].shape), atol=1e-6 if dtype == "fp32" else 1e-2)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("S,D", [(512, 64), (512, 32), (700, 128), (1536, 64), (1536, 128)])
-def test_fa2_padded_batches(backend, S, D, causal):
+@pytest.mark.parametrize("S,D", [(512, 64), (512, 32), (700, 128), (1536, 64), (1536, 128), (330, 48), (330, 80)])
+def test_fa2_padded_batches(backend, S, D, causal, dtype):
     """Right-padded batches: most tiles carry no mask bias at all and whole tiles of padding follow the real keys
     (the bf16 kernel runs the former like unmasked tiles and passes over the latter once every row of a wave has a
     real key behind it).  Lengths on and around tile edges; padding written as 0, as 0.5 (still an exact zero weight)
@@ -126,20 +127,21 @@ def test_fa2_padded_batches(backend, S, D, causal):
     lens = [S, 1, 63, 64, 65, 200, S - 1, S // 2, 0]
     B, H = len(lens) + 2, 2
     rng = np.random.default_rng(S + 7 * D + causal)
-    q, k, v = qkv(rng, B, S, H, D, "bf16")
+    q, k, v = qkv(rng, B, S, H, D, dtype)
     mask = np.ones((B, S), np.float32)
     for i, n in enumerate(lens):
         mask[i, n:] = (0.0, 0.5, 0.75)[i % 3]
     mask[B - 2, :96] = 0; mask[B - 2, 300:] = 0
     mask[B - 1, 400:] = 0; mask[B - 1, 77] = np.float32(1.0) + np.float32(2.0 ** -23)
-    o = backend.attention.flash_attention2(q, k, v, H, D, mask=mask, causal=causal, dtype="bf16")
+    o = backend.attention.flash_attention2(q, k, v, H, D, mask=mask, causal=causal, dtype=dtype)
     assert np.isfinite(o).all()
     ref = O.truth_attention(q, k, v, mask=mask, causal=causal)
     for i in range(B):
-        assert O.max_rel(o[i], ref[i]) < TOL_BF16, (i, S, D, causal)
+        assert O.max_rel(o[i], ref[i]) < tol(dtype), (i, S, D, causal)
     if not causal:
-        np.testing.assert_allclose(o[1], np.broadcast_to(v[1, 0], o[1].shape), atol=1e-2)
-        np.testing.assert_allclose(o[8], np.broadcast_to(v[8].mean(0), o[8].shape), atol=1e-2)
+        atol = 1e-2 if dtype == "bf16" else 1e-5
+        np.testing.assert_allclose(o[1], np.broadcast_to(v[1, 0], o[1].shape), atol=atol)
+        np.testing.assert_allclose(o[8], np.broadcast_to(v[8].mean(0), o[8].shape), atol=atol)
 
 
 def test_fa2_randomized_configurations(backend):
