@@ -147,3 +147,54 @@ def test_config4_swiglu_mlp_shapes(backend):
     assert O.max_rel(Y[rows], O.truth_linear(Hq[rows], Wd)) < TOL_BF16
     Y2 = backend.fnn.linear(2 * Hq[:1024], Wd, dtype="bf16")
     np.testing.assert_array_equal(Y2, 2 * Y[:1024])
+
+
+def test_randomized_shapes_over_every_kernel_variant(backend):
+    """Seeded sweep over what selects a GEMM kernel and what its edges see: K a multiple of the 128-byte slab (the
+    direct-to-LDS kernels), of 16 bytes only (register-staged loads with a zero-filled K tail) or of neither (one thread
+    per output); few tiles (128x128) or at least 192 tiles of 256x256 (the persistent kernel, with tile counts that do not
+    divide by the 256 workgroups or the 8 XCD runs); ragged M and N; every epilogue, with and without bias; both
+    dtypes.  Each case against the float64 closed form."""
+    rng = np.random.default_rng(977)
+    epis = ["none", "gelu", "silu", "relu", "res", "gcu", "roswish"]
+    worst = {"fp32": 0.0, "bf16": 0.0}
+    for case in range(42):
+        dtype = "bf16" if case % 2 else "fp32"
+        slab = 64 if dtype == "bf16" else 32
+        chunk = 8 if dtype == "bf16" else 4
+        kkind = case % 3                       # 0: whole slabs, 1: 16-byte rows with a K tail, 2: unaligned rows
+        if kkind == 0:
+            K = slab * int(rng.integers(1, 9))
+        elif kkind == 1:
+            K = chunk * int(rng.integers(1, 60))
+            K += chunk if K % slab == 0 else 0
+        else:
+            K = int(rng.integers(1, 300)) | 1
+        if case % 7 in (0, 3):                # the persistent big-tile kernels: >= 192 tiles
+            M = int(rng.integers(3100, 4600)); N = int(rng.integers(3100, 4600))
+            while ((M + 255) // 256) * ((N + 255) // 256) < 192:
+                N += 256
+            if kkind == 2:
+                M //= 8                        # the one-thread-per-output kernel is slow: keep it small
+        else:
+            M = int(rng.integers(1, 900)); N = int(rng.integers(1, 900))
+        epi = epis[int(rng.integers(0, len(epis)))]
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        W = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+        b = rng.standard_normal(N).astype(np.float32) if rng.random() < 0.7 else None
+        x, W = prep(dtype, x, W)
+        if epi == "res":
+            r = prep(dtype, (2.0 * rng.standard_normal((M, N))).astype(np.float32))[0]
+            y = backend.fnn.fused_linear_residual(x, W, b, r, dtype=dtype)
+            ref = O.truth_linear(x, W, b) + r.astype(np.float64)
+        elif epi == "none":
+            y = backend.fnn.linear(x, W, b, dtype=dtype)
+            ref = O.truth_linear(x, W, b)
+        else:
+            y = getattr(backend.fnn, "fused_linear_" + epi)(x, W, b, dtype=dtype)
+            ref = O.truth_linear(x, W, b, epi)
+        assert y.shape == (M, N) and np.isfinite(y).all(), (case, dtype, M, K, N, epi)
+        err = O.max_rel(y, ref)
+        worst[dtype] = max(worst[dtype], err)
+        assert err < tol(dtype), (case, dtype, M, K, N, epi, b is not None, err)
+    assert worst["fp32"] < TOL_F32 and worst["bf16"] < TOL_BF16
