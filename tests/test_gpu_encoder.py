@@ -84,6 +84,30 @@ def test_bert_base_layer_bf16_full_width(backend):
     assert np.abs(h.mean(-1)).max() < 2e-2 and np.abs(h.var(-1) - 1).max() < 5e-2
 
 
+def test_bert_base_layers_bf16_padded_batch(backend):
+    """Two full-width layers on a right-padded batch (lengths from 40 to 512 of 512 positions, one row of padding
+    written as 0.5): in the attention kernel most key tiles then carry no mask bias and the all-padding tiles are
+    passed over; every position, padded ones included, against the float64 oracle with bf16 storage emulated, and
+    the mean pooling over the real positions."""
+    cfg = EncoderConfig(layers=2)
+    w = random_bert_weights(cfg, seed=20260135)
+    rng = rng_for(5)
+    B, S = 5, 512
+    ids = rng.integers(0, cfg.vocab, (B, S))
+    lens = np.array([512, 40, 200, 333, 64])
+    mask = (np.arange(S)[None] < lens[:, None]).astype(np.float32)
+    enc = BertEncoder(backend, cfg, w, dtype="bf16")
+    h = enc.forward(ids, mask, pool=False)
+    ref = truth_encoder(w, cfg, ids, mask, O.bf16_round)
+    for i in range(B):
+        assert O.max_rel(h[i], ref[i]) < TOL_BF16, i
+    pooled = enc.forward(ids, mask, pool=True)
+    assert O.max_rel(pooled, O.truth_mean_pool(h, mask)) < 1e-3
+    half = mask.copy(); half[2, lens[2]:] = 0.5
+    h2 = enc.forward(ids, half, pool=False)
+    np.testing.assert_array_equal(h2[2], h[2])
+
+
 def test_encoder_batch_independence_full_config(backend):
     # full BERT-base depth (12 layers) in bf16: sequences are independent, so a batch run equals per-sequence runs
     cfg = EncoderConfig()
