@@ -116,6 +116,12 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
     f_qkv = lambda: lib.grl_gemm_nt(c.ctx, code, code, M, 3 * d, d, x.ptr, s.w_qkv, s.b_qkv, qkv.ptr, 0)
     f_fa = lambda: lib.grl_fa2_fwd_strided(c.ctx, code, B, S, H, D, qkv.ptr, qkv.ptr + d * es, qkv.ptr + 2 * d * es,
                                            None, attn.ptr, 3 * d, 3 * d, 3 * d, d, scale, 0, 0, 1e4, 1.0)
+    # the same attention launch under a key mask of right-padded sequences (lengths uniform in [S/2, S])
+    lens = np.random.default_rng(11).integers(S // 2, S + 1, B)
+    mask_h = (np.arange(S)[None] < lens[:, None]).astype(np.float32)
+    mask_d, attn_m = c.upload(mask_h), c.alloc(M * d * es)
+    f_fam = lambda: lib.grl_fa2_fwd_strided(c.ctx, code, B, S, H, D, qkv.ptr, qkv.ptr + d * es, qkv.ptr + 2 * d * es,
+                                            mask_d.ptr, attn_m.ptr, 3 * d, 3 * d, 3 * d, d, scale, 0, 0, 1e4, 1.0)
     f_out = lambda: lib.grl_gemm_nt(c.ctx, code, code, M, d, d, attn.ptr, s.w_o, s.b_o, proj.ptr, 0)
     f_ln = lambda: lib.grl_layernorm(c.ctx, code, M, d, x.ptr, proj.ptr, s.ln1_g, s.ln1_b, cfg.eps, x1.ptr)
     f_ff1 = lambda: lib.grl_gemm_nt(c.ctx, code, code, M, ff, d, x1.ptr, s.w_ff1, s.b_ff1, ffb.ptr, 1)
@@ -129,6 +135,7 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
         ("gemm_ffn2", "gemm_nt", f_ff2, 2.0 * M * d * ff, (M * ff + d * ff + M * d) * es),
         ("gemm_ffn1_gelu", "gemm_nt_gelu", f_ff1, 2.0 * M * d * ff, (M * d + d * ff + M * ff) * es),
         ("fa2_fwd", "fa2", f_fa, 4.0 * B * H * S * S * D, 4 * M * d * es),
+        ("fa2_fwd_key_mask", "fa2", f_fam, 4.0 * B * H * S * S * D, 4 * M * d * es),     # nominal FLOPs: padding counted
         ("layernorm_residual", "ln", f_ln, 0.0, 3 * M * d * es),
     ]
     out = {}
@@ -171,6 +178,9 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
         at = download_rows(c, attn, b0 * S, S, d, code).reshape(1, S, H, D)
         hs = [0, H - 1]
         errs["fa2_fwd"] = max_rel(at[:, :, hs], O.truth_attention(q3[:, :, 0][:, :, hs], q3[:, :, 1][:, :, hs], q3[:, :, 2][:, :, hs]))
+        atm = download_rows(c, attn_m, b0 * S, S, d, code).reshape(1, S, H, D)
+        errs["fa2_fwd_key_mask"] = max_rel(atm[:, :, hs], O.truth_attention(q3[:, :, 0][:, :, hs], q3[:, :, 1][:, :, hs], q3[:, :, 2][:, :, hs],
+                                                                            mask=mask_h[b0:b0 + 1]))
         errs["layernorm_residual"] = max_rel(gather_rows(c, x1, rows, d, code),
                                             O.truth_layernorm(gather_rows(c, x, rows, d, code), dl(s.ln1_g, d), dl(s.ln1_b, d), cfg.eps,
                                                               residual=gather_rows(c, proj, rows, d, code)))
@@ -178,7 +188,7 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
             if k in out:
                 out[k]["max_rel_vs_float64"] = float(f"{e:.3g}")
                 out[k]["within_tolerance"] = bool(e < TOL[dt])
-    for b in (qkv, attn, ffb, proj, x1, y2):
+    for b in (qkv, attn, ffb, proj, x1, y2, mask_d, attn_m):
         b.free()
     return out
 
