@@ -183,3 +183,46 @@ def test_fa2_randomized_configurations(backend):
         worst = max(worst, err)
         assert err < TOL_BF16, (case, S, D, causal, kind, err)
     assert worst < TOL_BF16
+
+
+def test_fa2_randomized_api_surface(backend):
+    """Seeded sweep over the whole flash_attention2 / flash_attention2_rope surface: both dtypes; head dims the MFMA
+    kernels take directly (32, 64, 128), head dims that run on zero-padded copies (8 ... 120) and head dims above 128
+    (one wave per query); both RoPE pairings with bases and scalings other than the default; right and left padding
+    and random holes in the key mask; causal; sequence lengths from one key to a few tiles.  Every case against the
+    float64 closed form (bf16 cases on bf16-rounded inputs)."""
+    rng = np.random.default_rng(424242)
+    worst = {"fp32": 0.0, "bf16": 0.0}
+    dims = [8, 24, 32, 40, 64, 80, 96, 120, 128, 160, 256]
+    for case in range(48):
+        dtype = "bf16" if case % 2 else "fp32"
+        D = int(dims[int(rng.integers(0, len(dims)))])
+        S = int(rng.choice([1, 2, 31, 64, 65, 130, 257, 400, 700]))
+        if D > 128:
+            S = min(S, 257)
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        causal = bool(rng.integers(0, 2))
+        style = [None, "interleaved", "half"][case % 3] if D <= 128 else None      # the fused rotation stops at head dim 128
+        base = float(rng.choice([10000.0, 500.0, 160000.0]))
+        scaling = float(rng.choice([1.0, 0.5, 4.0]))
+        q, k, v = qkv(rng, B, S, H, D, dtype)
+        mask = None
+        if case % 4 in (1, 2):
+            mask = (rng.random((B, S)) > 0.2).astype(np.float32)
+            if case % 4 == 2:
+                n = int(rng.integers(0, S + 1))
+                mask[0, n:] = 0                      # right padding (possibly the whole sequence)
+                mask[B - 1, : S // 3] = 0            # left padding
+            mask[:, 0] = 1                           # (every causal row keeps a key: masked-only rows weigh by rounding)
+        if style is None:
+            o = backend.attention.flash_attention2(q, k, v, H, D, mask=mask, causal=causal, dtype=dtype)
+            ref = O.truth_attention(q, k, v, mask=mask, causal=causal)
+        else:
+            o = backend.attention.flash_attention2_rope(q, k, v, H, D, mask=mask, causal=causal, rope_base=base,
+                                                        rope_scaling=scaling, rope_style=style, dtype=dtype)
+            ref = O.truth_attention(q, k, v, mask=mask, causal=causal, rope=style, base=base, scaling=scaling)
+        assert o.shape == (B, S, H, D) and np.isfinite(o).all(), (case, dtype, S, D, style, causal)
+        err = O.max_rel(o, ref)
+        worst[dtype] = max(worst[dtype], err)
+        assert err < tol(dtype), (case, dtype, B, S, H, D, style, base, scaling, causal, mask is not None, err)
+    assert worst["fp32"] < TOL_F32 and worst["bf16"] < TOL_BF16
