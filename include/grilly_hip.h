@@ -180,7 +180,9 @@ int grl_swiglu_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t 
 /* ---- attention -------------------------------------------------------------------
  * O[b,i,h,:] = sum_j softmax_j( scale*<Q'[b,i,h],K'[b,j,h]> + (mask[b,j]-1)*1e9 ) V[b,j,h,:]
  * with Q',K' optionally rotated (RoPE) and, if causal, keys j>i excluded.
- * Layout of Q,K,V,O: (B,S,H,D).  mask: fp32 (B,S), 1 keep / 0 drop, or NULL.
+ * Layout of Q,K,V,O: (B,S,H,D).  mask: fp32 (B,S), 1 keep / 0 drop, or NULL; any other value enters through the
+ * same bias (0.5 still drops, 1+2^-23 adds 119 to the key's scores), and a row whose visible keys are all dropped
+ * comes out as the mean of those keys' values (every score is rounded to the same -1e9, as in the shader).
  * Replaces VulkanAttention.flash_attention2 (backend/attention.py:361-597; contract in
  * its docstring :374-395; constants of shaders/flash-attention2.glsl:95,152,214) and
  * shaders/flash-attention2-rope.glsl:73-148 (interleaved pairs, theta =
