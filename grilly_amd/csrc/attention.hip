@@ -919,6 +919,18 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa2_bf16_kernel(Fa16Args p) {
         sfor<QT>([&](auto iu) __attribute__((always_inline)) { mx_tile[decltype(iu)::value] = tile_max(iu); });
         raise();
         relative_scores(kt, st, HAS_MASK);
+        // Against the reference just set no score exceeds 2^LAZY - in exact arithmetic.  A reference taken from masked keys
+        // (-1.4e9: a row that has seen padding only so far) leaves scores a granularity of 128, and the matrix core, which
+        // rounds after every k-slab, can land one step above what the single rounded sum of the absolute pass promised:
+        // 2^128 overflows, and the infinity would outlive the rescale by zero that real keys bring later.  Holding the
+        // scores at LAZY keeps every weight finite; rows with an ordinary reference are not touched by it.
+        sfor<QT>([&](auto iu) __attribute__((always_inline)) {
+            constexpr int u = decltype(iu)::value;
+#pragma unroll
+            for (int t = 0; t < NKB; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[u][t][r] = __builtin_fminf(sacc[u][t][r], LAZY);
+        });
         phase_PV(st, std::false_type{});
         ++kt; st = next_stage(st);
         hand_back();

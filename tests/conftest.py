@@ -34,5 +34,11 @@ def backend():
     b.cleanup()
 
 
+def sweep_rounds():
+    """How many times the seeded randomized sweeps repeat with fresh seeds (GRILLY_SWEEP_ROUNDS, default 1: the round
+    with the fixed seed that every run shares; more rounds are for longer parity runs on a GPU box)."""
+    return max(1, int(os.environ.get("GRILLY_SWEEP_ROUNDS", "1")))
+
+
 def rng_for(cfg):
     return np.random.default_rng(20260131 + cfg)

@@ -9,7 +9,7 @@ Tolerances: max|y-ref|/max|ref| <= 1e-4 (fp32), <= 2e-2 (bf16)."""
 import numpy as np
 import pytest
 
-from conftest import TOL_F32, TOL_BF16, rng_for
+from conftest import TOL_F32, TOL_BF16, rng_for, sweep_rounds
 from oracle import oracle_np as O
 
 pytestmark = pytest.mark.gpu
@@ -158,7 +158,7 @@ def test_randomized_shapes_over_every_kernel_variant(backend):
     rng = np.random.default_rng(977)
     epis = ["none", "gelu", "silu", "relu", "res", "gcu", "roswish"]
     worst = {"fp32": 0.0, "bf16": 0.0}
-    for case in range(42):
+    for case in range(42 * sweep_rounds()):
         dtype = "bf16" if case % 2 else "fp32"
         slab = 64 if dtype == "bf16" else 32
         chunk = 8 if dtype == "bf16" else 4
