@@ -173,6 +173,8 @@ def test_fa2_randomized_configurations(backend):
     rng = np.random.default_rng(20240611)
     worst = 0.0
     for case in range(36 * sweep_rounds()):
+        if case and case % 50 == 0:
+            print("sweep case", case, flush=True)      # long runs (pytest -s) show that they are alive
         D = int(rng.choice([32, 64, 128]))
         S = int(rng.choice([65, 128, 191, 256, 448, 512, 777, 1024, 1100, 1536]))
         B, H = 2, int(rng.choice([1, 3]))
@@ -216,6 +218,8 @@ def test_fa2_randomized_api_surface(backend):
     worst = {"fp32": 0.0, "bf16": 0.0}
     dims = [8, 24, 32, 40, 64, 80, 96, 120, 128, 160, 256]
     for case in range(48 * sweep_rounds()):
+        if case and case % 50 == 0:
+            print("sweep case", case, flush=True)      # long runs (pytest -s) show that they are alive
         dtype = "bf16" if case % 2 else "fp32"
         D = int(dims[int(rng.integers(0, len(dims)))])
         S = int(rng.choice([1, 2, 31, 64, 65, 130, 257, 400, 700]))

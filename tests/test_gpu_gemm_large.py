@@ -159,6 +159,8 @@ def test_randomized_shapes_over_every_kernel_variant(backend):
     epis = ["none", "gelu", "silu", "relu", "res", "gcu", "roswish"]
     worst = {"fp32": 0.0, "bf16": 0.0}
     for case in range(42 * sweep_rounds()):
+        if case and case % 50 == 0:
+            print("sweep case", case, flush=True)      # long runs (pytest -s) show that they are alive
         dtype = "bf16" if case % 2 else "fp32"
         slab = 64 if dtype == "bf16" else 32
         chunk = 8 if dtype == "bf16" else 4
