@@ -147,3 +147,41 @@ def test_bench_shape_forward_b128(backend):
         ref = truth_encoder(w1, cfg1, ids[b:b + 1], None, O.bf16_round)
         assert O.max_rel(h1[b:b + 1], ref) < TOL_BF16, b
     enc1.release_activations()
+
+
+def test_encoder_randomized_configurations(backend):
+    """Seeded sweep over small post-LN encoders: width, head count and head dim (32, 64, 128 run the MFMA attention kernels
+    on the packed QKV buffer, 16, 48 and 96 the zero-padded route), FFN width, depth, batch, sequence length, right and left
+    padding, both dtypes; every position against the float64 oracle (bf16 storage emulated)."""
+    from conftest import sweep_rounds
+    rng = np.random.default_rng(55001)
+    for case in range(10 * sweep_rounds()):
+        dtype = "bf16" if case % 2 else "fp32"
+        D = int(rng.choice([16, 32, 48, 64, 96, 128]))
+        heads = int(rng.choice([1, 2, 4, 6]))
+        d = D * heads
+        S = int(rng.choice([3, 17, 64, 100, 257, 384]))
+        B = int(rng.integers(1, 4))
+        cfg = EncoderConfig(layers=int(rng.integers(1, 3)), d_model=d, heads=heads, d_ff=int(rng.choice([2, 3, 4])) * d,
+                            vocab=211, max_pos=400)
+        w = random_bert_weights(cfg, seed=1000 + case, std=0.08)
+        for lw in w["layers"]:
+            for k in ("b_qkv", "b_o", "b_ff1", "b_ff2", "ln1_b", "ln2_b"):
+                lw[k] = (rng.standard_normal(lw[k].shape) * 0.05).astype(np.float32)
+            for k in ("ln1_g", "ln2_g"):
+                lw[k] = (1 + rng.standard_normal(lw[k].shape) * 0.05).astype(np.float32)
+        ids = rng.integers(0, cfg.vocab, (B, S))
+        mask = None
+        if case % 3:
+            lens = rng.integers(1, S + 1, B)
+            mask = (np.arange(S)[None] < lens[:, None]).astype(np.float32)
+            if case % 3 == 2:
+                mask[0] = mask[0, ::-1]                    # left padding
+        enc = BertEncoder(backend, cfg, w, dtype=dtype)
+        h = enc.forward(ids, mask, pool=False)
+        ref = truth_encoder(w, cfg, ids, mask, O.bf16_round if dtype == "bf16" else None)
+        assert np.isfinite(h).all(), (case, dtype, d, heads, S, B)
+        err = O.max_rel(h, ref)
+        assert err < (TOL_F32 if dtype == "fp32" else TOL_BF16), (case, dtype, d, heads, cfg.d_ff, cfg.layers, S, B, mask is not None, err)
+        if case and case % 10 == 0:
+            print("sweep case", case, flush=True)
