@@ -206,3 +206,65 @@ def test_gelu_epilogue_at_infinity_and_geglu_beyond_the_clip(backend):
     xg = np.zeros((2, 8), np.float32); xg[:, 0] = [60.0, 2.0]
     out = backend.fnn.fused_geglu(xg, W, W)[:, 0]            # gate * gelu(up), both 60 / 2
     np.testing.assert_allclose(out, [60.0 * 60.0, 2.0 * O.truth_gelu(np.array([2.0]))[0]], rtol=1e-5)
+
+
+def test_rowwise_randomized_shapes(backend):
+    """Seeded sweep over the row-wise kernels at random shapes (row widths from 1 to a few thousand, multiples of the
+    16-byte vector and not, single rows and thousands): LayerNorm with random gamma / beta / eps and rows far from zero,
+    softmax along the last axis with large spreads, rotate-half and interleaved RoPE with random position ids, GELU /
+    SiLU / SwiGLU activations, and the three gated dual GEMMs; both dtypes, each against the float64 closed form."""
+    from conftest import sweep_rounds
+    rng = np.random.default_rng(55003)
+    for case in range(40 * sweep_rounds()):
+        dtype = "bf16" if case % 2 else "fp32"
+        t = TOL_F32 if dtype == "fp32" else TOL_BF16
+        q = (lambda a: O.bf16_round(a)) if dtype == "bf16" else (lambda a: a)
+        what = case % 5
+        rows = int(rng.choice([1, 2, 7, 65, 300, 3001]))
+        F = int(rng.choice([1, 3, 8, 31, 64, 200, 384, 768, 1000, 1024, 2050, 4104]))
+        if what == 0:
+            # rows up to 20 standard deviations away from zero; narrow rows stay near it (among thousands of 3-element
+            # rows some have a spread a hundred times below the scale, and offset / spread times the float ulp is the
+            # conditioning of the fp32 normalisation itself, shader and kernel alike)
+            off = rng.uniform(-20, 20) if F >= 8 else rng.uniform(-1, 1)
+            x = q(((rng.standard_normal((rows, F)) + off) * rng.uniform(0.1, 5)).astype(np.float32))
+            g = rng.standard_normal(F).astype(np.float32); b = rng.standard_normal(F).astype(np.float32)
+            eps = float(rng.choice([1e-12, 1e-5, 1e-2]))
+            if F == 1:
+                continue                                   # a one-element row normalises to beta whatever the kernel does
+            # (bf16 rows far from zero keep few bits of their deviations: the oracle sees the same rounded inputs)
+            err = O.max_rel(backend.fnn.layernorm(x, g, b, eps=eps, dtype=dtype), O.truth_layernorm(x, g, b, eps))
+        elif what == 1:
+            x = q((rng.standard_normal((rows, F)) * rng.uniform(0.5, 30)).astype(np.float32))
+            x64 = x.astype(np.float64)
+            e = np.exp(x64 - x64.max(-1, keepdims=True))
+            err = O.max_rel(backend.fnn.activation_softmax(x, dtype=dtype), e / e.sum(-1, keepdims=True))
+        elif what == 2:
+            B, S, H = int(rng.integers(1, 3)), int(rng.choice([1, 5, 130])), int(rng.integers(1, 4))
+            D = int(rng.choice([2, 8, 32, 64, 96, 128]))
+            style = "half" if case % 10 < 5 else "interleaved"
+            x = q(rng.standard_normal((B, S, H, D)).astype(np.float32))
+            pid = rng.integers(0, 4000, (B, S)) if rng.random() < 0.5 else None
+            base, scaling = float(rng.choice([10000.0, 500.0])), float(rng.choice([1.0, 0.25, 8.0]))
+            y = backend.attention.apply_rope(x, position_ids=pid, rope_base=base, rope_scaling=scaling, rope_style=style, dtype=dtype)
+            err = O.max_rel(y, O.truth_rope(x, base, scaling, style, pid))
+        elif what == 3:
+            x = q((rng.standard_normal((rows, F)) * 3).astype(np.float32))
+            err = max(O.max_rel(backend.fnn.activation_gelu(x, dtype=dtype), O.truth_gelu(x)),
+                      O.max_rel(backend.fnn.activation_silu(x, dtype=dtype), O.truth_silu(x)))
+            if F % 2 == 0:
+                err = max(err, O.max_rel(backend.fnn.activation_swiglu(x, dtype=dtype), O.truth_swiglu_act(x)))
+        else:
+            M, K, N = min(rows, 400), 8 * int(rng.integers(1, 40)), int(rng.integers(1, 300))
+            x = q(rng.standard_normal((M, K)).astype(np.float32))
+            Wg = q((rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32))
+            Wu = q((rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32))
+            bias = rng.random() < 0.5
+            bg = rng.standard_normal(N).astype(np.float32) if bias else None
+            bu = rng.standard_normal(N).astype(np.float32) if bias else None
+            act = ["silu", "relu", "gelu"][int(rng.integers(0, 3))]
+            fn = {"silu": backend.fnn.fused_swiglu, "relu": backend.fnn.fused_reglu, "gelu": backend.fnn.fused_geglu}[act]
+            err = O.max_rel(fn(x, Wg, Wu, bg, bu, dtype=dtype), O.truth_fused_glu(x, Wg, Wu, bg, bu, act)[0])
+        assert err < t, (case, dtype, what, rows, F, err)
+        if case and case % 50 == 0:
+            print("sweep case", case, flush=True)
