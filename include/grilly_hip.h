@@ -202,7 +202,9 @@ int grl_fa2_fwd(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_
 /* Same as grl_fa2_fwd with explicit position strides (elements between consecutive sequence
  * positions of one batch entry), so Q, K and V can be the three column blocks of the packed
  * (B*S, 3*H*D) output of the fused QKV projection (shaders/fused-qkv-projection.glsl:58-70)
- * without a split copy.  Rotate-half RoPE is not offered here. */
+ * without a split copy.  Both RoPE pairings are offered; rotate-half takes its workspace (fp32: rotated copies of Q and
+ * K, bf16: the rotated K) from the pool.  Strides of at least H*D elements; operands that are not 16-byte granular
+ * (base addresses or strides) run on dense copies from the pool. */
 int grl_fa2_fwd_strided(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
                         const void* Q, const void* K, const void* V, const float* mask, void* O,
                         int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,

@@ -223,3 +223,75 @@ def test_rope_table_is_reused_across_calls(backend):
         assert O.max_rel(o, O.truth_attention(q, k, v, causal=True, rope="interleaved")) < TOL_BF16
     o2 = backend.attention.flash_attention2_rope(q, k, v, 2, 64, causal=True, rope_base=500.0, dtype="bf16")
     assert O.max_rel(o2, O.truth_attention(q, k, v, causal=True, rope="interleaved", base=500.0)) < TOL_BF16
+
+
+def test_fa2_strided_randomized(backend):
+    """Seeded sweep of grl_fa2_fwd_strided through the C ABI: Q, K and V as column blocks of one packed buffer or in
+    buffers of their own, position strides from exactly H*D upwards, block offsets and strides that are 16-byte granular
+    (the kernels read the operands in place) or not (dense copies from the pool), the output written into a strided buffer
+    whose other columns must stay untouched; both dtypes, key mask, causal, both RoPE pairings."""
+    from conftest import sweep_rounds
+    from grilly_amd import _lib as L
+    c = backend.core
+    rng = np.random.default_rng(55004)
+    for case in range(24 * sweep_rounds()):
+        dtype = "bf16" if case % 2 else "fp32"
+        code, es = (L.GRL_BF16, 2) if dtype == "bf16" else (L.GRL_F32, 4)
+        D = int(rng.choice([32, 64, 128, 40]))
+        H = int(rng.integers(1, 4))
+        S = int(rng.choice([1, 19, 64, 130, 300]))
+        B = int(rng.integers(1, 3))
+        hd = H * D
+        gran = 16 // es                                    # elements per 16 bytes
+        granular = case % 4 != 3
+        pad = lambda: int(rng.integers(0, 4)) * gran + (0 if granular else int(rng.integers(1, gran)))
+        packed = bool(rng.integers(0, 2))
+        q, k, v = qkv(rng, B, S, H, D, dtype)
+        flat = lambda a: a.reshape(B, S, hd)
+        bufs = []
+        if packed:
+            offs = [pad(), 0, 0]
+            offs[1] = offs[0] + hd + pad(); offs[2] = offs[1] + hd + pad()
+            stride = offs[2] + hd + pad()
+            host = rng.standard_normal((B, S, stride)).astype(np.float32)
+            for a, o in zip((q, k, v), offs):
+                host[:, :, o:o + hd] = flat(a)
+            dev = c.upload(host, code); bufs.append(dev)
+            ptrs = [dev.ptr + o * es for o in offs]; strides = [stride] * 3
+        else:
+            ptrs, strides = [], []
+            for a in (q, k, v):
+                o = pad(); stride = o + hd + pad()
+                host = rng.standard_normal((B, S, stride)).astype(np.float32)
+                host[:, :, o:o + hd] = flat(a)
+                dev = c.upload(host, code); bufs.append(dev)
+                ptrs.append(dev.ptr + o * es); strides.append(stride)
+        oo = pad(); ostride = oo + hd + pad()
+        sentinel = np.full((B, S, ostride), 7.0, np.float32)
+        dout = c.upload(sentinel, code); bufs.append(dout)
+        mask = None
+        if case % 3 == 1:
+            mask = (rng.random((B, S)) > 0.2).astype(np.float32); mask[:, 0] = 1
+        dmask = c.upload(mask) if mask is not None else None
+        causal = bool(rng.integers(0, 2))
+        style = [None, "interleaved", "half"][int(rng.integers(0, 3))]
+        rope = {None: L.ROPE_NONE, "interleaved": L.ROPE_INTERLEAVED, "half": L.ROPE_HALF}[style]
+        base, scaling = float(rng.choice([10000.0, 500.0])), float(rng.choice([1.0, 2.0]))
+        scale = 1.0 / np.sqrt(D)
+        try:
+            L.check(c.lib.grl_fa2_fwd_strided(c.ctx, code, B, S, H, D, ptrs[0], ptrs[1], ptrs[2], dmask.ptr if dmask else None,
+                                              dout.ptr + oo * es, strides[0], strides[1], strides[2], ostride, scale, int(causal),
+                                              rope, base, scaling), "fa2_fwd_strided")
+            got = c.download(dout, (B, S, ostride), code)
+        finally:
+            for b in bufs + ([dmask] if dmask else []):
+                b.free()
+        ref = O.truth_attention(q, k, v, mask=mask, causal=causal, rope=style, base=base, scaling=scaling)
+        info = (case, dtype, B, S, H, D, packed, granular, strides, ostride, style, causal, mask is not None)
+        o = got[:, :, oo:oo + hd].reshape(B, S, H, D)
+        assert np.isfinite(o).all(), info
+        assert O.max_rel(o, ref) < tol(dtype), info + (O.max_rel(o, ref),)
+        rest = np.delete(got, np.s_[oo:oo + hd], axis=2)
+        assert (rest == 7.0).all(), info
+        if case and case % 50 == 0:
+            print("sweep case", case, flush=True)
