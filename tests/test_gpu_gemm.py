@@ -308,3 +308,55 @@ def test_linear_residual_shapes_and_errors(backend):
     np.testing.assert_allclose(c.download(dr, (M, N)), res + b, rtol=1e-6, atol=1e-6)
     assert c.lib.grl_gemm_nt_res(c.ctx, L.GRL_F32, L.GRL_F32, M, N, 0, None, None, db.ptr, None, dr.ptr) != 0
     db.free(); dr.free()
+
+
+def test_gemm_nt_c_abi_randomized(backend):
+    """Seeded sweep of grl_gemm_nt / grl_gemm_nt_act through ctypes: all four (input, output) storage-type pairs, every
+    epilogue code, bias or NULL, ragged shapes on both sides of the kernel-selection thresholds, and an output that sits
+    inside a larger buffer at an aligned or an odd element offset (odd: the one-thread-per-output kernel) whose
+    surroundings must keep a sentinel: a tile-edge store that leaves the matrix shows up there."""
+    from conftest import sweep_rounds
+    c = backend.core
+    rng = np.random.default_rng(55005)
+    epis = [(L.EPI_NONE, "none"), (L.EPI_GELU, "gelu"), (L.EPI_SILU, "silu"), (L.EPI_RELU, "relu"), (L.EPI_GCU, "gcu"), (L.EPI_ROSWISH, "roswish")]
+    for case in range(32 * sweep_rounds()):
+        cin, cout = [(L.GRL_F32, L.GRL_F32), (L.GRL_BF16, L.GRL_BF16), (L.GRL_BF16, L.GRL_F32), (L.GRL_F32, L.GRL_BF16)][case % 4]
+        es_out = 2 if cout == L.GRL_BF16 else 4
+        K = int(rng.choice([8, 24, 64, 72, 128, 200, 512]))
+        if case % 8 == 7:                                      # >= 192 tiles of 256x256
+            M, N = int(rng.integers(3300, 3700)), int(rng.integers(3600, 4000))
+        else:
+            M, N = int(rng.integers(1, 700)), int(rng.integers(1, 700))
+        code, name = epis[int(rng.integers(0, len(epis)))]
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        W = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+        b = rng.standard_normal(N).astype(np.float32) if rng.random() < 0.6 else None
+        if cin == L.GRL_BF16:
+            x, W = O.bf16_round(x), O.bf16_round(W)
+        lead = int(rng.choice([0, 32, 1, 3]))                  # elements in front of the output inside its buffer
+        tail = 64
+        host_out = np.full(lead + M * N + tail, 7.0, np.float32)
+        dx, dw, dout = c.upload(x, cin), c.upload(W, cin), c.upload(host_out, cout)
+        db = c.upload(b) if b is not None else None
+        try:
+            cptr = dout.ptr + lead * es_out
+            bptr = db.ptr if db else None
+            if code <= L.EPI_SILU:
+                rc = c.lib.grl_gemm_nt(c.ctx, cin, cout, M, N, K, dx.ptr, dw.ptr, bptr, cptr, code)
+            else:
+                rc = c.lib.grl_gemm_nt_act(c.ctx, cin, cout, M, N, K, dx.ptr, dw.ptr, bptr, cptr, code, 0.7, 1.3)
+            L.check(rc, "gemm_nt")
+            got = c.download(dout, (lead + M * N + tail,), cout)
+        finally:
+            for t in (dx, dw, dout, db):
+                if t is not None:
+                    t.free()
+        ref = O.truth_linear(x, W, b, name, 0.7, 1.3)
+        info = (case, cin, cout, M, N, K, name, b is not None, lead)
+        y = got[lead:lead + M * N].reshape(M, N)
+        t = TOL_F32 if (cin == L.GRL_F32 and cout == L.GRL_F32) else TOL_BF16
+        assert np.isfinite(y).all(), info
+        assert O.max_rel(y, ref) < t, info + (O.max_rel(y, ref),)
+        assert (got[:lead] == 7.0).all() and (got[lead + M * N:] == 7.0).all(), info
+        if case and case % 50 == 0:
+            print("sweep case", case, flush=True)
