@@ -183,5 +183,7 @@ def test_encoder_randomized_configurations(backend):
         assert np.isfinite(h).all(), (case, dtype, d, heads, S, B)
         err = O.max_rel(h, ref)
         assert err < (TOL_F32 if dtype == "fp32" else TOL_BF16), (case, dtype, d, heads, cfg.d_ff, cfg.layers, S, B, mask is not None, err)
+        pooled = enc.forward(ids, mask, pool=True)             # masked mean over the positions + L2 normalisation
+        assert O.max_rel(pooled, O.truth_mean_pool(h, mask)) < 1e-3, (case, dtype, d, S, B)
         if case and case % 10 == 0:
             print("sweep case", case, flush=True)
