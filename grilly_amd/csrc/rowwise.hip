@@ -799,13 +799,14 @@ extern "C" int grl_embed(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F,
 }
 
 // ------------------------------------------------------------------ masked mean pool (+ L2 normalise)
-// grid (ceil(F/256), B).  F % 4 == 0: a lane owns 4 adjacent features (8- or 16-byte loads), the 4 waves
-// of a workgroup take every 4th position of the sequence and their partial sums meet in LDS.
-template <typename T>
-__global__ __launch_bounds__(256) void mean_pool_kernel(const T* __restrict__ x, const float* __restrict__ mask,
-                                                       float* __restrict__ out, int S, int F) {
-    __shared__ float part[4][256];
-    __shared__ float cpart[4];
+// grid (ceil(F/256), B).  F % 4 == 0: a lane owns 4 adjacent features (8- or 16-byte loads), the NW waves
+// of a workgroup take every NW-th position of the sequence and their partial sums meet in LDS (sixteen waves: a
+// batch of 128 sequences is only a few hundred workgroups, and the loads in flight per CU are what the rate hangs on).
+template <typename T, int NW>
+__global__ __launch_bounds__(NW * 64) void mean_pool_kernel(const T* __restrict__ x, const float* __restrict__ mask,
+                                                           float* __restrict__ out, int S, int F) {
+    __shared__ float part[NW][256];
+    __shared__ float cpart[NW];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int f0 = blockIdx.x * 256 + lane * 4;
     const int64_t b = blockIdx.y;
@@ -813,7 +814,7 @@ __global__ __launch_bounds__(256) void mean_pool_kernel(const T* __restrict__ x,
     const T* xb = x + b * S * (int64_t)F + f0;
     const bool live = f0 < F;
 #pragma unroll 8
-    for (int s = wave; s < S; s += 4) {
+    for (int s = wave; s < S; s += NW) {
         const float m = mask ? mask[b * S + s] : 1.0f;
         cnt += m;
         if (live) {
@@ -827,9 +828,10 @@ __global__ __launch_bounds__(256) void mean_pool_kernel(const T* __restrict__ x,
     if (lane == 0) cpart[wave] = cnt;
     __syncthreads();
     const int f = blockIdx.x * 256 + threadIdx.x;
-    if (f < F) {
-        const float tot = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
-        const float c = (cpart[0] + cpart[1]) + (cpart[2] + cpart[3]);
+    if (threadIdx.x < 256 && f < F) {
+        float tot = 0.f, c = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) { tot += part[w][threadIdx.x]; c += cpart[w]; }
         out[b * F + f] = tot / fmaxf(c, 1e-9f);
     }
 }
@@ -868,13 +870,14 @@ extern "C" int grl_mean_pool(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_
     GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_mean_pool: bad dtype %d", dtype);
     GRL_REQUIRE(B >= 0 && B < 65536 && S > 0 && F > 0 && S < (1LL << 31) && F < (1LL << 31), GRL_ERR_SHAPE, "grl_mean_pool: bad shape");
     if (B == 0) return GRL_OK;
-    dim3 g((unsigned)((F + 255) / 256), (unsigned)B), b(256);
+    constexpr int PW = 16;                                  // waves per workgroup of the vector kernel
+    dim3 g((unsigned)((F + 255) / 256), (unsigned)B), b(256), bv(PW * 64);
     const bool vec = F % 4 == 0 && aligned16(x);
     if (dtype == GRL_F32) {
-        if (vec) hipLaunchKernelGGL(mean_pool_kernel<float>, g, b, 0, c->stream, (const float*)x, mask, out, (int)S, (int)F);
+        if (vec) hipLaunchKernelGGL((mean_pool_kernel<float, PW>), g, bv, 0, c->stream, (const float*)x, mask, out, (int)S, (int)F);
         else hipLaunchKernelGGL(mean_pool_generic_kernel<float>, g, b, 0, c->stream, (const float*)x, mask, out, (int)S, (int)F);
     } else {
-        if (vec) hipLaunchKernelGGL(mean_pool_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, mask, out, (int)S, (int)F);
+        if (vec) hipLaunchKernelGGL((mean_pool_kernel<uint16_t, PW>), g, bv, 0, c->stream, (const uint16_t*)x, mask, out, (int)S, (int)F);
         else hipLaunchKernelGGL(mean_pool_generic_kernel<uint16_t>, g, b, 0, c->stream, (const uint16_t*)x, mask, out, (int)S, (int)F);
     }
     GRL_CHECK_LAUNCH();
