@@ -783,6 +783,32 @@ __global__ __launch_bounds__(256) void embed_kernel(const int32_t* __restrict__ 
     }
 }
 
+// F % 4 == 0 and 16-byte aligned tables: a lane owns 4 adjacent features of its wave's row (16-byte table loads, one 8- or
+// 16-byte streaming store), eight rows per workgroup
+template <typename T>
+__global__ __launch_bounds__(512) void embed_vec_kernel(const int32_t* __restrict__ ids, const float* __restrict__ tok,
+                                                       const float* __restrict__ pos, const float* __restrict__ typ,
+                                                       T* __restrict__ x, int64_t rows, int S, int F, int vocab) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    int id = ids[row];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // the host validates; this only keeps loads in bounds
+    const float* t = tok + (int64_t)id * F;
+    const float* p = pos ? pos + (int64_t)(row % S) * F : nullptr;
+    T* o = x + row * (int64_t)F;
+    for (int f = lane * 4; f < F; f += 256) {
+        f32x4 v = *(const f32x4*)(t + f);
+        // the shader's order: token + type + position
+        if (typ) v += *(const f32x4*)(typ + f);
+        if (p) v += *(const f32x4*)(p + f);
+        vec4<T> out;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out.set(i, v[i]);
+        out.store_stream(o + f);
+    }
+}
+
 extern "C" int grl_embed(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F, int64_t vocab, const int32_t* ids,
                          const float* tok_emb, const float* pos_emb, const float* type_emb, void* x) {
     GRL_REQUIRE(c && ids && tok_emb && x, GRL_ERR_ARG, "grl_embed: null argument");
@@ -791,6 +817,13 @@ extern "C" int grl_embed(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F,
                 GRL_ERR_SHAPE, "grl_embed: bad shape");
     int64_t rows = B * S;
     if (rows == 0) return GRL_OK;
+    if (F % 4 == 0 && aligned16(tok_emb) && aligned16(x) && (!pos_emb || aligned16(pos_emb)) && (!type_emb || aligned16(type_emb))) {
+        dim3 g8((unsigned)((rows + 7) / 8)), b8(512);
+        if (dtype == GRL_F32) hipLaunchKernelGGL(embed_vec_kernel<float>, g8, b8, 0, c->stream, ids, tok_emb, pos_emb, type_emb, (float*)x, rows, (int)S, (int)F, (int)vocab);
+        else hipLaunchKernelGGL(embed_vec_kernel<uint16_t>, g8, b8, 0, c->stream, ids, tok_emb, pos_emb, type_emb, (uint16_t*)x, rows, (int)S, (int)F, (int)vocab);
+        GRL_CHECK_LAUNCH();
+        return GRL_OK;
+    }
     dim3 g((unsigned)((rows + 3) / 4)), b(256);
     if (dtype == GRL_F32) hipLaunchKernelGGL(embed_kernel<float>, g, b, 0, c->stream, ids, tok_emb, pos_emb, type_emb, (float*)x, rows, (int)S, (int)F, (int)vocab);
     else hipLaunchKernelGGL(embed_kernel<uint16_t>, g, b, 0, c->stream, ids, tok_emb, pos_emb, type_emb, (uint16_t*)x, rows, (int)S, (int)F, (int)vocab);
