@@ -223,6 +223,17 @@ __device__ __forceinline__ float silu_clamped(float x) {
 __device__ __forceinline__ float silu_plain(float x) {
     return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
 }
+__device__ __forceinline__ void silu_plain4(float (&v)[4]) {       // four values stage by stage, like gelu_fast4 below
+    float e[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = __builtin_amdgcn_exp2f(-1.4426950408889634f * v[i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = 1.0f + e[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = __builtin_amdgcn_rcpf(e[i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = v[i] * e[i];
+}
 // v_mul_legacy_f32 (0 times anything, infinities and NaN included, is 0); the intrinsic has no clang builtin
 extern "C" __device__ float fmul_legacy(float, float) __asm("llvm.amdgcn.fmul.legacy");
 // shaders/fused-linear-gelu.glsl:45-63 rewritten with tanh(u) = 2/(1+exp(-2u)) - 1:

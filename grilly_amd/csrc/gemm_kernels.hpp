@@ -81,6 +81,18 @@ __device__ __forceinline__ float glu_apply(float gate, float up, const GemmArgs&
     if (p.act == GRL_EPI_GELU) return gate * gelu_fast(up);
     return gate * silu_plain(up);
 }
+// the same for four adjacent outputs, the transcendental activations stage by stage (see gelu_fast4)
+__device__ __forceinline__ void glu_apply4(float (&gate)[4], float (&up)[4], const GemmArgs& p) {
+    if (p.act == GRL_EPI_RELU) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gate[e] *= fmaxf(up[e], 0.0f);
+        return;
+    }
+    if (p.act == GRL_EPI_GELU) gelu_fast4(up);
+    else silu_plain4(up);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) gate[e] *= up[e];
+}
 
 // ---- one 128-byte-per-row K slab on the matrix cores --------------------------------------
 template <typename T> struct MfmaSlab;
@@ -645,13 +657,14 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                             for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] * rs + (b1[e] - rsm * c1[e]);
                         }
                         if (DUAL) {
+                            float up[4];
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
-                                float up = acc[a][DUAL ? b + TNO : b][4 * q + e];
-                                if constexpr (LN) up = up * rs + (b2[e] - rsm * c2[e]);
-                                else up += bv2[LN ? 0 : b][q][e];
-                                v[e] = glu_apply(v[e], up, p);
+                                up[e] = acc[a][DUAL ? b + TNO : b][4 * q + e];
+                                if constexpr (LN) up[e] = up[e] * rs + (b2[e] - rsm * c2[e]);
+                                else up[e] += bv2[LN ? 0 : b][q][e];
                             }
+                            glu_apply4(v, up, p);
                         } else {
                             if constexpr (EPI == EPI_GELU) gelu_fast4(v);
                             else
