@@ -201,8 +201,7 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
                             }
                             if (p.cache1) store4<float>(p.cache1 + o, v[0], v[1], v[2], v[3]);
                             if (p.cache2) store4<float>(p.cache2 + o, u[0], u[1], u[2], u[3]);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = glu_apply(v[e], u[e], p);
+                            glu_apply4(v, u, p);
                         } else {
                             if constexpr (EPI == EPI_GELU) gelu_fast4(v);
                             else
