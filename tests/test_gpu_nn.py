@@ -104,3 +104,61 @@ def test_multihead_attention_weights_and_cross_length(backend, Sq, Sk):
     if Sq == Sk:
         out2, none = mha(q, kv, kv, mask, need_weights=False)
         assert none is None and O.max_rel(out2, ref) < TOL_F32
+
+
+def test_nn_modules_randomized(backend):
+    """Seeded sweep over the attention-bearing modules at random widths, head counts (head dims that run the MFMA
+    kernels directly and head dims that run on padded copies), sequence lengths (query and key lengths apart for
+    MultiheadAttention), FFN widths, activations and key masks, against the float64 composition of the pinned pieces."""
+    from conftest import sweep_rounds
+    rng = np.random.default_rng(55006)
+    for case in range(12 * sweep_rounds()):
+        np.random.seed(1000 + case)
+        H = int(rng.choice([1, 2, 3, 4]))
+        D = int(rng.choice([8, 24, 32, 64]))
+        d, B = H * D, int(rng.integers(1, 4))
+        if case % 2 == 0:
+            S, ff = int(rng.choice([1, 9, 50, 130])), 8 * int(rng.integers(1, 60))
+            act = ["gelu", "relu"][int(rng.integers(0, 2))]
+            layer = nn.TransformerEncoderLayer(d, H, dim_feedforward=ff, activation=act).to_backend(backend).eval()
+            for n, p in layer.named_parameters():
+                if n.startswith("norm"):
+                    p.data[...] = 1.0 + 0.1 * rng.standard_normal(p.shape) if n.endswith("weight") else 0.1 * rng.standard_normal(p.shape)
+                else:
+                    p.data[...] = rng.standard_normal(p.shape) * (0.08 if n.endswith("weight") else 0.05)
+            x = rng.standard_normal((B, S, d)).astype(np.float32)
+            mask = None
+            if rng.random() < 0.6:
+                mask = (np.arange(S)[None] < rng.integers(1, S + 1, B)[:, None]).astype(np.float32)
+            y = layer(x, mask)
+            P = {n: p.data.astype(np.float64) for n, p in layer.named_parameters()}
+            h = O.truth_layernorm(x, P["norm1.weight"], P["norm1.bias"])
+            proj = lambda t, n: t @ P[f"self_attn.{n}.weight"].T + P[f"self_attn.{n}.bias"]
+            sh = (B, S, H, D)
+            a = O.truth_attention(proj(h, "q_proj").reshape(sh), proj(h, "k_proj").reshape(sh), proj(h, "v_proj").reshape(sh), mask=mask)
+            x1 = x + proj(a.reshape(B, S, d), "out_proj")
+            h2 = O.truth_layernorm(x1, P["norm2.weight"], P["norm2.bias"])
+            f = h2 @ P["linear1.weight"].T + P["linear1.bias"]
+            f = O.truth_gelu(f) if act == "gelu" else np.maximum(f, 0)
+            ref = x1 + f @ P["linear2.weight"].T + P["linear2.bias"]
+            assert y.shape == (B, S, d)
+            assert O.max_rel(y, ref) < TOL_F32, (case, "layer", d, H, ff, act, B, S, mask is not None)
+        else:
+            Sq, Sk = int(rng.choice([1, 7, 40, 100])), int(rng.choice([1, 9, 45, 130]))
+            mha = nn.MultiheadAttention(d, H).to_backend(backend)
+            for n, p in mha.named_parameters():
+                p.data[...] = rng.standard_normal(p.shape) * (0.1 if n.endswith("weight") else 0.05)
+            q = rng.standard_normal((B, Sq, d)).astype(np.float32)
+            kv = rng.standard_normal((B, Sk, d)).astype(np.float32)
+            mask = (np.arange(Sk)[None] < rng.integers(1, Sk + 1, B)[:, None]).astype(np.float32)
+            out, w = mha(q, kv, kv, mask)
+            P = {n: p.data.astype(np.float64) for n, p in mha.named_parameters()}
+            proj = lambda t, n: t @ P[f"{n}.weight"].T + P[f"{n}.bias"]
+            qh = proj(q, "q_proj").reshape(B, Sq, H, D); kh = proj(kv, "k_proj").reshape(B, Sk, H, D); vh = proj(kv, "v_proj").reshape(B, Sk, H, D)
+            sc = np.einsum("bqhd,bkhd->bhqk", qh, kh) / np.sqrt(D) + ((mask.astype(np.float64) - 1) * 1e9)[:, None, None, :]
+            pw = np.exp(sc - sc.max(-1, keepdims=True)); pw /= pw.sum(-1, keepdims=True)
+            ref = proj(np.einsum("bhqk,bkhd->bqhd", pw, vh).reshape(B, Sq, d), "out_proj")
+            assert out.shape == (B, Sq, d) and w.shape == (B, H, Sq, Sk)
+            assert O.max_rel(w, pw) < TOL_F32 and O.max_rel(out, ref) < TOL_F32, (case, "mha", d, H, B, Sq, Sk)
+        if case and case % 20 == 0:
+            print("sweep case", case, flush=True)
