@@ -179,3 +179,101 @@ def test_ln_linear_argument_errors(backend):
     # empty problems are no-ops
     L.check(c.lib.grl_ln_gemm_nt(c.ctx, 0, 0, 0, 4, 8, None, None, None, None, 1e-5, None, None))
     L.check(c.lib.grl_ln_fold(c.ctx, 0, 0, 8, None, None, None, None, None, None, None))
+
+
+def test_gated_and_ln_folded_gemms_c_abi_randomized(backend):
+    """Seeded sweep through ctypes of grl_glu_nt (gate and up caches on and off), grl_gemm_nt_res, grl_ln_gemm_nt and
+    grl_ln_glu_nt: the four storage-type pairs where the entry point has them, the three gate activations, biases on and
+    off, ragged shapes on both sides of the 256x256-tile threshold, K a whole number of 128-byte slabs or not; outputs and
+    caches sit inside larger buffers whose surroundings must keep a sentinel."""
+    from conftest import sweep_rounds
+    c = backend.core
+    rng = np.random.default_rng(55007)
+    acts = [(L.EPI_SILU, "silu"), (L.EPI_RELU, "relu"), (L.EPI_GELU, "gelu")]
+    PAD = 48
+
+    def padded(n, code):
+        return c.upload(np.full(n + 2 * PAD, 7.0, np.float32), code)
+
+    def take(buf, n, code, info):
+        es = 2 if code == L.GRL_BF16 else 4
+        got = c.download(buf, (n + 2 * PAD,), code)
+        assert (got[:PAD] == 7.0).all() and (got[PAD + n:] == 7.0).all(), info
+        return got[PAD:PAD + n]
+
+    for case in range(24 * sweep_rounds()):
+        cin, cout = [(L.GRL_F32, L.GRL_F32), (L.GRL_BF16, L.GRL_BF16), (L.GRL_BF16, L.GRL_F32), (L.GRL_F32, L.GRL_BF16)][case % 4]
+        es_out = 2 if cout == L.GRL_BF16 else 4
+        q = (lambda a: O.bf16_round(a)) if cin == L.GRL_BF16 else (lambda a: a)
+        t = TOL_F32 if (cin == L.GRL_F32 and cout == L.GRL_F32) else TOL_BF16
+        K = int(rng.choice([16, 64, 96, 128, 264, 512]))
+        if case % 7 == 6:                                      # >= 192 tiles of 256x256 (256x128 output tiles for the dual forms)
+            M, N = int(rng.integers(3300, 3600)), int(rng.integers(1900, 2100))
+        else:
+            M, N = int(rng.integers(1, 500)), int(rng.integers(1, 400))
+        x = q((rng.standard_normal((M, K)) * 1.5 + 0.3).astype(np.float32))
+        W1 = q((rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32))
+        W2 = q((rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32))
+        bias = rng.random() < 0.6
+        b1 = rng.standard_normal(N).astype(np.float32) if bias else None
+        b2 = rng.standard_normal(N).astype(np.float32) if bias else None
+        code, name = acts[int(rng.integers(0, 3))]
+        what = case % 3
+        info = (case, what, cin, cout, M, N, K, name, bias)
+        dx, dw1, dw2 = c.upload(x, cin), c.upload(W1, cin), c.upload(W2, cin)
+        db1, db2 = (c.upload(b1), c.upload(b2)) if bias else (None, None)
+        dout = padded(M * N, cout)
+        held = [dx, dw1, dw2, dout] + ([db1, db2] if bias else [])
+        optr = dout.ptr + PAD * es_out
+        try:
+            if what == 0:                                      # gated GEMM, with or without the pre-activation caches
+                caches = rng.random() < 0.5
+                dg, du = (padded(M * N, L.GRL_F32), padded(M * N, L.GRL_F32)) if caches else (None, None)
+                held += [dg, du] if caches else []
+                L.check(c.lib.grl_glu_nt(c.ctx, cin, cout, M, N, K, dx.ptr, dw1.ptr, dw2.ptr, db1.ptr if bias else None, db2.ptr if bias else None,
+                                         optr, dg.ptr + PAD * 4 if caches else None, du.ptr + PAD * 4 if caches else None, code), "glu_nt")
+                ref, g, u = O.truth_fused_glu(x, W1, W2, b1, b2, name)
+                y = take(dout, M * N, cout, info).reshape(M, N)
+                assert O.max_rel(y, ref) < t, info + (O.max_rel(y, ref),)
+                if caches:
+                    tc = TOL_F32 if cin == L.GRL_F32 else TOL_BF16
+                    assert O.max_rel(take(dg, M * N, L.GRL_F32, info).reshape(M, N), g) < tc, info
+                    assert O.max_rel(take(du, M * N, L.GRL_F32, info).reshape(M, N), u) < tc, info
+            elif what == 1:                                    # GEMM + residual of the output type
+                r = (2.0 * rng.standard_normal((M, N))).astype(np.float32)
+                if cout == L.GRL_BF16:
+                    r = O.bf16_round(r)
+                dr = c.upload(r, cout); held.append(dr)
+                L.check(c.lib.grl_gemm_nt_res(c.ctx, cin, cout, M, N, K, dx.ptr, dw1.ptr, db1.ptr if bias else None, dr.ptr, optr), "gemm_nt_res")
+                y = take(dout, M * N, cout, info).reshape(M, N)
+                ref = O.truth_linear(x, W1, b1) + r.astype(np.float64)
+                assert O.max_rel(y, ref) < t, info + (O.max_rel(y, ref),)
+            else:                                              # LayerNorm folded into the GEMM / the gated GEMM
+                gamma = (1 + 0.2 * rng.standard_normal(K)).astype(np.float32); beta = (0.2 * rng.standard_normal(K)).astype(np.float32)
+                dgm, dbt = c.upload(gamma), c.upload(beta)
+                es_in = 2 if cin == L.GRL_BF16 else 4
+                ws1, ws2 = c.alloc(N * K * es_in), c.alloc(N * K * es_in)
+                c1, c2, f1, f2 = (c.alloc(N * 4) for _ in range(4))
+                stats = c.alloc(2 * M * 4 + 16)
+                held += [dgm, dbt, ws1, ws2, c1, c2, f1, f2, stats]
+                L.check(c.lib.grl_ln_fold(c.ctx, cin, N, K, dw1.ptr, dgm.ptr, dbt.ptr, db1.ptr if bias else None, ws1.ptr, c1.ptr, f1.ptr), "ln_fold")
+                L.check(c.lib.grl_ln_fold(c.ctx, cin, N, K, dw2.ptr, dgm.ptr, dbt.ptr, db2.ptr if bias else None, ws2.ptr, c2.ptr, f2.ptr), "ln_fold")
+                eps = 1e-5
+                ln = O.truth_layernorm(x, gamma, beta, eps)
+                gated = case % 2 == 0
+                if gated:
+                    L.check(c.lib.grl_ln_glu_nt(c.ctx, cin, cout, M, N, K, dx.ptr, ws1.ptr, ws2.ptr, c1.ptr, c2.ptr, f1.ptr, f2.ptr, eps, stats.ptr, optr, code), "ln_glu_nt")
+                    ref = O.truth_fused_glu(ln, W1, W2, b1 if bias else np.zeros(N), b2 if bias else np.zeros(N), name)[0]
+                else:
+                    L.check(c.lib.grl_ln_gemm_nt(c.ctx, cin, cout, M, N, K, dx.ptr, ws1.ptr, c1.ptr, f1.ptr, eps, stats.ptr, optr), "ln_gemm_nt")
+                    ref = O.truth_linear(ln, W1, b1)
+                y = take(dout, M * N, cout, info).reshape(M, N)
+                # the folded weight gamma*W is rounded to the storage type once more than the composed form rounds
+                tl = t if cin == L.GRL_F32 else 1.5 * TOL_BF16
+                assert O.max_rel(y, ref) < tl, info + (gated, O.max_rel(y, ref))
+        finally:
+            for b in held:
+                if b is not None:
+                    b.free()
+        if case and case % 50 == 0:
+            print("sweep case", case, flush=True)
