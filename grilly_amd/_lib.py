@@ -82,6 +82,8 @@ SIGNATURES = {
     "grl_softmax": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_void_p]),
     "grl_swiglu_act": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_void_p]),
     "grl_embed": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "grl_embed_layernorm": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                    c_float, c_void_p]),
     "grl_mean_pool": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_int]),
     "grl_bert_layer_workspace": (c_i64, [c_int, c_i64, c_i64, c_i64, c_i64, c_i64]),
     "grl_bert_layer_fwd": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_i64, ctypes.POINTER(BertLayer), c_void_p, c_float, c_void_p, c_void_p]),

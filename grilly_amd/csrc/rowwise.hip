@@ -831,6 +831,92 @@ extern "C" int grl_embed(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F,
     return GRL_OK;
 }
 
+// Embedding gather and the LayerNorm that follows it in one pass: a wave gathers its row (token + type + position, in
+// that order), rounds it to the storage type as the two-kernel sequence stores it, and normalises it in registers
+// (two-pass mean / variance like layernorm_rows_kernel).  F % 4 == 0, F <= 2048, 16-byte aligned tables.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_layernorm_kernel(const int32_t* __restrict__ ids, const float* __restrict__ tok,
+                                                             const float* __restrict__ pos, const float* __restrict__ typ,
+                                                             const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                             T* __restrict__ x, int64_t rows, int S, int F, int vocab, float eps) {
+    constexpr int MAXC = 8;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    int id = ids[row];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // the host validates; this only keeps loads in bounds
+    const float* tr = tok + (int64_t)id * F;
+    const float* pr = pos ? pos + (int64_t)(row % S) * F : nullptr;
+    const int nch = F >> 2;
+    float t[MAXC][4];
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        const int ch = lane + c * 64;
+        if (ch < nch) {
+            f32x4 v = *(const f32x4*)(tr + ch * 4);
+            if (typ) v += *(const f32x4*)(typ + ch * 4);
+            if (pr) v += *(const f32x4*)(pr + ch * 4);
+            vec4<T> q;                                   // through the storage type: what grl_embed would have written
+#pragma unroll
+            for (int i = 0; i < 4; ++i) q.set(i, v[i]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { t[c][i] = q.get(i); s += t[c][i]; }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t[c][i] = 0.f;
+        }
+    }
+    const float mean = wave_sum(s) / (float)F;
+    float q2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        if (lane + c * 64 < nch) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { const float d = t[c][i] - mean; q2 += d * d; }
+        }
+    }
+    const float sd = sqrtf(wave_sum(q2) / (float)F + eps);
+    T* yr = x + row * (int64_t)F;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        const int ch = lane + c * 64;
+        if (ch < nch) {
+            const f32x4 g = *(const f32x4*)(gamma + ch * 4);
+            const f32x4 b = *(const f32x4*)(beta + ch * 4);
+            vec4<T> o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o.set(i, g[i] * ((t[c][i] - mean) / sd) + b[i]);
+            o.store(yr + ch * 4);      // plain: the first GEMM reads these rows at once
+        }
+    }
+}
+
+extern "C" int grl_layernorm(grl_ctx* c, int dtype, int64_t rows, int64_t F, const void* x, const void* residual,
+                             const float* gamma, const float* beta, float eps, void* y);
+
+extern "C" int grl_embed_layernorm(grl_ctx* c, int dtype, int64_t B, int64_t S, int64_t F, int64_t vocab, const int32_t* ids,
+                                   const float* tok_emb, const float* pos_emb, const float* type_emb,
+                                   const float* gamma, const float* beta, float eps, void* x) {
+    GRL_REQUIRE(c && ids && tok_emb && gamma && beta && x, GRL_ERR_ARG, "grl_embed_layernorm: null argument");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_embed_layernorm: bad dtype %d", dtype);
+    GRL_REQUIRE(B >= 0 && S > 0 && F > 0 && vocab > 0 && S < (1LL << 31) && F < (1LL << 31) && vocab < (1LL << 31),
+                GRL_ERR_SHAPE, "grl_embed_layernorm: bad shape");
+    const int64_t rows = B * S;
+    if (rows == 0) return GRL_OK;
+    const bool fused = F % 4 == 0 && F <= 2048 && aligned16(tok_emb) && aligned16(x) && aligned16(gamma) && aligned16(beta) &&
+                       (!pos_emb || aligned16(pos_emb)) && (!type_emb || aligned16(type_emb));
+    if (!fused) {
+        int rc = grl_embed(c, dtype, B, S, F, vocab, ids, tok_emb, pos_emb, type_emb, x);
+        return rc ? rc : grl_layernorm(c, dtype, rows, F, x, nullptr, gamma, beta, eps, x);
+    }
+    dim3 g((unsigned)((rows + 3) / 4)), b(256);
+    if (dtype == GRL_F32) hipLaunchKernelGGL(embed_layernorm_kernel<float>, g, b, 0, c->stream, ids, tok_emb, pos_emb, type_emb, gamma, beta, (float*)x, rows, (int)S, (int)F, (int)vocab, eps);
+    else hipLaunchKernelGGL(embed_layernorm_kernel<uint16_t>, g, b, 0, c->stream, ids, tok_emb, pos_emb, type_emb, gamma, beta, (uint16_t*)x, rows, (int)S, (int)F, (int)vocab, eps);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
 // ------------------------------------------------------------------ masked mean pool (+ L2 normalise)
 // grid (ceil(F/256), B).  F % 4 == 0: a lane owns 4 adjacent features (8- or 16-byte loads), the NW waves
 // of a workgroup take every NW-th position of the sequence and their partial sums meet in LDS (sixteen waves: a

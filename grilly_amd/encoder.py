@@ -135,10 +135,9 @@ class BertEncoder:
         B, S = self._shape
         cfg, c, lib = self.cfg, self.core, self.core.lib
         mask = self.mask.ptr if self.has_mask else None
-        L.check(lib.grl_embed(c.ctx, self.code, B, S, cfg.d_model, cfg.vocab, self.ids.ptr, self.tok.ptr,
-                              self.pos.ptr, self.typ.ptr, self.x.ptr), "embed")
-        L.check(lib.grl_layernorm(c.ctx, self.code, B * S, cfg.d_model, self.x.ptr, None, self.emb_g.ptr,
-                                  self.emb_b.ptr, cfg.embedding_eps, self.x.ptr), "embedding layernorm")
+        L.check(lib.grl_embed_layernorm(c.ctx, self.code, B, S, cfg.d_model, cfg.vocab, self.ids.ptr, self.tok.ptr,
+                                        self.pos.ptr, self.typ.ptr, self.emb_g.ptr, self.emb_b.ptr, cfg.embedding_eps,
+                                        self.x.ptr), "embedding + layernorm")
         for s in self.layer_structs:
             L.check(lib.grl_bert_layer_fwd(c.ctx, self.code, B, S, cfg.heads, cfg.head_dim, cfg.d_ff, ctypes.byref(s),
                                            mask, cfg.eps, self.x.ptr, self.ws.ptr), "bert_layer_fwd")
@@ -304,9 +303,8 @@ class PreNormEncoder:
         M, d, ff, H, D = B * S, cfg.d_model, cfg.d_ff, cfg.heads, cfg.head_dim
         es = 2 if code == L.GRL_BF16 else 4
         mask = self.mask.ptr if self.has_mask else None
-        L.check(lib.grl_embed(c.ctx, code, B, S, d, cfg.vocab, self.ids.ptr, self.tok.ptr, None, None, self.x.ptr), "embed")
-        L.check(lib.grl_layernorm(c.ctx, code, M, d, self.x.ptr, None, self.emb_g.ptr, self.emb_b.ptr, cfg.emb_eps,
-                                  self.x.ptr), "embedding layernorm")
+        L.check(lib.grl_embed_layernorm(c.ctx, code, B, S, d, cfg.vocab, self.ids.ptr, self.tok.ptr, None, None,
+                                        self.emb_g.ptr, self.emb_b.ptr, cfg.emb_eps, self.x.ptr), "embedding + layernorm")
         for w in self.layers:
             # one GEMM with the packed weight; attention reads Q, K, V as column blocks of its output and applies
             # the rotation itself (queries as they are loaded, keys once per row from the cached table)

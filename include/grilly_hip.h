@@ -281,6 +281,14 @@ int grl_swiglu_act(grl_ctx* ctx, int dtype, int64_t rows, int64_t h, const void*
 int grl_embed(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t F, int64_t vocab,
               const int32_t* ids, const float* tok_emb, const float* pos_emb,
               const float* type_emb, void* x);
+
+/* grl_embed followed by grl_layernorm on the gathered rows, in one pass over them (the embedding LayerNorm of the
+ * encoders: utils/vulkan_sentence_transformer.py:729-736 after :563-707).  The gathered row is rounded to the storage
+ * type before it is normalised, as the two calls would store it; feature counts the fused kernel does not take
+ * (not a multiple of 4, above 2048, unaligned tables) run the two kernels one after the other. */
+int grl_embed_layernorm(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t F, int64_t vocab,
+                        const int32_t* ids, const float* tok_emb, const float* pos_emb, const float* type_emb,
+                        const float* gamma, const float* beta, float eps, void* x);
 /* out[b,:] = sum_s mask[b,s]*x[b,s,:] / max(sum_s mask[b,s], 1e-9), optionally L2-normalised
  * (x / max(||x||, 1e-12)); out fp32 (B,F).
  * Replaces mean pooling + normalise of encode (utils/vulkan_sentence_transformer.py:1177-1201). */

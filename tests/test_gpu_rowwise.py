@@ -268,3 +268,43 @@ def test_rowwise_randomized_shapes(backend):
         assert err < t, (case, dtype, what, rows, F, err)
         if case and case % 50 == 0:
             print("sweep case", case, flush=True)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("F,tables", [(768, "all"), (384, "all"), (2048, "tok"), (36, "tok+pos"), (250, "all"), (2052, "all")])
+def test_embed_layernorm_one_pass(backend, dtype, F, tables):
+    """grl_embed_layernorm against grl_embed followed by grl_layernorm (same rows within an ulp of the storage type:
+    the two LayerNorm kernels reduce in different lane orders) and against the float64 oracle; feature counts the
+    one-pass kernel takes (multiples of 4 up to 2048) and those that run the two kernels, with and without the
+    position / type tables."""
+    c = backend.core
+    code = L.GRL_BF16 if dtype == "bf16" else L.GRL_F32
+    es = 2 if dtype == "bf16" else 4
+    rng = np.random.default_rng(F)
+    B, S, V = 3, 37, 101
+    tok = rng.standard_normal((V, F)).astype(np.float32)
+    pos = rng.standard_normal((S, F)).astype(np.float32) if tables != "tok" else None
+    typ = rng.standard_normal((2, F)).astype(np.float32) if tables == "all" else None
+    g = (1 + 0.2 * rng.standard_normal(F)).astype(np.float32); b = (0.2 * rng.standard_normal(F)).astype(np.float32)
+    ids = rng.integers(0, V, (B, S)).astype(np.int32)
+    dtok, dg, db, dids = c.upload(tok), c.upload(g), c.upload(b), c.upload_raw(ids)
+    dpos = c.upload(pos) if pos is not None else None
+    dtyp = c.upload(typ) if typ is not None else None
+    x1, x2 = c.alloc(B * S * F * es), c.alloc(B * S * F * es)
+    pp, tp = (dpos.ptr if dpos else None), (dtyp.ptr if dtyp else None)
+    try:
+        L.check(c.lib.grl_embed_layernorm(c.ctx, code, B, S, F, V, dids.ptr, dtok.ptr, pp, tp, dg.ptr, db.ptr, 1e-5, x1.ptr), "embed_layernorm")
+        L.check(c.lib.grl_embed(c.ctx, code, B, S, F, V, dids.ptr, dtok.ptr, pp, tp, x2.ptr), "embed")
+        L.check(c.lib.grl_layernorm(c.ctx, code, B * S, F, x2.ptr, None, dg.ptr, db.ptr, 1e-5, x2.ptr), "layernorm")
+        y1, y2 = c.download(x1, (B, S, F), code), c.download(x2, (B, S, F), code)
+    finally:
+        for t in (dtok, dg, db, dids, dpos, dtyp, x1, x2):
+            if t is not None:
+                t.free()
+    e = tok[ids].astype(np.float64) + (typ[0] if typ is not None else 0.0) + (pos[None] if pos is not None else 0.0)
+    if dtype == "bf16":
+        e = O.bf16_round(e.astype(np.float32)).astype(np.float64)
+    ref = O.truth_layernorm(e, g, b, 1e-5)
+    t = TOL_F32 if dtype == "fp32" else TOL_BF16
+    assert O.max_rel(y1, ref) < t and O.max_rel(y2, ref) < t
+    np.testing.assert_allclose(y1, y2, rtol=2.0 ** -7 if dtype == "bf16" else 1e-5, atol=2.0 ** -9 if dtype == "bf16" else 1e-6)
