@@ -4,6 +4,7 @@ backend/compute.py:153-195, `cleanup()` and `set_architecture()`."""
 from .core import HipCore
 from .fnn import HipFNN
 from .attention import HipAttention
+from .embedding import HipLearning, HipPooling
 
 
 class HipCompute:
@@ -12,6 +13,9 @@ class HipCompute:
         self.architecture = architecture
         self.fnn = HipFNN(self.core)
         self.attention = HipAttention(self.core, architecture)
+        # the encoder's first and last step (reference compute.py:44, :47 bind whole namespaces; only these two methods are on the path)
+        self.learning = HipLearning(self.core)
+        self.pooling = HipPooling(self.core)
         # always present here; the reference only binds it after set_architecture (compute.py:99)
         self.flash_attention2 = self.attention.flash_attention2
         self.flash_attention2_rope = self.attention.flash_attention2_rope
@@ -47,6 +51,7 @@ class HipCompute:
     def fused_reglu(self, *a, **k): return self.fnn.fused_reglu(*a, **k)
     def fused_geglu(self, *a, **k): return self.fnn.fused_geglu(*a, **k)
     def apply_rope(self, *a, **k): return self.attention.apply_rope(*a, **k)
+    def embedding_lookup(self, *a, **k): return self.learning.embedding_lookup(*a, **k)     # reference compute.py:324-326
 
     def __enter__(self):
         return self

@@ -139,8 +139,9 @@ class HipCore:
         return float(ms.value)
 
     def clock_probe_begin(self, millis):
-        """start the shader-clock probe: it runs for `millis` beside whatever is enqueued next"""
-        L.check(self.lib.grl_clock_probe_begin(self.ctx, float(millis)), "clock_probe_begin")
+        """start the shader-clock probe: it runs for `millis` (held within the library's (0, 500] ms range) beside
+        whatever is enqueued next"""
+        L.check(self.lib.grl_clock_probe_begin(self.ctx, min(max(float(millis), 0.05), 500.0)), "clock_probe_begin")
 
     def clock_probe_end(self):
         """wait for the probe; average shader clock in GHz while it ran"""

@@ -23,13 +23,17 @@ struct grl_ctx {
     std::map<void*, size_t> live;
     grl_pool_stats stats{};
     // cos/sin tables of the rotary embedding, built once per (head dim, base, scaling, pairing) and kept until the
-    // context goes away; a table built for S positions serves every shorter sequence
+    // context goes away; a table built for S positions serves every shorter sequence.  A table that a longer one
+    // replaces is retired, not freed: callers hold its raw pointer between lookup and launch (grl_destroy frees
+    // every live pool block, retired tables included)
     struct rope_table { int S, D, style; float base, scaling; void* dev; };
     std::mutex tab_mu;
     std::vector<rope_table> rope_tables;
+    std::vector<void*> retired_tables;
     // shader-clock probe (grl_clock_probe_begin / _end): its own stream, so that it runs beside the work it observes
     hipStream_t probe_stream = nullptr;
     uint64_t* probe_out = nullptr;      // device: {shader cycles, 100 MHz ticks}
+    bool probe_pending = false;         // a probe was launched and its result not read yet (under timer_mu)
 };
 
 // device pointer to a (>= S, D/2) table of {cos, sin}; builds it on first use (on the context stream)
@@ -234,8 +238,14 @@ __device__ __forceinline__ void silu_plain4(float (&v)[4]) {       // four value
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = v[i] * e[i];
 }
-// v_mul_legacy_f32 (0 times anything, infinities and NaN included, is 0); the intrinsic has no clang builtin
-extern "C" __device__ float fmul_legacy(float, float) __asm("llvm.amdgcn.fmul.legacy");
+// v_mul_legacy_f32 (0 times anything, infinities and NaN included, is 0).  clang has no builtin for it, so it is
+// one inline-asm instruction.  The hazard recognizer does not look inside inline asm: a transcendental result (the
+// reciprocal below) needs one wait state before an ordinary VALU instruction reads it, hence the leading s_nop.
+__device__ __forceinline__ float fmul_legacy(float a, float b) {
+    float r;
+    asm("s_nop 0\n\tv_mul_legacy_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 // shaders/fused-linear-gelu.glsl:45-63 rewritten with tanh(u) = 2/(1+exp(-2u)) - 1:
 //   0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (c + 0.044715 c^3), c = clamp(x, +-50).
 // The +-50 clamp needs no instruction of its own: beyond |x| = 50 (already from |x| > 7) the exponential saturates
@@ -258,7 +268,8 @@ __device__ __forceinline__ void gelu_fast4(float (&v)[4]) {
     for (int i = 0; i < 4; ++i) e[i] = 1.0f + e[i];
 #pragma unroll
     for (int i = 0; i < 4; ++i) e[i] = __builtin_amdgcn_rcpf(e[i]);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = fmul_legacy(v[i], e[i]);
+    // the four products in one statement behind one wait state (whichever reciprocal the scheduler placed last)
+    asm("s_nop 0\n\tv_mul_legacy_f32 %0, %0, %4\n\tv_mul_legacy_f32 %1, %1, %5\n\tv_mul_legacy_f32 %2, %2, %6\n\tv_mul_legacy_f32 %3, %3, %7"
+        : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : "v"(e[0]), "v"(e[1]), "v"(e[2]), "v"(e[3]));
 }
 #endif

@@ -243,15 +243,20 @@ extern "C" int grl_clock_probe_begin(grl_ctx* c, float millis) {
     GRL_CHECK_HIP(hipSetDevice(c->device));
     if (!c->probe_stream) GRL_CHECK_HIP(hipStreamCreateWithFlags(&c->probe_stream, hipStreamNonBlocking));
     if (!c->probe_out) GRL_CHECK_HIP(hipMalloc((void**)&c->probe_out, 2 * sizeof(uint64_t)));
+    c->probe_pending = false;
+    GRL_CHECK_HIP(hipStreamSynchronize(c->probe_stream));        // an earlier probe that nobody read has ended by now
     hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, c->probe_stream, c->probe_out, (uint64_t)((double)millis * 1e5));
     GRL_CHECK_LAUNCH();
+    c->probe_pending = true;
     return GRL_OK;
 }
 
 extern "C" int grl_clock_probe_end(grl_ctx* c, float* ghz) {
     GRL_REQUIRE(c && ghz, GRL_ERR_ARG, "grl_clock_probe_end: null argument");
     std::lock_guard<std::mutex> lk(c->timer_mu);
-    GRL_REQUIRE(c->probe_stream && c->probe_out, GRL_ERR_ARG, "grl_clock_probe_end: no probe was started");
+    GRL_REQUIRE(c->probe_stream && c->probe_out && c->probe_pending, GRL_ERR_ARG,
+                "grl_clock_probe_end: no probe was started since the last reading");
+    c->probe_pending = false;       // one reading per probe, also when the copy below fails
     uint64_t h[2] = {0, 0};
     // copied on the probe's own stream: a copy on the null stream would serialise with the work being observed
     GRL_CHECK_HIP(hipMemcpyAsync(h, c->probe_out, sizeof(h), hipMemcpyDeviceToHost, c->probe_stream));

@@ -213,6 +213,7 @@ extern "C" int grl_gemm_nn(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, i
 static __device__ __align__(256) unsigned char scratch[GRL_NN_SCRATCH_BYTES];
 
 static std::mutex g_scratch_mu;
+static std::mutex g_scratch_pair_mu;     // held from a call's transpose launch to its GEMM launch
 static void* g_scratch_ptr[64];          // per device ordinal; null until looked up
 
 // device address of this GPU's copy of `scratch` (looked up on first use, with the device current)
@@ -255,7 +256,10 @@ extern "C" int grl_gemm_nn_noalloc(grl_ctx* c, int in_dtype, int out_dtype, int6
     rc = nn_scratch_address(c, &ws);
     if (rc) return rc;
     // the transpose overwrites every byte of the (N,K) image the GEMM reads, so nothing of the previous
-    // call's contents needs clearing
+    // call's contents needs clearing.  The two launches must sit next to each other on the stream: host threads
+    // that share a context share its stream, and without the lock thread B's transpose could be enqueued between
+    // thread A's transpose and A's GEMM (A would then multiply by B's matrix).
+    std::lock_guard<std::mutex> pair(g_scratch_pair_mu);
     rc = grl_transpose2d(c, in_dtype, K, N, B, ws);   // (K,N) -> (N,K)
     if (!rc) rc = grl_gemm_nt(c, in_dtype, out_dtype, M, N, K, A, ws, nullptr, C, GRL_EPI_NONE);
     return rc;

@@ -640,23 +640,27 @@ int grl_rope_table_get(grl_ctx* c, int S, int D, float base, float scaling, int 
     std::lock_guard<std::mutex> lk(c->tab_mu);
     for (auto& t : c->rope_tables)
         if (t.D == D && t.style == style && t.base == base && t.scaling == scaling && t.S >= S) { *out = (const float*)t.dev; return GRL_OK; }
-    // not there (or too short): build one; a shorter table of the same kind is replaced.  Kernels already queued
-    // on the stream may still read the old one, and the pool hands a freed block to the next request of its
-    // size, so the old table is only dropped once the stream has drained.
+    // Not there (or too short): build one.  The pointer handed out leaves this function without any hold on the
+    // table (another thread of the same context may be between its lookup and its launch), so a table is NEVER
+    // freed while the context lives: a superseded one moves to the retired list and keeps its memory until
+    // grl_destroy.  Lengths are rounded up to a power of two (at least 1024 positions), so one kind of table is
+    // rebuilt at most once per doubling of the sequence length and the retired ones add up to less than the live one.
+    int64_t cap = 1024;
+    while (cap < S) cap *= 2;
+    if (cap * (D / 2) >= (1LL << 31)) cap = S;
     for (size_t i = 0; i < c->rope_tables.size(); ++i) {
         auto& t = c->rope_tables[i];
         if ((t.D == D && t.style == style && t.base == base && t.scaling == scaling) || c->rope_tables.size() >= 16) {
-            GRL_CHECK_HIP(hipStreamSynchronize(c->stream));
-            grl_free(c, t.dev);
+            c->retired_tables.push_back(t.dev);
             c->rope_tables.erase(c->rope_tables.begin() + i);
             break;
         }
     }
-    void* dev = grl_malloc(c, (size_t)S * (D / 2) * sizeof(float2));
+    void* dev = grl_malloc(c, (size_t)cap * (D / 2) * sizeof(float2));
     if (!dev) return GRL_ERR_OOM;
-    int rc = grl_build_rope_table_styled(c, (float*)dev, S, D, base, scaling, style);
+    int rc = grl_build_rope_table_styled(c, (float*)dev, (int)cap, D, base, scaling, style);
     if (rc) { grl_free(c, dev); return rc; }
-    c->rope_tables.push_back({S, D, style, base, scaling, dev});
+    c->rope_tables.push_back({(int)cap, D, style, base, scaling, dev});
     *out = (const float*)dev;
     return GRL_OK;
 }

@@ -137,8 +137,10 @@ int grl_gemm_nn(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N,
  * capture, tight serving loops, harnesses that forbid device allocation.  The transposed copy of B goes into
  * a static device array of grl_gemm_nn_noalloc_max_bytes() = 32 MiB that every GPU the library runs on holds
  * until the process ends (its address is looked up in grl_create); K*N*sizeof(in_dtype) beyond that returns
- * GRL_ERR_SHAPE.  All calls on one GPU share the array: calls that overlap on one GPU (two contexts, i.e. two
- * streams, of the same device) race, calls on one context are ordered by its stream. */
+ * GRL_ERR_SHAPE.  All calls on one GPU share the array.  Host threads that call it on ONE context are safe: a lock
+ * keeps each call's two launches (transpose into the array, GEMM out of it) adjacent on the context's stream,
+ * which then orders the calls.  Calls on two contexts of the same GPU run on two streams and race on the
+ * array: the caller must not overlap them. */
 int grl_gemm_nn_noalloc(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
                         const void* A, const void* B, void* C);
 int64_t grl_gemm_nn_noalloc_max_bytes(void);

@@ -308,3 +308,39 @@ def test_embed_layernorm_one_pass(backend, dtype, F, tables):
     t = TOL_F32 if dtype == "fp32" else TOL_BF16
     assert O.max_rel(y1, ref) < t and O.max_rel(y2, ref) < t
     np.testing.assert_allclose(y1, y2, rtol=2.0 ** -7 if dtype == "bf16" else 1e-5, atol=2.0 ** -9 if dtype == "bf16" else 1e-6)
+
+
+def test_embedding_lookup_and_mean_pool_facade(backend):
+    """numpy-in / numpy-out `learning.embedding_lookup` (reference backend/learning.py:811-877, shaders/embedding-lookup.glsl:
+    out-of-range ids give zero rows, 1-D ids are one batch entry) and `pooling.mean_pool` (backend/pooling.py:22-143,
+    shaders/embedding-pool.glsl: the mask is a 0.5 threshold, a sequence without kept positions pools to zeros)."""
+    rng = np.random.default_rng(31)
+    for (B, S, V, F) in [(3, 17, 50, 384), (2, 5, 9, 7), (1, 1, 1, 1), (4, 64, 300, 768)]:
+        table = rng.standard_normal((V, F)).astype(np.float32)
+        ids = rng.integers(0, V, (B, S))
+        out = backend.learning.embedding_lookup(ids, table)
+        assert out.dtype == np.float32 and out.shape == (B, S, F)
+        np.testing.assert_array_equal(out, table[ids])
+        np.testing.assert_array_equal(backend.embedding_lookup(ids[0], table), table[ids[0]][None])      # 1-D ids, Compute delegate
+        bad = ids.copy(); bad[0, 0] = V; bad[-1, -1] = -1
+        got = backend.learning.embedding_lookup(bad, table)
+        want = table[np.clip(bad, 0, V - 1)]; want[0, 0] = 0; want[-1, -1] = 0
+        np.testing.assert_array_equal(got, want)
+        x = rng.standard_normal((B, S, F)).astype(np.float32)
+        np.testing.assert_allclose(backend.pooling.mean_pool(x), x.astype(np.float64).mean(1), rtol=1e-5, atol=1e-6)
+        mask = (rng.random((B, S)) < 0.6).astype(np.float32)
+        mask[0] = 0                                     # nothing kept: zeros
+        if B > 1:
+            mask[1] = np.where(np.arange(S) % 2, 0.51, 0.49)    # threshold, not weight
+        keep = (mask > 0.5)
+        cnt = keep.sum(1, keepdims=True)
+        want = np.where(cnt > 0, (x.astype(np.float64) * keep[..., None]).sum(1) / np.maximum(cnt, 1), 0.0)
+        got = backend.pooling.mean_pool(x, mask)
+        assert got.dtype == np.float32 and got.shape == (B, F)
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        backend.pooling.mean_pool(np.zeros((2, 3), np.float32))
+    with pytest.raises(ValueError):
+        backend.pooling.mean_pool(np.zeros((2, 3, 4), np.float32), np.zeros((2, 4), np.float32))
+    with pytest.raises(ValueError):
+        backend.learning.embedding_lookup(np.zeros((2, 3), np.int64), np.zeros(5, np.float32))

@@ -342,3 +342,55 @@ def test_prenorm_geglu_layer_structure():
     np.testing.assert_allclose(got, rot, rtol=1e-9, atol=1e-9)
     assert np.abs(got - plain).max() > 1e-3
     assert full.shape == x.shape
+
+
+def test_postln_layer_written_out(corc):
+    """The post-LN layer written out step by step from the reference's own CPU branches
+    (utils/vulkan_sentence_transformer.py:976-1035 with _attention_cpu :1069-1107), independently of both oracles:
+    separate Q, K, V projections on row blocks of the packed weight, heads = plain reshape of the last dimension,
+    scores.scale + (1-mask).(-1e9) per key, softmax, out-proj, LayerNorm(attn_out + x) with the numpy mean / var of
+    the fallback, tanh GELU, LayerNorm(ffn_out + x1).  Structural mutations that a shared ordering mistake in the
+    two oracles would hide must each move the result: residual taken after instead of before LN1, the second
+    residual taken from the layer input instead of from x1, and the LayerNorm parameter pairs swapped."""
+    rng = np.random.default_rng(21)
+    B, S, H, D, ff = 2, 11, 3, 8, 40
+    d = H * D
+    n = lambda *s: rng.standard_normal(s) * 0.3
+    w = {"w_qkv": n(3 * d, d), "b_qkv": n(3 * d), "w_o": n(d, d), "b_o": n(d), "ln1_g": 1 + n(d), "ln1_b": n(d),
+         "w_ff1": n(ff, d), "b_ff1": n(ff), "w_ff2": n(d, ff), "b_ff2": n(d), "ln2_g": 1 + n(d), "ln2_b": n(d)}
+    x = n(B, S, d)
+    mask = np.ones((B, S), np.float32); mask[1, 7:] = 0
+
+    def ln(t, g, b):
+        return (t - t.mean(-1, keepdims=True)) / np.sqrt(t.var(-1, keepdims=True) + 1e-5) * g + b
+
+    def layer(variant=None):
+        q = x @ w["w_qkv"][:d].T + w["b_qkv"][:d]
+        k = x @ w["w_qkv"][d:2 * d].T + w["b_qkv"][d:2 * d]
+        v = x @ w["w_qkv"][2 * d:].T + w["b_qkv"][2 * d:]
+        q, k, v = (t.reshape(B, S, H, D) for t in (q, k, v))
+        out = np.zeros((B, S, H, D))
+        for b in range(B):
+            for h in range(H):
+                sc = q[b, :, h] @ k[b, :, h].T / np.sqrt(D) + ((1.0 - mask[b]) * -1e9)[None, :]
+                p = np.exp(sc - sc.max(-1, keepdims=True))
+                out[b, :, h] = (p / p.sum(-1, keepdims=True)) @ v[b, :, h]
+        a = out.reshape(B, S, d) @ w["w_o"].T + w["b_o"]
+        g1, b1, g2, b2 = w["ln1_g"], w["ln1_b"], w["ln2_g"], w["ln2_b"]
+        if variant == "swapped_ln":
+            g1, b1, g2, b2 = g2, b2, g1, b1
+        x1 = ln(a + x, g1, b1) if variant != "residual_after_ln1" else ln(a, g1, b1) + x
+        f = x1 @ w["w_ff1"].T + w["b_ff1"]
+        f = 0.5 * f * (1 + np.tanh(np.sqrt(2 / np.pi) * (f + 0.044715 * f ** 3)))
+        f = f @ w["w_ff2"].T + w["b_ff2"]
+        return ln(f + (x if variant == "second_residual_from_input" else x1), g2, b2)
+
+    want = layer()
+    got64 = O.truth_bert_layer(x, w, mask, H)
+    np.testing.assert_allclose(got64, want, rtol=0, atol=1e-7)       # the oracle forms score + bias in fp32, as the shader does
+    w32 = {k: v.astype(np.float32) for k, v in w.items()}
+    got_c = corc.bert_layer(x.astype(np.float32), w32, mask, H)
+    assert rel(got_c, want) < 2e-5
+    for variant in ("residual_after_ln1", "second_residual_from_input", "swapped_ln"):
+        assert np.abs(layer(variant) - want).max() > 5e-2, variant
+        assert np.abs(layer(variant) - got64).max() > 5e-2, variant

@@ -65,3 +65,39 @@ def test_gemm_nn_noalloc_limit_and_arguments(backend):
         assert c.lib.grl_gemm_nn_noalloc(c.ctx, L.GRL_F32, L.GRL_F32, 2, 2, 2, None, t.ptr, t.ptr) == L.ERR_ARG
         assert c.lib.grl_gemm_nn_noalloc(c.ctx, L.GRL_F32, L.GRL_F32, 0, 5, 5, None, None, None) == 0
     assert c.lib.grl_gemm_nn_noalloc(None, 0, 0, 1, 1, 1, None, None, None) == L.ERR_ARG
+
+
+def test_concurrent_noalloc_gemm_on_one_context(backend):
+    """Two threads call the allocation-free gemm(A,B) on one context with different B matrices: its two launches
+    (transpose into the shared static array, GEMM out of it) must stay adjacent on the stream, so each thread gets
+    the product with its own B."""
+    import threading
+    c = backend.core
+    errors = []
+
+    def worker(tid):
+        try:
+            rng = np.random.default_rng(900 + tid)
+            M, K, N = 200 + 8 * tid, 512, 384
+            A = rng.standard_normal((M, K)).astype(np.float32)
+            B = (rng.standard_normal((K, N)) * (1.0 + tid)).astype(np.float32)
+            want = O.truth_gemm(A, B)
+            da, db = c.upload(A), c.upload(B)
+            dc = c.alloc(M * N * 4)
+            try:
+                for r in range(40):
+                    L.check(c.lib.grl_gemm_nn_noalloc(c.ctx, L.GRL_F32, L.GRL_F32, M, N, K, da.ptr, db.ptr, dc.ptr), "noalloc")
+                    got = c.download(dc, (M, N))
+                    assert O.max_rel(got, want) < TOL_F32, (tid, r)
+            finally:
+                da.free(); db.free(); dc.free()
+        except Exception as e:
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(3)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=120)
+    assert not any(t.is_alive() for t in threads), "a worker did not finish"
+    assert not errors, errors
