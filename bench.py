@@ -4,9 +4,9 @@ FFN 3072 GELU, fused QKV) at batch 128 x seq 512, bf16 storage with fp32 accumul
 MI355X.  A step = one full forward over one synthetic batch already resident in HBM.
 
 Prints one JSON line: encoder tokens/s, plus
-  roofline     -- the dominant kernel (the plain bf16 MFMA GEMM): algorithmic FLOPs per launch divided
-                  by its average launch duration, measured here with HIP events on the library's
-                  own stream, against the 2.5 PFLOP/s dense bf16 MFMA peak;
+  roofline     -- the dominant kernel (the bf16 MFMA GEMM instantiation with the largest share of the forward):
+                  algorithmic FLOPs per launch divided by its average launch duration, measured here with HIP
+                  events on the library's own stream, against the 2.5 PFLOP/s dense bf16 MFMA peak;
   kernels      -- the same measurement for every kernel of the layer (GEMMs and attention against
                   the MFMA peak, LayerNorm against 8 TB/s HBM), each launched on the data the layer really
                   hands it, each with a sampled check of the timed output buffer against the float64 closed form;
@@ -36,10 +36,10 @@ PEAK_HBM = 8.0e12       # B/s
 NOMINAL_GHZ = 2.4        # engine clock the MFMA peaks are quoted at (256 CUs x 4 SIMDs x 1024 bf16 FLOP/cycle x 2.4 GHz = 2.5 PFLOP/s)
 TOL = {"bf16": 2e-2, "fp32": 1e-4}
 
-WARM = 5
+WARM = 10
 
 
-def gemm_traffic(dtype, B, S):
+def gemm_traffic(dtype, B, S, kernel):
     """HBM bytes per launch of the dominant kernel: a profiler reading (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE),
     not something this script can measure itself, so it comes from the tracked record next to the profile
     summary and is reported only for exactly the workload it was taken on."""
@@ -49,7 +49,7 @@ def gemm_traffic(dtype, B, S):
     except (OSError, ValueError):
         return None, None
     k = rec.get("key", {})
-    if (k.get("dtype"), k.get("batch"), k.get("seq")) != (dtype, B, S):
+    if (k.get("dtype"), k.get("batch"), k.get("seq"), k.get("kernel")) != (dtype, B, S, kernel):
         return None, None
     return rec.get("traffic_bytes_per_launch"), rec.get("measured_at_commit")
 
@@ -63,6 +63,31 @@ def time_launches(core, fn, reps, warm=WARM):
     for _ in range(reps):
         fn()
     return core.timer_stop() / reps
+
+
+def lap_times(core, fn, reps, warm=WARM):
+    """per-launch milliseconds of `reps` back-to-back calls of fn() (which only enqueues): one event between every two
+    launches on the context stream, no host synchronisation inside the sequence"""
+    from grilly_amd import _lib as L
+    import ctypes
+    reps = min(reps, 255)
+    for _ in range(warm):
+        fn()
+    core.sync()
+    for i in range(reps):
+        L.check(core.lib.grl_timer_lap(core.ctx, i))
+        fn()
+    L.check(core.lib.grl_timer_lap(core.ctx, reps))
+    ms = ctypes.c_float()
+    out = []
+    for i in range(reps):
+        L.check(core.lib.grl_timer_lap_ms(core.ctx, i, i + 1, ctypes.byref(ms)))
+        out.append(float(ms.value))
+    return out
+
+
+def median(v):
+    return float(np.median(np.asarray(v, np.float64)))
 
 
 def download_rows(core, buf, row0, nrows, ncols, code):
@@ -129,6 +154,32 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
     for f in (f_qkv, f_fa, f_out, f_ln, f_ff1, f_ff2):       # data-flow order, untimed
         L.check(f())
     c.sync()
+    fused_runs = []
+    if getattr(enc, "fused", False):
+        # the four GEMMs of the layer in the form the forward launches them (LayerNorms folded in): the raw residual
+        # stream r0 = x (its "LayerNorm" statistics are those of x itself), r1 = out-proj + LN(r0), ff, r2 = FFN2 + LN(r1)
+        fs = enc.fused_structs[0]
+        r1, r2, ffl = c.alloc(M * d * es), c.alloc(M * d * es), c.alloc(M * ff * es)
+        qkvl = c.alloc(M * 3 * d * es)
+        st0, st1, st2 = c.alloc(M * 8), c.alloc(M * 8), c.alloc(M * 8)
+        part = c.alloc(lib.grl_gemm_nt_resln_workspace(M, d))
+        f_st = lambda: lib.grl_ln_stats(c.ctx, code, M, d, x.ptr, cfg.eps, st0.ptr)
+        f_qkvl = lambda: lib.grl_ln_gemm_nt_stats(c.ctx, code, code, M, 3 * d, d, x.ptr, fs.ws_qkv, fs.c_qkv, fs.bf_qkv, st0.ptr, qkvl.ptr, 0)
+        f_outl = lambda: lib.grl_gemm_nt_resln(c.ctx, code, M, d, d, attn.ptr, fs.w_o, fs.b_o, x.ptr, st0.ptr, fs.in_g, fs.in_b, r1.ptr,
+                                               cfg.eps, st1.ptr, part.ptr)
+        f_ff1l = lambda: lib.grl_ln_gemm_nt_stats(c.ctx, code, code, M, ff, d, r1.ptr, fs.ws_ff1, fs.c_ff1, fs.bf_ff1, st1.ptr, ffl.ptr, 1)
+        f_ff2l = lambda: lib.grl_gemm_nt_resln(c.ctx, code, M, d, ff, ffl.ptr, fs.w_ff2, fs.b_ff2, r1.ptr, st1.ptr, fs.ln1_g, fs.ln1_b, r2.ptr,
+                                               cfg.eps, st2.ptr, part.ptr)
+        for f in (f_st, f_qkvl, f_outl, f_ff1l, f_ff2l):
+            L.check(f())
+        c.sync()
+        fused_runs = [
+            ("gemm_qkv_ln", "gemm_nt_ln", f_qkvl, 2.0 * M * 3 * d * d, (M * d + 3 * d * d + M * 3 * d) * es),
+            ("gemm_out_resln", "gemm_nt_resln", f_outl, 2.0 * M * d * d, (3 * M * d + d * d) * es),
+            ("gemm_ffn1_ln_gelu", "gemm_nt_ln_gelu", f_ff1l, 2.0 * M * d * ff, (M * d + d * ff + M * ff) * es),
+            ("gemm_ffn2_resln", "gemm_nt_resln", f_ff2l, 2.0 * M * d * ff, (M * ff + d * ff + 2 * M * d) * es),
+            ("ln_stats", "ln", f_st, 0.0, M * d * es + M * 8),
+        ]
     runs = [
         ("gemm_qkv", "gemm_nt", f_qkv, 2.0 * M * 3 * d * d, (M * d + 3 * d * d + M * 3 * d) * es),
         ("gemm_out", "gemm_nt", f_out, 2.0 * M * d * d, (2 * M * d + d * d) * es),
@@ -137,13 +188,13 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
         ("fa2_fwd", "fa2", f_fa, 4.0 * B * H * S * S * D, 4 * M * d * es),
         ("fa2_fwd_key_mask", "fa2", f_fam, 4.0 * B * H * S * S * D, 4 * M * d * es),     # nominal FLOPs: padding counted
         ("layernorm_residual", "ln", f_ln, 0.0, 3 * M * d * es),
-    ]
+    ] + fused_runs
     out = {}
     for name, group, fn, flops, nbytes in runs:
         if only and name not in only:
             continue
         ms = time_launches(c, fn, reps)
-        rec = {"ms": round(ms, 4), "group": group, "flops": flops, "bytes": nbytes}
+        rec = {"ms": round(ms, 4), "median_ms": round(median(lap_times(c, fn, reps)), 4), "group": group, "flops": flops, "bytes": nbytes}
         # the shader clock these launches run at: a one-wave probe on a second stream lives for 70 % of a repeat of the
         # same launch sequence (the clock is one domain for the whole GPU)
         c.sync()
@@ -188,6 +239,36 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
             if k in out:
                 out[k]["max_rel_vs_float64"] = float(f"{e:.3g}")
                 out[k]["within_tolerance"] = bool(e < TOL[dt])
+    if fused_runs and check:
+        from oracle import oracle_np as O
+        rng = np.random.default_rng(8)
+        rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 30)]))
+        dl = lambda ptr, n: download_rows(c, _Ptr(ptr), 0, 1, n, L.GRL_F32)[0]
+        wt = lambda ptr, r, k: download_rows(c, _Ptr(ptr), 0, r, k, code)
+        s0 = enc.layer_structs[0]
+        xs = gather_rows(c, x, rows, d, code)
+        xn = O.truth_layernorm(xs, dl(fs.in_g, d), dl(fs.in_b, d), cfg.eps)
+        e = {"gemm_qkv_ln": max_rel(gather_rows(c, qkvl, rows, 3 * d, code), O.truth_linear(xn, wt(s0.w_qkv, 3 * d, d), dl(s0.b_qkv, 3 * d)))}
+        r1s = gather_rows(c, r1, rows, d, code)
+        e["gemm_out_resln"] = max_rel(r1s, O.truth_linear(gather_rows(c, attn, rows, d, code), wt(s0.w_o, d, d), dl(s0.b_o, d)) + xn)
+        x1n = O.truth_layernorm(r1s, dl(s0.ln1_g, d), dl(s0.ln1_b, d), cfg.eps)
+        ffs = gather_rows(c, ffl, rows, ff, code)
+        e["gemm_ffn1_ln_gelu"] = max_rel(ffs, O.truth_linear(x1n, wt(s0.w_ff1, ff, d), dl(s0.b_ff1, ff), "gelu"))
+        e["gemm_ffn2_resln"] = max_rel(gather_rows(c, r2, rows, d, code), O.truth_linear(ffs, wt(s0.w_ff2, d, ff), dl(s0.b_ff2, d)) + x1n)
+        st = download_rows(c, st1, 0, M, 2, L.GRL_F32)[rows]
+        r64 = r1s.astype(np.float64)
+        sd = np.sqrt(r64.var(-1) + cfg.eps)
+        # 1/sd relative, mean/sd absolute (it is a number of spreads, near zero for these rows)
+        e["row_statistics_out"] = max(max_rel(st[:, 0], 1 / sd), float(np.abs(st[:, 1] - r64.mean(-1) / sd).max()))
+        for k, v in e.items():
+            if k == "row_statistics_out":
+                out["gemm_out_resln"]["row_statistics_max_err"] = float(f"{v:.3g}")
+            else:
+                out[k]["max_rel_vs_float64"] = float(f"{v:.3g}")
+                out[k]["within_tolerance"] = bool(v < TOL[dt])
+    if fused_runs:
+        for b in (r1, r2, ffl, qkvl, st0, st1, st2, part):
+            b.free()
     for b in (qkv, attn, ffb, proj, x1, y2, mask_d, attn_m):
         b.free()
     return out
@@ -297,6 +378,111 @@ def side_workload(backend, mode, seed, reps, check=True):
     return res
 
 
+def small_configs(backend, reps, check=True):
+    """BASELINE configs[0] (the README quick-start operators, fp32: linear x[32,384].W[384,128] + 0 -> swiglu, and
+    attention on (32,8,64,64) Q/K/V, no mask, scale 1/8) in microseconds, device-resident (per-launch events, median
+    and mean) and numpy -> numpy through the facade (host clock around the whole call, uploads and downloads
+    included, like the reference's API), and configs[1] (MiniLM-L6-shaped fp32 encoder, batch 64 x seq 256, padding
+    mask with lengths uniform in [32,256]) as a device-resident forward.  Each result is checked: the operators
+    against the float64 closed forms, two sequences of the encoder against the C restatement of the shaders."""
+    from grilly_amd import _lib as L
+    from grilly_amd import BertEncoder, random_bert_weights
+    from grilly_amd.encoder import MINILM_L6
+    c, lib = backend.core, backend.core.lib
+    rng = np.random.default_rng(20260131 + 1)
+    x = rng.standard_normal((32, 384)).astype(np.float32)
+    Wt = np.ascontiguousarray(rng.standard_normal((384, 128)).astype(np.float32).T)
+    b0 = np.zeros(128, np.float32)
+    q, k, v = (np.ascontiguousarray(rng.standard_normal((32, 8, 64, 64)).astype(np.float32).transpose(0, 2, 1, 3)) for _ in range(3))
+    dx, dw, db = c.upload(x), c.upload(Wt), c.upload(b0)
+    dy, dg = c.alloc(32 * 128 * 4), c.alloc(32 * 64 * 4)
+    dq, dk, dv, do = c.upload(q), c.upload(k), c.upload(v), c.alloc(q.size * 4)
+    f_lin = lambda: lib.grl_gemm_nt(c.ctx, L.GRL_F32, L.GRL_F32, 32, 128, 384, dx.ptr, dw.ptr, db.ptr, dy.ptr, 0)
+    f_act = lambda: lib.grl_swiglu_act(c.ctx, L.GRL_F32, 32, 64, dy.ptr, dg.ptr)
+    f_fa = lambda: lib.grl_fa2_fwd(c.ctx, L.GRL_F32, 32, 64, 8, 64, dq.ptr, dk.ptr, dv.ptr, None, do.ptr, 0.125, 0, 0, 1e4, 1.0, None)
+    us = lambda v: {"median_us": round(median(v) * 1e3, 2), "mean_us": round(float(np.mean(v)) * 1e3, 2), "launches": len(v)}
+
+    def host_us(fn, n=20):
+        fn(); t = []
+        for _ in range(n):
+            t0 = time.perf_counter(); fn(); t.append((time.perf_counter() - t0) * 1e3)
+        return us(t)
+    r0 = {"workload": "BASELINE configs[0]: linear x[32,384].W[384,128]+0 -> swiglu; attention Q/K/V (32,8,64,64), no mask, fp32",
+          "linear": {"device_resident": us(lap_times(c, f_lin, 50)), "numpy_to_numpy": host_us(lambda: backend.fnn.linear(x, Wt, b0))},
+          "activation_swiglu": {"device_resident": us(lap_times(c, f_act, 50)),
+                                "numpy_to_numpy": host_us(lambda: backend.fnn.activation_swiglu(np.zeros((32, 128), np.float32)))},
+          "flash_attention2": {"device_resident": us(lap_times(c, f_fa, 50)),
+                               "numpy_to_numpy": host_us(lambda: backend.attention.flash_attention2(q, k, v, 8, 64, scale=0.125))}}
+    if check:
+        from oracle import oracle_np as O
+        y = c.download(dy, (32, 128)); g = c.download(dg, (32, 64)); o = c.download(do, q.shape)
+        yd = y.astype(np.float64)
+        e = [max_rel(y, O.truth_linear(x, Wt, b0)), max_rel(g, yd[:, :64] * (yd[:, 64:] / (1 + np.exp(-yd[:, 64:])))),
+             max_rel(o, O.truth_attention(q, k, v, scale=0.125))]
+        r0["max_rel_vs_float64"] = {"linear": float(f"{e[0]:.3g}"), "activation_swiglu": float(f"{e[1]:.3g}"), "flash_attention2": float(f"{e[2]:.3g}")}
+        r0["within_tolerance"] = bool(max(e) < TOL["fp32"])
+    for t in (dx, dw, db, dy, dg, dq, dk, dv, do):
+        t.free()
+    # configs[1]
+    cfg = MINILM_L6
+    w = random_bert_weights(cfg, seed=20260131 + 2)
+    rng = np.random.default_rng(20260131 + 2)
+    B, S = 64, 256
+    ids = rng.integers(0, cfg.vocab, (B, S))
+    lens = rng.integers(32, 257, B)
+    mask = (np.arange(S)[None] < lens[:, None]).astype(np.float32)
+    enc = BertEncoder(backend, cfg, w, dtype="fp32")
+    enc.set_inputs(ids, mask)
+    t = lap_times(c, lambda: enc.launch(pool=True), reps, warm=3)
+    flops = enc.flops_per_forward(B, S)
+    r1 = {"workload": "BASELINE configs[1]: MiniLM-L6-shaped encoder forward, 6 post-LN layers, d=384, 12x32 heads, FFN 1536 GELU, fp32, "
+                      "batch 64 x seq 256, lengths uniform in [32,256], embeddings + layers + masked mean pooling",
+          "median_ms": round(median(t), 4), "mean_ms": round(float(np.mean(t)), 4), "steps": len(t),
+          "tokens_per_s": round(B * S / median(t) * 1e3, 1), "real_tokens_per_s": round(float(lens.sum()) / median(t) * 1e3, 1),
+          "flops": flops, "tflops": round(flops / median(t) / 1e9, 1), "frac_mfma": round(flops / (median(t) * 1e-3) / PEAK_FP32, 4),
+          "peak": "fp32 MFMA 157.3 TFLOP/s (nominal FLOPs: padding counted)"}
+    if check:
+        from oracle import oracle_np as O
+        O.build()
+        C = O.COracle()
+        h = c.download(enc.x, (B, S, cfg.d_model))
+        worst = 0.0
+        for bi in (int(np.argmin(lens)), 17):
+            xr = C.layernorm(C.embed(ids[bi:bi + 1], w["tok_emb"], w["pos_emb"], w["type_emb"]), w["emb_ln_g"], w["emb_ln_b"], cfg.eps)
+            for lw in w["layers"]:
+                xr = C.bert_layer(xr, lw, mask[bi:bi + 1], cfg.heads, cfg.eps)
+            worst = max(worst, max_rel(h[bi:bi + 1], xr))
+        r1["max_rel_vs_cpu_port"] = float(f"{worst:.3g}"); r1["within_tolerance"] = bool(worst < TOL["fp32"])
+    enc.release_activations()
+    return r0, r1
+
+
+def mfma_ceiling(backend, iters=20000):
+    """What the matrix cores deliver under the board's power limit with nothing else going on: a register-resident loop
+    of MFMAs (grl_mfma_probe: eight waves per CU, the GEMM's 128 x 64 wave tile, no memory access in the loop) for both
+    bf16 instruction shapes, on all-zero operands and on N(0,1) x N(0,0.02) random ones, with the shader clock read
+    beside each run.  The fractions are of the published 2.5 PFLOP/s."""
+    import ctypes
+    from grilly_amd import _lib as L
+    c = backend.core
+    rng = np.random.default_rng(3)
+    blk = np.concatenate([rng.standard_normal(16384), rng.standard_normal(16384) * 0.02]).astype(np.float32)   # 32768 bf16 = 64 KiB
+    rnd = c.upload(rng.permutation(blk), L.GRL_BF16)
+    out = {}
+    for kind, name in ((0, "v_mfma_f32_32x32x16_bf16"), (1, "v_mfma_f32_16x16x32_bf16")):
+        for label, ptr in (("zero_operands", None), ("random_operands", rnd.ptr)):
+            ms, fl = ctypes.c_float(), ctypes.c_double()
+            L.check(c.lib.grl_mfma_probe(c.ctx, kind, ptr, iters, ctypes.byref(ms), ctypes.byref(fl)), "mfma_probe")
+            c.clock_probe_begin(max(0.7 * ms.value, 0.05))
+            ms2, fl2 = ctypes.c_float(), ctypes.c_double()
+            L.check(c.lib.grl_mfma_probe(c.ctx, kind, ptr, iters, ctypes.byref(ms2), ctypes.byref(fl2)), "mfma_probe")
+            ghz = c.clock_probe_end()
+            out.setdefault(name, {})[label] = {"ms": round(ms.value, 3), "tflops": round(fl.value / ms.value / 1e9, 1),
+                                               "frac_of_peak": round(fl.value / (ms.value * 1e-3) / PEAK_BF16, 4), "shader_clock_ghz": round(ghz, 3)}
+    rnd.free()
+    return out
+
+
 def cpu_baseline(cfg, weights, ids, nseq):
     """C restatement of the reference shaders on the host cores: the first `nseq` sequences of the workload
     (S=512 each) through embeddings + all layers.  tokens/s = nseq*512 / elapsed.  Returns the record and the
@@ -370,14 +556,18 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the fp32 forward and the two single-operator configurations")
-    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "kernels", "copy", "fa2_long", "swiglu_mlp", "prenorm_forward"],
+    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "kernels", "copy", "fa2_long", "swiglu_mlp", "prenorm_forward", "small", "mfma_ceiling"],
                     help="forward: the benchmark; gemm / copy: only launch the dominant GEMM kernel at its three "
                          "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs); kernels: every kernel of "
                          "the layer at its layer shape, nothing else (counter runs); fa2_long: "
                          "causal attention with RoPE at batch 4, 32 heads, seq 8192, head dim 128, bf16; swiglu_mlp: "
                          "X[16384,4096] through gate/up [11008,4096] + silu*up + down [4096,11008], bf16; prenorm_forward: the "
-                         "pre-norm / rotary / GeGLU encoder at the ModernBERT-base shape, batch 128 x seq 512, bf16")
+                         "pre-norm / rotary / GeGLU encoder at the ModernBERT-base shape, batch 128 x seq 512, bf16; small: the README "
+                         "operators (configs[0]) in microseconds and the MiniLM-shaped fp32 encoder (configs[1]); mfma_ceiling: "
+                         "register-resident MFMA loops, zero and random operands (what the power limit leaves of the matrix peak)")
     ap.add_argument("--cpu-sequences", type=int, default=12)
+    ap.add_argument("--unfused", action="store_true", help="run the seven-launch layer (two LayerNorm passes per layer) instead of the "
+                    "layer with both LayerNorms folded into its GEMMs")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one MI355X: this path has no multi-GPU leg (data-parallel sharding over "
@@ -400,19 +590,30 @@ def main():
                           "ms": round(ms, 4), "gbps": round(2 * nbytes / ms / 1e6, 1), "launches": a.kernel_reps + WARM}))
         backend.cleanup()
         return
+    if a.mode == "small":
+        r0, r1 = small_configs(backend, a.kernel_reps, check=not a.no_cpu_baseline)
+        print(json.dumps({"mode": "small", "readme_ops": r0, "minilm_forward": r1}))
+        backend.cleanup()
+        return
+    if a.mode == "mfma_ceiling":
+        print(json.dumps({"mode": "mfma_ceiling", "device": info, "peak_tflops": PEAK_BF16 / 1e12, "mfma_ceiling": mfma_ceiling(backend)}))
+        backend.cleanup()
+        return
     if a.mode in ("fa2_long", "swiglu_mlp", "prenorm_forward"):
         print(json.dumps(side_workload(backend, a.mode, seed, a.kernel_reps, check=not a.no_cpu_baseline)))
         backend.cleanup()
         return
     weights = random_bert_weights(cfg, seed=seed)
-    enc = BertEncoder(backend, cfg, weights, dtype=a.dtype)
+    enc = BertEncoder(backend, cfg, weights, dtype=a.dtype, fused=False if a.unfused else None)
     rng = np.random.default_rng(seed)
     B, S = a.batch, a.seq
     ids = rng.integers(0, cfg.vocab, (B, S))
     enc.set_inputs(ids, None)                 # no padding in this configuration
 
     if a.mode in ("gemm", "kernels"):
-        only = ("gemm_qkv", "gemm_out", "gemm_ffn2") if a.mode == "gemm" else None
+        only = None
+        if a.mode == "gemm":        # the launches of the dominant GEMM instantiation only (counter runs)
+            only = ("gemm_out_resln", "gemm_ffn2_resln") if enc.fused else ("gemm_qkv", "gemm_out", "gemm_ffn2")
         kt = kernel_table(backend, enc, B, S, a.kernel_reps, only=only, check=False)
         print(json.dumps({"mode": a.mode, "kernels": kt, "launches_each": a.kernel_reps + WARM}))
         backend.cleanup()
@@ -420,6 +621,8 @@ def main():
 
     wall, ev_ms = timed_forward(backend, enc, a.steps, a.warmup)
     ms_per_step = wall * 1e3 / a.steps
+    # the same steps once more with an event between every two of them: the median step next to the mean
+    step_ms = lap_times(backend.core, lambda: enc.launch(pool=True), a.steps, warm=0)
     # shader clock during the forward: probe beside three more (untimed) steps
     backend.core.clock_probe_begin(max(2.0 * ms_per_step, 0.05))
     for _ in range(3):
@@ -438,6 +641,7 @@ def main():
                                "12x64 heads, FFN 3072 GELU, fused QKV, no padding, random init N(0,0.02)",
                    "batch": B, "seq_len": S, "tokens_per_step": B * S, "flops_per_step": flops},
         "event_ms_per_step": round(ev_ms / a.steps, 3),
+        "median_ms_per_step": round(median(step_ms), 3), "median_steps": len(step_ms),
         "model_tflops": round(flops / (ms_per_step * 1e-3) / 1e12, 1),
         "model_frac_mfma": round(flops / (ms_per_step * 1e-3) / peak, 4),
         "shader_clock_ghz_during_forward": round(fwd_clock, 3),
@@ -449,27 +653,37 @@ def main():
     if not a.no_kernels:
         kt = kernel_table(backend, enc, B, S, a.kernel_reps, check=not a.no_cpu_baseline)
         out["kernels"] = kt
-        # dominant kernel = the plain (no activation) GEMM instantiation, launched three times per layer
-        # (QKV, out-proj, FFN2): average FLOPs per launch over average duration per launch
-        g = [kt[k] for k in ("gemm_qkv", "gemm_out", "gemm_ffn2")]
-        avg_flops = sum(r["flops"] for r in g) / 3
-        avg_ms = sum(r["ms"] for r in g) / 3
+        # dominant kernel = the GEMM instantiation with the largest share of the forward.  With the LayerNorms folded
+        # into the GEMMs that is the one whose epilogue adds the re-formed LayerNorm residual and reduces the row
+        # statistics (out-proj and FFN2: two launches per layer); in the seven-launch layer the plain instantiation
+        # (QKV, out-proj, FFN2: three launches per layer).  Average FLOPs per launch over average duration per launch.
+        fused = getattr(enc, "fused", False)
+        names = ("gemm_out_resln", "gemm_ffn2_resln") if fused else ("gemm_qkv", "gemm_out", "gemm_ffn2")
+        tname = "float" if a.dtype == "fp32" else "bf16"
+        kname = f"gemm_nt_dma_kernel<{tname},{tname},256,256,2,4,{'EPI_RESLN' if fused else 'EPI_NONE'}>"
+        g = [kt[k] for k in names]
+        avg_flops = sum(r["flops"] for r in g) / len(g)
+        avg_ms = sum(r["ms"] for r in g) / len(g)
+        clk = sum(r["shader_clock_ghz"] for r in g) / len(g)
         ach = avg_flops / (avg_ms * 1e-3) / 1e12
-        traffic, at_commit = gemm_traffic(a.dtype, B, S)
-        out["roofline"] = {"kernel": "gemm_nt_dma_kernel<bf16,bf16,256,256,2,4,EPI_NONE>" if a.dtype == "bf16" else "gemm_nt_dma_kernel<f32,f32,256,256,2,4,EPI_NONE>",
+        traffic, at_commit = gemm_traffic(a.dtype, B, S, kname)
+        out["roofline"] = {"kernel": kname, "launches": list(names),
                            "bound": "mfma", "achieved": round(ach, 1), "peak": peak / 1e12, "unit": "TFLOP/s",
                            "frac": round(ach * 1e12 / peak, 4),
                            "traffic": traffic, "traffic_measured_at_commit": at_commit,
-                           "algorithmic_bytes": sum(r["bytes"] for r in g) / 3,
-                           "avg_launch_ms": round(avg_ms, 4), "flops_per_launch": avg_flops,
-                           "shader_clock_ghz": round(sum(r["shader_clock_ghz"] for r in g) / 3, 3), "nominal_clock_ghz": NOMINAL_GHZ,
-                           "frac_at_measured_clock": round(ach * 1e12 / (peak * (sum(r["shader_clock_ghz"] for r in g) / 3) / NOMINAL_GHZ), 4),
-                           "launches_per_step": 3 * cfg.layers,
+                           "algorithmic_bytes": sum(r["bytes"] for r in g) / len(g),
+                           "avg_launch_ms": round(avg_ms, 4), "median_launch_ms": round(sum(r["median_ms"] for r in g) / len(g), 4),
+                           "flops_per_launch": avg_flops,
+                           "shader_clock_ghz": round(clk, 3), "nominal_clock_ghz": NOMINAL_GHZ,
+                           "frac_at_measured_clock": round(ach * 1e12 / (peak * clk / NOMINAL_GHZ), 4),
+                           "launches_per_step": len(names) * cfg.layers,
                            "clock_note": "peak = 256 CUs x 4 SIMDs x 1024 bf16 FLOP per cycle (fp32: 64) x the nominal 2.4 GHz; under the board's "
                                          "power limit the timed launches run at shader_clock_ghz (probe kernel beside them), and "
                                          "frac_at_measured_clock is the same achieved rate against the peak at that clock",
-                           "note": "launches timed back to back on the layer's real operands; inside the forward the same launches "
-                                   "run about 10 % longer (operands come from HBM): see profiles/encoder_forward_bert_base_bf16_kernel_stats.md"}
+                           "note": "launches timed back to back on the layer's real operands; per-kernel durations move by about +-10 % "
+                                   "with the power state of the board and differ by up to 20 % between boxes (the same launches inside "
+                                   "the forward, between other kernels, are not systematically slower or faster): see "
+                                   "profiles/encoder_forward_bert_base_bf16_kernel_stats.md"}
     extra = {}
     hidden32 = None
     if not a.no_extra and a.dtype == "bf16":
@@ -491,6 +705,9 @@ def main():
             r.pop("mode")
             extra[mode] = r
             backend.core.lib.grl_pool_trim(backend.core.ctx)
+        r0, r1 = small_configs(backend, 20, check=not a.no_cpu_baseline)
+        extra["readme_ops"], extra["minilm_forward"] = r0, r1
+        extra["mfma_ceiling"] = mfma_ceiling(backend)
         out["extra"] = extra
     if not a.no_cpu_baseline:
         rec, cpu_hidden = cpu_baseline(cfg, weights, ids, nseq)

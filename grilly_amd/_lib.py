@@ -36,6 +36,11 @@ class BertLayer(ctypes.Structure):
                                         "w_ff2", "b_ff2", "ln2_g", "ln2_b")]
 
 
+class BertLayerFused(ctypes.Structure):
+    _fields_ = [(n, c_void_p) for n in ("ws_qkv", "c_qkv", "bf_qkv", "in_g", "in_b", "w_o", "b_o", "ln1_g", "ln1_b",
+                                        "ws_ff1", "c_ff1", "bf_ff1", "w_ff2", "b_ff2")]
+
+
 # name -> (restype, argtypes); every symbol include/grilly_hip.h declares
 SIGNATURES = {
     "grl_create": (c_void_p, [c_int]),
@@ -54,6 +59,9 @@ SIGNATURES = {
     "grl_sync": (c_int, [c_void_p]),
     "grl_timer_start": (c_int, [c_void_p]),
     "grl_timer_stop": (c_int, [c_void_p, ctypes.POINTER(c_float)]),
+    "grl_timer_lap": (c_int, [c_void_p, c_int]),
+    "grl_timer_lap_ms": (c_int, [c_void_p, c_int, c_int, ctypes.POINTER(c_float)]),
+    "grl_mfma_probe": (c_int, [c_void_p, c_int, c_void_p, c_int, ctypes.POINTER(c_float), ctypes.POINTER(ctypes.c_double)]),
     "grl_clock_probe_begin": (c_int, [c_void_p, c_float]),
     "grl_clock_probe_end": (c_int, [c_void_p, ctypes.POINTER(c_float)]),
     "grl_cast": (c_int, [c_void_p, c_int, c_int, c_i64, c_void_p, c_void_p]),
@@ -72,6 +80,9 @@ SIGNATURES = {
     "grl_ln_stats": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_float, c_void_p]),
     "grl_ln_gemm_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 4 + [c_float, c_void_p, c_void_p]),
     "grl_ln_glu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 7 + [c_float, c_void_p, c_void_p, c_int]),
+    "grl_ln_gemm_nt_stats": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 6 + [c_int]),
+    "grl_gemm_nt_resln_workspace": (c_i64, [c_i64, c_i64]),
+    "grl_gemm_nt_resln": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 8 + [c_float, c_void_p, c_void_p]),
     "grl_layernorm": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p]),
     "grl_add": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p, c_void_p]),
     "grl_gelu": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p]),
@@ -86,6 +97,9 @@ SIGNATURES = {
                                     c_float, c_void_p]),
     "grl_mean_pool": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_int]),
     "grl_bert_layer_workspace": (c_i64, [c_int, c_i64, c_i64, c_i64, c_i64, c_i64]),
+    "grl_bert_layer_fused_workspace": (c_i64, [c_int, c_i64, c_i64, c_i64, c_i64, c_i64]),
+    "grl_bert_layer_fwd_fused": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_i64, ctypes.POINTER(BertLayerFused), c_void_p, c_float,
+                                 c_void_p, c_void_p, c_void_p]),
     "grl_bert_layer_fwd": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_i64, ctypes.POINTER(BertLayer), c_void_p, c_float, c_void_p, c_void_p]),
 }
 

@@ -11,10 +11,12 @@
 #include "../../include/grilly_hip.h"
 
 // ---------------------------------------------------------------- context
+#define GRL_MAX_LAPS 256
 struct grl_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipEvent_t laps[GRL_MAX_LAPS] = {};   // lap events (grl_timer_lap), created on first use
     hipDeviceProp_t prop{};
     std::mutex mu;          // guards the pool
     std::mutex timer_mu;    // guards the event pair

@@ -60,6 +60,7 @@ extern "C" void grl_destroy(grl_ctx* c) {
     for (auto& kv : c->live) hipFree(kv.first);
     hipEventDestroy(c->ev0);
     hipEventDestroy(c->ev1);
+    for (auto& e : c->laps) if (e) hipEventDestroy(e);
     if (c->probe_stream) { hipStreamSynchronize(c->probe_stream); hipStreamDestroy(c->probe_stream); }
     if (c->probe_out) hipFree(c->probe_out);
     hipStreamDestroy(c->stream);
@@ -217,6 +218,121 @@ extern "C" int grl_timer_stop(grl_ctx* c, float* ms) {
     GRL_CHECK_HIP(hipEventSynchronize(c->ev1));
     GRL_CHECK_HIP(hipEventElapsedTime(ms, c->ev0, c->ev1));
     return GRL_OK;
+}
+
+// ---- lap events: per-launch durations of a back-to-back sequence without a host synchronisation in between -----
+extern "C" int grl_timer_lap(grl_ctx* c, int index) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_timer_lap: null context");
+    GRL_REQUIRE(index >= 0 && index < GRL_MAX_LAPS, GRL_ERR_ARG, "grl_timer_lap: index %d outside 0..%d", index, GRL_MAX_LAPS - 1);
+    std::lock_guard<std::mutex> lk(c->timer_mu);
+    if (!c->laps[index]) {
+        GRL_CHECK_HIP(hipSetDevice(c->device));
+        GRL_CHECK_HIP(hipEventCreate(&c->laps[index]));
+    }
+    GRL_CHECK_HIP(hipEventRecord(c->laps[index], c->stream));
+    return GRL_OK;
+}
+extern "C" int grl_timer_lap_ms(grl_ctx* c, int from, int to, float* ms) {
+    GRL_REQUIRE(c && ms, GRL_ERR_ARG, "grl_timer_lap_ms: null argument");
+    GRL_REQUIRE(from >= 0 && from < GRL_MAX_LAPS && to >= 0 && to < GRL_MAX_LAPS, GRL_ERR_ARG, "grl_timer_lap_ms: index outside 0..%d", GRL_MAX_LAPS - 1);
+    std::lock_guard<std::mutex> lk(c->timer_mu);
+    GRL_REQUIRE(c->laps[from] && c->laps[to], GRL_ERR_ARG, "grl_timer_lap_ms: lap %d or %d was never recorded", from, to);
+    GRL_CHECK_HIP(hipEventSynchronize(c->laps[to]));
+    GRL_CHECK_HIP(hipEventElapsedTime(ms, c->laps[from], c->laps[to]));
+    return GRL_OK;
+}
+
+// ---- matrix-core ceiling probe ---------------------------------------------------------------------------------
+// Nothing but MFMAs on register-resident operands: eight waves per CU (two per SIMD, as in the GEMM kernels), each
+// with the GEMM wave tile's accumulators (128 registers) and two alternating sets of operand fragments, no memory
+// access inside the loop.  What this reaches is what the matrix cores deliver under the board's power limit for the
+// given operand bits (zeros, or the caller's data), i.e. the ceiling the GEMM and attention kernels work under.
+template <int KIND>
+__global__ __launch_bounds__(512) void mfma_probe_kernel(const u32x4* __restrict__ operands, float* __restrict__ sink, int iters) {
+    const int lane = threadIdx.x & 63;
+    constexpr int NA = KIND == 0 ? 4 : 8, NB = KIND == 0 ? 2 : 4;       // fragments of a 128 x 64 wave tile
+    u32x4 fa[2][NA], fb[2][NB];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int i = 0; i < NA; ++i) fa[s][i] = operands ? operands[((s * 12 + i) * 64 + lane) % 4096] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < NB; ++i) fb[s][i] = operands ? operands[((s * 12 + 8 + i) * 64 + lane) % 4096] : u32x4{0u, 0u, 0u, 0u};
+    }
+    if constexpr (KIND == 0) {
+        f32x16 acc[NA][NB];
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int a = 0; a < NA; ++a)
+#pragma unroll
+                    for (int b = 0; b < NB; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb[s][b]), __builtin_bit_cast(bf16x8, fa[s][a]), acc[a][b], 0, 0, 0);
+        }
+        float t = 0.f;
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) t += acc[a][b][r];
+        if (t == 12345.678f) sink[0] = t;          // keeps the accumulators alive; practically never true
+    } else {
+        f32x4 acc[NA][NB];
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int a = 0; a < NA; ++a)
+#pragma unroll
+                    for (int b = 0; b < NB; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fb[s][b]), __builtin_bit_cast(bf16x8, fa[s][a]), acc[a][b], 0, 0, 0);
+        }
+        float t = 0.f;
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) t += acc[a][b][r];
+        if (t == 12345.678f) sink[0] = t;
+    }
+}
+
+extern "C" int grl_mfma_probe(grl_ctx* c, int kind, const void* operands, int iters, float* ms, double* flops) {
+    GRL_REQUIRE(c && ms && flops, GRL_ERR_ARG, "grl_mfma_probe: null argument");
+    GRL_REQUIRE(kind == 0 || kind == 1, GRL_ERR_ARG, "grl_mfma_probe: kind must be 0 (32x32x16 bf16) or 1 (16x16x32 bf16)");
+    GRL_REQUIRE(iters > 0 && iters <= (1 << 20), GRL_ERR_ARG, "grl_mfma_probe: iters must be in 1..2^20");
+    GRL_REQUIRE((((uintptr_t)operands) & 15u) == 0, GRL_ERR_ARG, "grl_mfma_probe: operands must be 16-byte aligned (64 KiB of them, or NULL for zeros)");
+    float* sink = (float*)grl_malloc(c, 256);
+    if (!sink) return GRL_ERR_OOM;
+    const int cus = c->prop.multiProcessorCount;
+    auto launch = [&](int n) {
+        if (kind == 0) hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(cus), dim3(512), 0, c->stream, (const u32x4*)operands, sink, n);
+        else hipLaunchKernelGGL(mfma_probe_kernel<1>, dim3(cus), dim3(512), 0, c->stream, (const u32x4*)operands, sink, n);
+    };
+    launch(iters);                                   // warm-up: clocks and power settle
+    int rc = GRL_OK;
+    if (hipGetLastError() != hipSuccess) rc = GRL_ERR_HIP;
+    if (!rc) rc = grl_timer_start(c);
+    if (!rc) { launch(iters); if (hipGetLastError() != hipSuccess) rc = GRL_ERR_HIP; }
+    if (!rc) rc = grl_timer_stop(c, ms);
+    grl_free(c, sink);
+    if (rc == GRL_ERR_HIP) grl_set_error("grl_mfma_probe: launch failed");
+    // per iteration and wave: 2 fragment sets x a 128 x 64 wave tile x 16 (32) deep = 2 x 128*64*2*16 flops (kind 0), x 32 (kind 1)
+    *flops = (double)iters * 2.0 * 128.0 * 64.0 * 2.0 * (kind == 0 ? 16.0 : 32.0) * 8.0 * cus;
+    return rc;
 }
 
 // ---- shader-clock probe ---------------------------------------------------------------------------------------

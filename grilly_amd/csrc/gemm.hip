@@ -151,6 +151,78 @@ extern "C" int grl_ln_gemm_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M
     return dispatch_types_ln(c, a, in_dtype, out_dtype, EPI_NONE);
 }
 
+// the same with the row statistics given (computed earlier, e.g. by the GEMM that produced x) and a choice of epilogue
+extern "C" int grl_ln_gemm_nt_stats(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                                    const void* W_scaled, const float* colsum, const float* bias_folded,
+                                    const float* stats, void* out, int epilogue) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_ln_gemm_nt_stats: null context");
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_ln_gemm_nt_stats: bad dtype");
+    GRL_REQUIRE(epilogue == GRL_EPI_NONE || epilogue == GRL_EPI_GELU, GRL_ERR_ARG,
+                "grl_ln_gemm_nt_stats: epilogue must be GRL_EPI_NONE or GRL_EPI_GELU (got %d)", epilogue);
+    int rc = check_dims("grl_ln_gemm_nt_stats", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    GRL_REQUIRE(out && K > 0 && x && W_scaled && colsum && bias_folded && stats, GRL_ERR_ARG, "grl_ln_gemm_nt_stats: null argument or K == 0");
+    GemmArgs a{};
+    a.A = x; a.W = W_scaled; a.bias = bias_folded; a.C = out;
+    a.ln_stats = stats; a.ln_c = colsum;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.act = epilogue;
+    return dispatch_types_ln(c, a, in_dtype, out_dtype, epilogue == GRL_EPI_GELU ? EPI_GELU : EPI_NONE);
+}
+
+// ---- C = A.W^T + bias + LayerNorm(R), and the row statistics of C ------------------------------------------------
+extern template int launch_gemm_resln<float, float>(grl_ctx*, GemmArgs&, int*);
+extern template int launch_gemm_resln<uint16_t, uint16_t>(grl_ctx*, GemmArgs&, int*);
+
+// per row: the per-tile partials {sum, sum of squares} merged in a fixed order into {1/sd, mean/sd} (var = E[x^2] - mean^2
+// in float: rows whose mean is more than about a hundred spreads away from zero lose the variance to cancellation,
+// the same conditioning as the folded LayerNorm that consumes the statistics)
+__global__ __launch_bounds__(256) void ln_stats_merge_kernel(const float* __restrict__ part, float* __restrict__ stats, int M, int N,
+                                                             int nparts, float eps) {
+    const int m = blockIdx.x * 256 + threadIdx.x;
+    if (m >= M) return;
+    float tot = 0.f, sq = 0.f;
+    for (int t = 0; t < nparts; ++t) {
+        const float2 pr = *(const float2*)(part + ((int64_t)t * M + m) * 2);
+        tot += pr.x; sq += pr.y;
+    }
+    const float mean = tot / (float)N;
+    const float var = fmaxf(sq / (float)N - mean * mean, 0.f);
+    const float sd = sqrtf(var + eps);
+    *(float2*)(stats + 2 * (int64_t)m) = make_float2(1.0f / sd, mean / sd);
+}
+
+extern "C" int64_t grl_gemm_nt_resln_workspace(int64_t M, int64_t N) {
+    if (M < 0 || N < 0) return -1;
+    return ((N + 127) / 128) * M * 8 + 256;          // one {sum, sum of squares} pair per row and 128-column tile (the narrowest tile)
+}
+
+extern "C" int grl_gemm_nt_resln(grl_ctx* c, int dtype, int64_t M, int64_t N, int64_t K, const void* A, const void* W,
+                                 const float* bias, const void* R, const float* r_stats, const float* r_gamma,
+                                 const float* r_beta, void* C, float eps, float* stats_out, void* workspace) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_gemm_nt_resln: null context");
+    GRL_REQUIRE(grl_valid_dtype(dtype), GRL_ERR_ARG, "grl_gemm_nt_resln: bad dtype");
+    int rc = check_dims("grl_gemm_nt_resln", M, N, K);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return GRL_OK;
+    GRL_REQUIRE(A && W && R && r_stats && r_gamma && r_beta && C && stats_out && workspace && K > 0, GRL_ERR_ARG,
+                "grl_gemm_nt_resln: null argument or K == 0");
+    GRL_REQUIRE((((uintptr_t)workspace) & 15u) == 0 && (((uintptr_t)stats_out) & 15u) == 0, GRL_ERR_ARG, "grl_gemm_nt_resln: workspace and stats_out must be 16-byte aligned");
+    GemmArgs a{};
+    a.A = A; a.W = W; a.bias = bias; a.C = C; a.residual = R;
+    a.res_stats = r_stats; a.res_gamma = r_gamma; a.res_beta = r_beta; a.part_out = (float*)workspace;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    int tile_cols = 0;
+    rc = dtype == GRL_F32 ? launch_gemm_resln<float, float>(c, a, &tile_cols) : launch_gemm_resln<uint16_t, uint16_t>(c, a, &tile_cols);
+    if (rc) return rc;
+    const int nparts = (int)((N + tile_cols - 1) / tile_cols);
+    hipLaunchKernelGGL(ln_stats_merge_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, c->stream, (const float*)workspace, stats_out,
+                       (int)M, (int)N, nparts, eps);
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
 extern "C" int grl_ln_glu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
                              const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
                              const float* bias_gate_folded, const float* bias_up_folded, float eps, float* stats,

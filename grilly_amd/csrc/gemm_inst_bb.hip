@@ -3,3 +3,4 @@
 
 template int dispatch_epi<uint16_t, uint16_t>(grl_ctx*, GemmArgs&, int);
 template int dispatch_epi_ln<uint16_t, uint16_t>(grl_ctx*, GemmArgs&, int);
+template int launch_gemm_resln<uint16_t, uint16_t>(grl_ctx*, GemmArgs&, int*);

@@ -47,13 +47,21 @@ struct GemmArgs {
     const float* ln_stats; // (M,2): {rstd, rstd*mean} per row
     const float* ln_c;     // (N) column sums of the scaled weight W
     const float* ln_c2;    // (N) the same for W2, else null
+    // EPI_RESLN: the residual is LayerNorm(residual) re-formed from the raw rows in `residual`, their statistics and
+    // the norm's parameters; the row statistics of the OUTPUT leave the kernel as one partial per (column tile, row)
+    const float* res_stats;  // (M,2): {rstd, rstd*mean} of the residual rows
+    const float* res_gamma;  // (N)
+    const float* res_beta;   // (N)
+    float* part_out;         // (tiles_n, M, 2): {sum, sum of squares} of each output row's columns in that tile
 };
 
 // Epilogue template codes.  NONE / GELU / SILU are compiled in (the encoder's hot shapes); EPI_RT picks
 // ReLU / GCU / RoSwish from GemmArgs::act at run time (one more instantiation instead of three), and the
 // dual-weight epilogue EPI_GLU picks the gate activation (SiLU / ReLU / GELU) the same way.
 // EPI_RES adds a residual tensor of the output type where the result is stored (C may be the residual itself).
-enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_RT = 3, EPI_GLU = 4, EPI_RES = 5 };
+// EPI_RESLN adds LayerNorm(residual) formed on the fly (GemmArgs::res_*) and writes per-tile row statistics of the
+// result; only the direct-to-LDS kernels with the LDS-staged epilogue implement it (the host checks).
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_RT = 3, EPI_GLU = 4, EPI_RES = 5, EPI_RESLN = 6 };
 
 // shaders/fused-linear-relu.glsl:63, fused-linear-gcu.glsl:44-46 (x*cos(x)), fused-linear-roswish.glsl:46-58
 // ((x+alpha)*sigmoid(beta*x) - alpha/2; the shader's sign-split sigmoid equals 1/(1+exp(-beta*x)) with the
@@ -109,6 +117,50 @@ template <> struct MfmaSlab<float> {      // fp32: 16 B = 4 values, each feeds o
     }
 };
 
+// ---- acc[m,n] += xs[m] * ws[n] on the matrix cores (one extra k-slab with register-built operands): the term
+// -mean_m * c[n] of the LayerNorm-folded GEMM.  bf16: each factor is split into three bf16 numbers (hi + mid + lo, exact
+// to 2^-24) and the nine cross products sit at k = 0..8 of one 32x32x16 instruction (k = 8*(lane/32) + e);
+// fp32: one 32x32x2 instruction with the factors at k = 0.
+// (conversions through v_cvt_pk_bf16_f32; the value sits in both halves of the returned words)
+__device__ __forceinline__ void split3_bf16(float v, uint32_t& hh, uint32_t& mm, uint32_t& ll) {
+    hh = pack_bf16x2(v, v);
+    const float r1 = v - bf16hi(hh);
+    mm = pack_bf16x2(r1, r1);
+    const float r2 = r1 - bf16hi(mm);
+    ll = pack_bf16x2(r2, r2);
+}
+__device__ __forceinline__ uint32_t lo_hi(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060100u); }   // low half of a | high half of b
+template <typename T> struct MfmaOuter;
+template <> struct MfmaOuter<uint16_t> {
+    // activation-row side (MFMA "B" operand): [h,h,h,m,m,m,l,l | l,0,...]
+    static __device__ __forceinline__ u32x4 xfrag(float v, int lg) {
+        uint32_t h, m, l;
+        split3_bf16(v, h, m, l);
+        const u32x4 lo = {h, lo_hi(h, m), m, l};
+        const u32x4 hi = {l & 0xffffu, 0u, 0u, 0u};
+        return lg ? hi : lo;
+    }
+    // weight-row side (MFMA "A" operand): [h,m,l,h,m,l,h,m | l,0,...]
+    static __device__ __forceinline__ u32x4 wfrag(float v, int lg) {
+        uint32_t h, m, l;
+        split3_bf16(v, h, m, l);
+        const uint32_t hm = lo_hi(h, m);
+        const u32x4 lo = {hm, lo_hi(l, h), lo_hi(m, l), hm};
+        const u32x4 hi = {l & 0xffffu, 0u, 0u, 0u};
+        return lg ? hi : lo;
+    }
+    static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), acc, 0, 0, 0);
+    }
+};
+template <> struct MfmaOuter<float> {
+    static __device__ __forceinline__ u32x4 xfrag(float v, int lg) { return u32x4{lg ? 0u : f2u(v), 0u, 0u, 0u}; }
+    static __device__ __forceinline__ u32x4 wfrag(float v, int lg) { return u32x4{lg ? 0u : f2u(v), 0u, 0u, 0u}; }
+    static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u2f(w[0]), u2f(x[0]), acc, 0, 0, 0);
+    }
+};
+
 // compile-time loop: f(std::integral_constant<int, 0..N-1>)
 template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
     if constexpr (N > 0) {
@@ -155,6 +207,27 @@ template <> __device__ __forceinline__ u32x4 add_chunk<uint16_t>(u32x4 c, u32x4 
     }
     return o;
 }
+
+// one 16-byte chunk of outputs <-> its 8 (bf16) or 4 (fp32) values
+template <typename OutT> struct Chunk;
+template <> struct Chunk<float> {
+    static constexpr int N = 4;
+    static __device__ __forceinline__ void unpack(const u32x4& c, float (&v)[4]) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = u2f(c[e]);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&v)[4]) { return u32x4{f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])}; }
+};
+template <> struct Chunk<uint16_t> {
+    static constexpr int N = 8;
+    static __device__ __forceinline__ void unpack(const u32x4& c, float (&v)[8]) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { const uint32_t w = c[e]; v[2 * e] = bf16lo(w); v[2 * e + 1] = bf16hi(w); }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
+        return u32x4{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])};
+    }
+};
 
 // ---- direct epilogue: lane (li, lg) holds, for output row m = .. + li, the columns
 // n = .. + 8*q + 4*lg + {0..3} in accumulator registers 4q..4q+3 and stores them itself
@@ -253,7 +326,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
     constexpr int STAGE = (BM + BN) * 128;
     __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // the wave index is wave-uniform; telling the compiler so keeps everything derived from it (LDS stage addresses of
+    // the transfers, the wave's tile coordinates, the branch that picks the requesting wave) in scalar registers
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const int li = lane & 31, lg = lane >> 5;
 
@@ -410,11 +485,15 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     // one tile's per-column vectors, fp32: bias slice(s); with LN also the column sums c (c2) behind them and the
     // tile's BM row-statistics pairs
     constexpr int COLB = BN * 4;
-    constexpr int BIASB = LN ? 2 * COLB + BM * 8 : COLB;
+    constexpr bool RL = EPI == EPI_RESLN;                   // LayerNorm(residual) formed in the epilogue + row statistics out
+    static_assert(!(LN && RL) && !(RL && DUAL), "one set of row statistics per tile");
+    constexpr int BIASB = (LN || RL) ? 2 * COLB + BM * 8 : COLB;
     static_assert(!LN || NW >= 4, "the per-tile vectors are fetched by distinct waves");
     __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + 2 * BIASB];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // the wave index is wave-uniform; telling the compiler so keeps everything derived from it (LDS stage addresses of
+    // the transfers, the wave's tile coordinates, the branch that picks the requesting wave) in scalar registers
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const int li = lane & 31, lg = lane >> 5;
     const int ntiles = p.tiles_m * p.tiles_n;
@@ -502,14 +581,15 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
     };
     // rows m0t .. m0t+BM of the statistics (rows past M read zero), fetched by the last wave
     auto issue_stats = [&](int m0t, int buf) {
-        if constexpr (LN) {
+        if constexpr (LN || RL) {
             if (wave == NW - 1) {
                 int left = (p.M - m0t) * 8;
-                __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)(p.ln_stats + 2 * (int64_t)m0t), 0, left > 0 ? left : 0, 0x00020000);
+                const float* sbase = LN ? p.ln_stats : p.res_stats;
+                __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)(sbase + 2 * (int64_t)m0t), 0, left > 0 ? left : 0, 0x00020000);
 #pragma unroll
                 for (int j = 0; j < BM * 8 / 1024; ++j)
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + 2 * STAGE + buf * BIASB + 2 * COLB + j * 1024),
-                                                             16, j * 1024 + lane * 16, 0, 0, 0);
+                                                             16, lane * 16, j * 1024, 0, 0);      // one per-lane offset for every transfer of the tile's vectors
             }
         }
     };
@@ -567,14 +647,17 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                 }
             }
             const char* s = lds + (kt & 1) * STAGE;
-#pragma unroll
-            for (int sl = 0; sl < 4; ++sl) {
+#ifndef GRL_KLOOP
+#define GRL_KLOOP 2
+#endif
+            auto load_frags = [&](int sl, u32x4 (&xf)[TM], u32x4 (&wf)[TN]) {
                 const int ch = 2 * sl + lg;
-                u32x4 xf[TM], wf[TN];
 #pragma unroll
                 for (int a = 0; a < TM; ++a) xf[a] = *(const u32x4*)(s + rowX[a] * 128 + ((ch ^ lds_swz<8>(rowX[a])) << 4));
 #pragma unroll
                 for (int b = 0; b < TN; ++b) wf[b] = *(const u32x4*)(s + BM * 128 + rowW[b] * 128 + ((ch ^ lds_swz<8>(rowW[b])) << 4));
+            };
+            auto run_mfmas = [&](int sl, const u32x4 (&xf)[TM], const u32x4 (&wf)[TN]) {
                 static_for<TM>([&](auto ia) {
                     static_for<TN>([&](auto ib) {
                         constexpr int a = decltype(ia)::value, b = decltype(ib)::value;
@@ -585,19 +668,74 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                         MfmaSlab<T>::run(wf[b], xf[a], acc[a][b]);
                     });
                 });
+            };
+            if constexpr (GRL_KLOOP == 2) {
+                // two fragment sets: the reads of the next 16-deep step are issued in front of this step's MFMAs
+                u32x4 xf[2][TM], wf[2][TN];
+                load_frags(0, xf[0], wf[0]);
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) {
+                    if (sl + 1 < 4) load_frags(sl + 1, xf[(sl + 1) & 1], wf[(sl + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    run_mfmas(sl, xf[sl & 1], wf[sl & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) {
+                    u32x4 xf[TM], wf[TN];
+                    load_frags(sl, xf, wf);
+                    // The kernels whose epilogues need more registers make the scheduler shrink this loop's fragment set to
+                    // one activation fragment at a time (a wait in front of every second MFMA); the fence keeps the six
+                    // reads of a 16-deep step together in front of its eight MFMAs, as in the other kernels.
+                    if constexpr (LN || RL || GRL_KLOOP == 1) __builtin_amdgcn_sched_barrier(0);
+                    run_mfmas(sl, xf, wf);
+                }
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();
         };
-        k_slab(0, std::true_type{});              // the host never launches this kernel with K == 0
+        if (LN && staged) {
+            // Folded LayerNorm: sum_k LN(x)[m,k] W0[n,k] = rstd_m * (acc[m,n] - mean_m * c[n]) + b'[n].  The outer product
+            // -mean_m * c[n] is what the accumulators start from: one MFMA per 32x32 block whose operands are built from
+            // the tile's row statistics and column sums (they arrived in LDS with the first slab).  What is left for
+            // the epilogue is one multiply-add per element, the instruction count of the plain bias add.
+            if constexpr (LN) {
+                const char* bl = lds + 2 * STAGE + bbuf * BIASB;
+                const float* stl = (const float*)(bl + 2 * COLB);
+                const float* cl = (const float*)(bl + COLB);
+                u32x4 xm[TM], wc[TN];
+#pragma unroll
+                for (int a = 0; a < TM; ++a) {
+                    const float rs = stl[2 * rowX[a]], rsm = stl[2 * rowX[a] + 1];
+                    // -mean = -(mean/sd) / (1/sd); rows past M carry zero statistics (0 * 1/0 = NaN in rows that are never stored)
+                    xm[a] = MfmaOuter<T>::xfrag(-rsm * __builtin_amdgcn_rcpf(rs), lg);
+                }
+#pragma unroll
+                for (int b = 0; b < TN; ++b) wc[b] = MfmaOuter<T>::wfrag(cl[rowW[b]], lg);
+                static_for<TM>([&](auto ia) {
+                    static_for<TN>([&](auto ib) {
+                        constexpr int a = decltype(ia)::value, b = decltype(ib)::value;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+                        MfmaOuter<T>::run(wc[b], xm[a], acc[a][b]);
+                    });
+                });
+            }
+            k_slab(0, std::false_type{});
+        } else {
+            k_slab(0, std::true_type{});          // the host never launches this kernel with K == 0
+        }
         for (int kt = 1; kt < KT; ++kt) k_slab(kt, std::false_type{});
 
         // both LDS stages are free now: request the next tile's first slab into stage 0
-        if (has_next) {
-            issue(rsAn, rsWn, 0);
-            issue_bias(n0n, bbuf ^ 1);
-            issue_stats(m0n, bbuf ^ 1);
-        }
+        auto issue_next = [&]() {
+            if (has_next) {
+                issue(rsAn, rsWn, 0);
+                issue_bias(n0n, bbuf ^ 1);
+                issue_stats(m0n, bbuf ^ 1);
+            }
+        };
 
         if (staged) {
             // ---- LDS-staged epilogue in stage 1, one 32-row band of every wave-row per pass
@@ -605,10 +743,11 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             char* stg = lds + STAGE;
             const char* bias_lds = lds + 2 * STAGE + bbuf * BIASB;
             // bias of this lane's 4-column groups, once per tile (columns past N hold zero)
-            // (with the folded LayerNorm every per-column vector is read from LDS where it is used instead: the
-            // epilogue then keeps nothing more in registers across its bands than the plain one)
-            f32x4 bv1[LN ? 1 : TNO][4], bv2[LN ? 1 : TNO][4];
-            if constexpr (!LN) {
+            // (the dual-weight kernel with the folded LayerNorm reads them from LDS where they are used instead: two bias
+            // sets in registers next to its two accumulator sets and the row factor do not fit)
+            constexpr bool BREG = !(LN && DUAL);
+            f32x4 bv1[BREG ? TNO : 1][4], bv2[BREG ? TNO : 1][4];
+            if constexpr (BREG) {
 #pragma unroll
                 for (int b = 0; b < TNO; ++b)
 #pragma unroll
@@ -617,6 +756,13 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                         bv1[b][q] = p.bias ? *(const f32x4*)(bias_lds + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
                         if (DUAL) bv2[b][q] = p.bias2 ? *(const f32x4*)(bias_lds + BNO * 4 + nl * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
                     }
+            }
+            // LN: 1/sd of this lane's row in each of the TM bands, read up front (a read inside the band loop would make the
+            // loop wait for the staged rows that are on their way back from LDS at that point)
+            float rsv[LN ? TM : 1];
+            if constexpr (LN) {
+#pragma unroll
+                for (int a = 0; a < TM; ++a) rsv[a] = ((const float*)(bias_lds + 2 * COLB))[2 * (wm * WM + a * 32 + li)];
             }
             constexpr int TOTAL = WGM * 32 * CPR;
             static_assert(TOTAL % NT == 0, "staged chunks divide over the threads");
@@ -628,40 +774,29 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             auto stage_band = [&](auto ia) {
                 constexpr int a = decltype(ia)::value;
                 char* crow = stg + (NREG == 2 ? (a & 1) * RG : 0) + r_w * CROWB;
-                // LN: this row's {rstd, rstd*mean} once per band, the column sums from LDS where they are used:
-                // nothing more stays live across the bands than without the folded LayerNorm
-                float rs = 1.f, rsm = 0.f;
-                if constexpr (LN) {
-                    const float* st = (const float*)(bias_lds + 2 * COLB) + 2 * (wm * WM + a * 32 + li);
-                    rs = st[0]; rsm = st[1];
-                }
+                const float rs = LN ? rsv[LN ? a : 0] : 1.f;
                 static_for<TNO>([&](auto ib) {
                     constexpr int b = decltype(ib)::value;
                     static_for<4>([&](auto iq) {
                         constexpr int q = decltype(iq)::value;
                         const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
                         float v[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] + (LN ? 0.f : bv1[LN ? 0 : b][q][e]);
-                        f32x4 c2 = {0.f, 0.f, 0.f, 0.f}, b2 = {0.f, 0.f, 0.f, 0.f};
-                        if constexpr (LN) {
-                            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-                            const f32x4 c1 = *(const f32x4*)(bias_lds + COLB + nl * 4);
-                            const f32x4 b1 = p.bias ? *(const f32x4*)(bias_lds + nl * 4) : zero;
-                            if constexpr (DUAL) {
-                                c2 = *(const f32x4*)(bias_lds + COLB + BNO * 4 + nl * 4);
-                                b2 = p.bias2 ? *(const f32x4*)(bias_lds + BNO * 4 + nl * 4) : zero;
-                            }
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = acc[a][b][4 * q + e] * rs + (b1[e] - rsm * c1[e]);
+                        f32x4 b1, b2 = {0.f, 0.f, 0.f, 0.f};
+                        if constexpr (BREG) {
+                            b1 = bv1[BREG ? b : 0][q];
+                            if (DUAL) b2 = bv2[BREG ? b : 0][q];
+                        } else {
+                            b1 = *(const f32x4*)(bias_lds + nl * 4);            // the folded biases always exist
+                            b2 = *(const f32x4*)(bias_lds + BNO * 4 + nl * 4);
                         }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = LN ? acc[a][b][4 * q + e] * rs + b1[e] : acc[a][b][4 * q + e] + b1[e];
                         if (DUAL) {
                             float up[4];
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
                                 up[e] = acc[a][DUAL ? b + TNO : b][4 * q + e];
-                                if constexpr (LN) up[e] = up[e] * rs + (b2[e] - rsm * c2[e]);
-                                else up[e] += bv2[LN ? 0 : b][q][e];
+                                up[e] = LN ? up[e] * rs + b2[e] : up[e] + b2[e];
                             }
                             glu_apply4(v, up, p);
                         } else {
@@ -688,9 +823,71 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             };
             // EPI_RES: this thread's residual chunks of band a, requested while the band is still on its way
             // through LDS (chunks outside the matrix are not read)
+            // EPI_RESLN: this thread's columns are the same in every chunk it handles (the chunk index advances by a
+            // multiple of the chunks per row), so the norm's gamma / beta for them are loaded once per tile
+            static_assert(NT % CPR == 0, "a thread keeps its chunk column");
+            float gq[RL ? EPCO : 1], bq[RL ? EPCO : 1];
+            if constexpr (RL) {
+                const int nq = n0 + (tid % CPR) * EPCO;          // N is a multiple of the chunk here: whole chunks in or out
+#pragma unroll
+                for (int e = 0; e < EPCO; e += 4) {
+                    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                    const f32x4 gv = nq + e < p.N ? *(const f32x4*)(p.res_gamma + nq + e) : zero;
+                    const f32x4 bv = nq + e < p.N ? *(const f32x4*)(p.res_beta + nq + e) : zero;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) { gq[e + k] = gv[k]; bq[e + k] = bv[k]; }
+                }
+            }
+            // last step of a staged chunk: residual (plain, or LayerNorm re-formed from the raw residual rows and
+            // their statistics in LDS), the tile's share of the output row statistics, and the global store.
+            // Called by every lane for the same (a, i): the row reduction runs over the CPR lanes that hold one row.
+            auto fetch_rstats = [&](auto ia, f32x2_t (&rst)[PER]) {
+                constexpr int a = decltype(ia)::value;
+                if constexpr (RL) {
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) {
+                        const int r = (tid + i * NT) / CPR;
+                        rst[i] = *(const f32x2_t*)(bias_lds + 2 * COLB + 8 * ((r >> 5) * WM + a * 32 + (r & 31)));
+                    }
+                }
+            };
+            auto emit = [&](auto ia, int i, u32x4 out, u32x4 rres, f32x2_t rstat) {
+                constexpr int a = decltype(ia)::value;
+                const int id = tid + i * NT;
+                const int r = id / CPR, cc = id % CPR;
+                const int rt = (r >> 5) * WM + a * 32 + (r & 31);
+                const int m = m0 + rt;
+                const int n = n0 + cc * EPCO;
+                const bool in = m < p.M && n < p.N;
+                if constexpr (EPI == EPI_RES) out = add_chunk<OutT>(out, rres);
+                if constexpr (RL) {
+                    const float rs = rstat[0], rsm = rstat[1];
+                    float xr[EPCO], g[EPCO], o[EPCO];
+                    Chunk<OutT>::unpack(rres, xr);
+                    Chunk<OutT>::unpack(out, g);
+                    // sum and sum of squares of the row's columns in this tile (columns past N contribute 0: gamma, beta,
+                    // bias and the products are 0 there); the two reductions are independent and interleave
+                    float sum = 0.f, sq = 0.f;
+#pragma unroll
+                    for (int e = 0; e < EPCO; ++e) {
+                        o[e] = fmaf(fmaf(xr[e], rs, -rsm), gq[e], bq[e] + g[e]);
+                        sum += o[e];
+                        sq = fmaf(o[e], o[e], sq);
+                    }
+                    sum = group_sum<CPR>(sum);
+                    sq = group_sum<CPR>(sq);
+                    out = Chunk<OutT>::pack(o);
+                    if (cc == 0 && m < p.M) {
+                        const f32x2_t pr = {sum, sq};
+                        *(f32x2_t*)(p.part_out + ((int64_t)(n0 / BNO) * p.M + m) * 2) = pr;
+                    }
+                }
+                // written once, read by another kernel: keep it from displacing the operand panels in L2
+                if (in) __builtin_nontemporal_store(out, (u32x4*)(C + (int64_t)m * p.N + n));
+            };
             auto fetch_res = [&](auto ia, u32x4 (&res)[PER]) {
                 constexpr int a = decltype(ia)::value;
-                if constexpr (EPI == EPI_RES) {
+                if constexpr (EPI == EPI_RES || RL) {
 #pragma unroll
                     for (int i = 0; i < PER; ++i) {
                         const int id = tid + i * NT;
@@ -702,41 +899,37 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                     }
                 }
             };
-            auto store_band = [&](auto ia, const u32x4 (&val)[PER], const u32x4 (&res)[PER]) {
-                constexpr int a = decltype(ia)::value;
+            auto store_band = [&](auto ia, const u32x4 (&val)[PER], const u32x4 (&res)[PER], const f32x2_t (&rst)[PER]) {
 #pragma unroll
-                for (int i = 0; i < PER; ++i) {
-                    const int id = tid + i * NT;
-                    const int r = id / CPR, cc = id % CPR;
-                    const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
-                    const int n = n0 + cc * EPCO;
-                    u32x4 out = val[i];
-                    if constexpr (EPI == EPI_RES) out = add_chunk<OutT>(out, res[i]);
-                    // written once, read by another kernel: keep it from displacing the operand panels in L2
-                    if (m < p.M && n < p.N) __builtin_nontemporal_store(out, (u32x4*)(C + (int64_t)m * p.N + n));
-                }
+                for (int i = 0; i < PER; ++i) emit(ia, i, val[i], res[i], rst[i]);
             };
             // Barriers here are LDS-only (a fence would also wait for the global stores of earlier bands).
             if constexpr (NREG == 2) {
                 // two regions: band a+1 is converted and written while band a's staged rows are on their
                 // way back from LDS, one barrier per band
+                issue_next();
                 stage_band(std::integral_constant<int, 0>{});
                 static_for<TM>([&](auto ia) {
                     constexpr int a = decltype(ia)::value;
                     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
                     u32x4 val[PER], res[PER];
+                    f32x2_t rst[PER];
                     fetch_band(ia, val);
+                    fetch_rstats(ia, rst);
                     fetch_res(ia, res);
                     if constexpr (a + 1 < TM) stage_band(std::integral_constant<int, a + 1>{});
-                    store_band(ia, val, res);
+                    store_band(ia, val, res, rst);
                 });
             } else {
+                issue_next();
                 static_for<TM>([&](auto ia) {
                     stage_band(ia);
                     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
                     u32x4 val[PER];
+                    f32x2_t rst[PER];
                     fetch_band(ia, val);
-                    if constexpr (EPI == EPI_RES) {
+                    fetch_rstats(ia, rst);
+                    if constexpr (EPI == EPI_RES || RL) {
                         // residual chunks in two halves: a whole band of them next to the staged values and
                         // the other band's accumulators does not fit the register file
                         constexpr int a = decltype(ia)::value;
@@ -756,22 +949,17 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                                 if (in[j]) rr[j] = __builtin_nontemporal_load((const u32x4*)((const OutT*)p.residual + (int64_t)m * p.N + n));
                             }
 #pragma unroll
-                            for (int j = 0; j < HP; ++j) {
-                                const int id = tid + (h * HP + j) * NT;
-                                const int r = id / CPR, cc = id % CPR;
-                                const int m = m0 + (r >> 5) * WM + a * 32 + (r & 31);
-                                const int n = n0 + cc * EPCO;
-                                if (in[j]) __builtin_nontemporal_store(add_chunk<OutT>(val[h * HP + j], rr[j]), (u32x4*)(C + (int64_t)m * p.N + n));
-                            }
+                            for (int j = 0; j < HP; ++j) emit(ia, h * HP + j, val[h * HP + j], rr[j], rst[h * HP + j]);
                         }
                     } else {
                         u32x4 res[PER];
-                        store_band(ia, val, res);
+                        store_band(ia, val, res, rst);
                     }
                     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
                 });
             }
-        } else {
+        } else if constexpr (!RL) {        // EPI_RESLN exists in the staged form only: the host launches it for nothing else
+            issue_next();
             epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL, LN>(acc, p, m0, n0, wm, wn, li, lg);
         }
         if (!has_next) break;
@@ -862,6 +1050,35 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     return GRL_OK;
 }
 
+// EPI_RESLN: only the direct-to-LDS kernels with their LDS-staged epilogue implement it, so the problem must be one
+// they take (whole 128-byte K slabs, 16-byte aligned operands, output rows a multiple of 16 bytes).  *tile_cols
+// returns the column width of the tiles, i.e. of the row-statistics partials the kernel writes.
+template <typename T, typename OutT>
+int launch_gemm_resln(grl_ctx* c, GemmArgs& a, int* tile_cols) {
+    const int64_t bke = 128 / (int64_t)sizeof(T);
+    const bool aligned = ((((uintptr_t)a.A) | ((uintptr_t)a.W) | ((uintptr_t)a.C) | ((uintptr_t)a.bias) | ((uintptr_t)a.residual) |
+                           ((uintptr_t)a.res_stats) | ((uintptr_t)a.res_gamma) | ((uintptr_t)a.res_beta) | ((uintptr_t)a.part_out)) & 15u) == 0;
+    GRL_REQUIRE(aligned && a.K % bke == 0 && ((int64_t)a.N * (int64_t)sizeof(OutT)) % 16 == 0, GRL_ERR_SHAPE,
+                "gemm (LayerNorm residual): needs 16-byte aligned operands, K a multiple of %lld and output rows a multiple of 16 bytes",
+                (long long)bke);
+    GRL_REQUIRE(a.K * (int64_t)sizeof(T) * 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: K too large (256 rows must span < 2 GiB)");
+    static const int group = [] { const char* e = getenv("GRL_GEMM_GROUP"); return e ? atoi(e) : 0; }();
+    a.group = group > 0 ? group : (a.K * (int64_t)sizeof(T) >= 8192 ? 2 : 8);
+    const int64_t big_m = (a.M + 255) / 256, big_n = (a.N + 255) / 256;
+    const int64_t sm = (a.M + 127) / 128, sn = (a.N + 127) / 128;
+    GRL_REQUIRE(sm * sn < (1LL << 31), GRL_ERR_SHAPE, "gemm: too many tiles");
+    const int64_t cus = c->prop.multiProcessorCount;
+    if (big_m * big_n >= 192) {
+        a.tiles_m = (int)big_m; a.tiles_n = (int)big_n; *tile_cols = 256;
+        hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 256, 256, 2, 4, EPI_RESLN, false, false>), dim3((unsigned)std::min<int64_t>(big_m * big_n, cus)), dim3(512), 0, c->stream, a);
+    } else {
+        a.tiles_m = (int)sm; a.tiles_n = (int)sn; *tile_cols = 128;
+        hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 128, 128, 2, 2, EPI_RESLN, false, false>), dim3((unsigned)std::min<int64_t>(sm * sn, 2 * cus)), dim3(256), 0, c->stream, a);
+    }
+    GRL_CHECK_LAUNCH();
+    return GRL_OK;
+}
+
 template <typename T, typename OutT>
 int dispatch_epi(grl_ctx* c, GemmArgs& a, int epi) {
     switch (epi) {
@@ -881,6 +1098,7 @@ template <typename T, typename OutT>
 int dispatch_epi_ln(grl_ctx* c, GemmArgs& a, int epi) {
     switch (epi) {
         case EPI_NONE: return launch_gemm<T, OutT, EPI_NONE, false, true>(c, a);
+        case EPI_GELU: return launch_gemm<T, OutT, EPI_GELU, false, true>(c, a);
         case EPI_GLU: return launch_gemm<T, OutT, EPI_GLU, true, true>(c, a);
     }
     grl_set_error("gemm: epilogue %d has no LayerNorm-folded form", epi);

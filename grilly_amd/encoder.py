@@ -64,7 +64,13 @@ def random_bert_weights(cfg, seed=0, std=0.02):
 
 
 class BertEncoder:
-    def __init__(self, core, cfg, weights, dtype="fp32"):
+    """fused=None (default): both LayerNorms of every layer are folded into the GEMMs around them whenever the
+    direct-to-LDS GEMM kernels take the layer's shapes (d_model and d_ff multiples of 64 in bf16, 32 in fp32): the
+    residual stream then travels as raw rows plus row statistics and no LayerNorm pass runs over HBM between the
+    embedding and the final LayerNorm (grl_bert_layer_fwd_fused).  fused=False keeps the seven-launch layer with its
+    two LayerNorm passes (grl_bert_layer_fwd); fused=True insists and raises for shapes the fused layer does not take."""
+
+    def __init__(self, core, cfg, weights, dtype="fp32", fused=None):
         self.core = core.core if hasattr(core, "core") else core
         if not isinstance(self.core, HipCore):
             raise TypeError("BertEncoder needs a Compute() backend or its HipCore")
@@ -84,6 +90,32 @@ class BertEncoder:
             for k in _VECS:
                 setattr(s, k, up(np.asarray(lw[k]).reshape(-1)).ptr)
             self.layer_structs.append(s)
+        slab = 64 if self.code == L.GRL_BF16 else 32
+        eligible = cfg.d_model % slab == 0 and cfg.d_ff % slab == 0 and cfg.layers > 0
+        if fused and not eligible:
+            raise ValueError(f"the fused layer needs d_model and d_ff to be multiples of {slab} in {dtype}")
+        self.fused = eligible if fused is None else bool(fused)
+        self.fused_structs = []
+        if self.fused:
+            # every GEMM that reads a LayerNorm's output gets that norm folded into its weight (once, here):
+            # QKV of layer l reads the embedding norm (l = 0) or the second norm of layer l-1, FFN1 reads ln1
+            d, ff = cfg.d_model, cfg.d_ff
+            es = 2 if self.code == L.GRL_BF16 else 4
+
+            def fold(w_ptr, b_ptr, g_ptr, bt_ptr, n, k):
+                ws, cs, bf = self._own(c.alloc(n * k * es)), self._own(c.alloc(n * 4)), self._own(c.alloc(n * 4))
+                L.check(c.lib.grl_ln_fold(c.ctx, self.code, n, k, w_ptr, g_ptr, bt_ptr, b_ptr, ws.ptr, cs.ptr, bf.ptr), "fold layernorm")
+                return ws.ptr, cs.ptr, bf.ptr
+            in_g, in_b = self.emb_g.ptr, self.emb_b.ptr
+            for s in self.layer_structs:
+                f = L.BertLayerFused()
+                f.ws_qkv, f.c_qkv, f.bf_qkv = fold(s.w_qkv, s.b_qkv, in_g, in_b, 3 * d, d)
+                f.in_g, f.in_b = in_g, in_b
+                f.w_o, f.b_o, f.ln1_g, f.ln1_b = s.w_o, s.b_o, s.ln1_g, s.ln1_b
+                f.ws_ff1, f.c_ff1, f.bf_ff1 = fold(s.w_ff1, s.b_ff1, s.ln1_g, s.ln1_b, ff, d)
+                f.w_ff2, f.b_ff2 = s.w_ff2, s.b_ff2
+                self.fused_structs.append(f)
+                in_g, in_b = s.ln2_g, s.ln2_b
         self._shape = None
 
     def _own(self, buf):
@@ -99,8 +131,10 @@ class BertEncoder:
         if S > cfg.max_pos:
             raise ValueError(f"sequence length {S} exceeds max_pos {cfg.max_pos}")
         es = 2 if self.code == L.GRL_BF16 else 4
-        ws = c.lib.grl_bert_layer_workspace(self.code, B, S, cfg.heads, cfg.head_dim, cfg.d_ff)
+        wsfn = c.lib.grl_bert_layer_fused_workspace if self.fused else c.lib.grl_bert_layer_workspace
+        ws = wsfn(self.code, B, S, cfg.heads, cfg.head_dim, cfg.d_ff)
         self.x = c.alloc(B * S * cfg.d_model * es)
+        self.stats = c.alloc(max(B * S, 1) * 8)        # {1/sd, mean/sd} per row of the raw residual stream (fused layers)
         self.ws = c.alloc(ws)
         self.ids = c.alloc(B * S * 4)
         self.mask = c.alloc(B * S * 4)
@@ -109,7 +143,7 @@ class BertEncoder:
 
     def release_activations(self):
         if self._shape is not None:
-            for b in (self.x, self.ws, self.ids, self.mask, self.pooled):
+            for b in (self.x, self.stats, self.ws, self.ids, self.mask, self.pooled):
                 b.free()
             self._shape = None
 
@@ -135,12 +169,25 @@ class BertEncoder:
         B, S = self._shape
         cfg, c, lib = self.cfg, self.core, self.core.lib
         mask = self.mask.ptr if self.has_mask else None
-        L.check(lib.grl_embed_layernorm(c.ctx, self.code, B, S, cfg.d_model, cfg.vocab, self.ids.ptr, self.tok.ptr,
-                                        self.pos.ptr, self.typ.ptr, self.emb_g.ptr, self.emb_b.ptr, cfg.embedding_eps,
-                                        self.x.ptr), "embedding + layernorm")
-        for s in self.layer_structs:
-            L.check(lib.grl_bert_layer_fwd(c.ctx, self.code, B, S, cfg.heads, cfg.head_dim, cfg.d_ff, ctypes.byref(s),
-                                           mask, cfg.eps, self.x.ptr, self.ws.ptr), "bert_layer_fwd")
+        if self.fused and B * S > 0:
+            # raw embedding rows + their statistics; every layer consumes and produces (raw rows, statistics); the last
+            # layer's second LayerNorm is the one pass that writes normalised rows
+            L.check(lib.grl_embed(c.ctx, self.code, B, S, cfg.d_model, cfg.vocab, self.ids.ptr, self.tok.ptr, self.pos.ptr,
+                                  self.typ.ptr, self.x.ptr), "embedding")
+            L.check(lib.grl_ln_stats(c.ctx, self.code, B * S, cfg.d_model, self.x.ptr, cfg.embedding_eps, self.stats.ptr), "embedding statistics")
+            for f in self.fused_structs:
+                L.check(lib.grl_bert_layer_fwd_fused(c.ctx, self.code, B, S, cfg.heads, cfg.head_dim, cfg.d_ff, ctypes.byref(f),
+                                                     mask, cfg.eps, self.x.ptr, self.stats.ptr, self.ws.ptr), "bert_layer_fwd_fused")
+            last = self.layer_structs[-1]
+            L.check(lib.grl_layernorm(c.ctx, self.code, B * S, cfg.d_model, self.x.ptr, None, last.ln2_g, last.ln2_b, cfg.eps,
+                                      self.x.ptr), "final layernorm")
+        else:
+            L.check(lib.grl_embed_layernorm(c.ctx, self.code, B, S, cfg.d_model, cfg.vocab, self.ids.ptr, self.tok.ptr,
+                                            self.pos.ptr, self.typ.ptr, self.emb_g.ptr, self.emb_b.ptr, cfg.embedding_eps,
+                                            self.x.ptr), "embedding + layernorm")
+            for s in self.layer_structs:
+                L.check(lib.grl_bert_layer_fwd(c.ctx, self.code, B, S, cfg.heads, cfg.head_dim, cfg.d_ff, ctypes.byref(s),
+                                               mask, cfg.eps, self.x.ptr, self.ws.ptr), "bert_layer_fwd")
         if pool:
             L.check(lib.grl_mean_pool(c.ctx, self.code, B, S, cfg.d_model, self.x.ptr, mask, self.pooled.ptr, 1), "mean_pool")
 

@@ -104,6 +104,18 @@ int grl_sync(grl_ctx* ctx);
  * each other's start. */
 int grl_timer_start(grl_ctx* ctx);
 int grl_timer_stop(grl_ctx* ctx, float* elapsed_ms);   /* synchronises */
+/* Lap events on the context stream (measurement aid, no counterpart in the reference): grl_timer_lap records event
+ * `index` (0..255) behind whatever is enqueued so far, without waiting; grl_timer_lap_ms waits for event `to` and
+ * returns the time between two recorded events.  A lap before and after each launch of a back-to-back sequence gives
+ * per-launch durations (for medians) without host synchronisations between the launches. */
+int grl_timer_lap(grl_ctx* ctx, int index);
+int grl_timer_lap_ms(grl_ctx* ctx, int from, int to, float* elapsed_ms);
+/* Matrix-core ceiling probe (measurement aid, no counterpart in the reference): every CU runs eight waves that issue
+ * nothing but MFMAs on register-resident operands (kind 0: v_mfma_f32_32x32x16_bf16, kind 1: v_mfma_f32_16x16x32_bf16)
+ * for `iters` loop iterations, after one untimed warm-up launch.  `operands` points to 64 KiB of device memory whose
+ * bits become the operand fragments (NULL: all-zero operands).  Returns the launch duration and the FLOPs it
+ * executed: the rate the matrix cores sustain under the board's power limit for those operand bits. */
+int grl_mfma_probe(grl_ctx* ctx, int kind, const void* operands, int iters, float* elapsed_ms, double* flops);
 /* Shader-clock probe, a measurement aid with no counterpart in the reference: _begin starts a one-wave kernel on a
  * second stream of the context that runs for `millis` of wall time beside whatever the caller enqueues next; _end
  * waits for it and returns the average shader clock in GHz over that time (shader cycles over 100 MHz reference
@@ -250,11 +262,31 @@ int grl_ln_glu_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t 
                   const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
                   const float* bias_gate_folded, const float* bias_up_folded, float eps, float* stats,
                   void* out, int activation);
+/* grl_ln_gemm_nt with the row statistics given ({1/sd, mean/sd} per row of x, as grl_ln_stats or grl_gemm_nt_resln
+ * write them) and a choice of epilogue: GRL_EPI_NONE or GRL_EPI_GELU (out = gelu(LN(x).W^T + b), the first half of the
+ * feed-forward block behind a LayerNorm, utils/vulkan_sentence_transformer.py:1004-1012). */
+int grl_ln_gemm_nt_stats(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                         const void* W_scaled, const float* colsum, const float* bias_folded, const float* stats,
+                         void* out, int epilogue);
+/* C = A.W^T + bias + LayerNorm(R; r_gamma, r_beta), and stats_out = {1/sd, mean/sd} of every row of C (with eps).
+ * The post-LN sub-block "x + f(x)" where x is itself the output of a LayerNorm that was never written out: R holds the
+ * raw rows in front of that LayerNorm, r_stats their {1/sd, mean/sd}; the GEMM epilogue re-forms x from them, adds it,
+ * and reduces each output row's sum and sum of squares per column tile, which a small merge kernel turns into the
+ * statistics the NEXT LayerNorm-folded GEMM (grl_ln_gemm_nt_stats) reads.  Together the two entry points run the
+ * reference's linear -> add -> layer_norm -> linear chain (utils/vulkan_sentence_transformer.py:996-1026) without a
+ * LayerNorm pass over HBM.  C may be R (in place).  A, W, R, C of `dtype`; only for problems the direct-to-LDS kernels
+ * take: K a multiple of 64 (bf16) / 32 (fp32), N a multiple of 8 / 4, 16-byte aligned pointers, else GRL_ERR_SHAPE.
+ * workspace: grl_gemm_nt_resln_workspace(M, N) bytes, 16-byte aligned. */
+int64_t grl_gemm_nt_resln_workspace(int64_t M, int64_t N);
+int grl_gemm_nt_resln(grl_ctx* ctx, int dtype, int64_t M, int64_t N, int64_t K, const void* A, const void* W,
+                      const float* bias, const void* R, const float* r_stats, const float* r_gamma, const float* r_beta,
+                      void* C, float eps, float* stats_out, void* workspace);
 
 /* out = a + b.  Replaces VulkanFNN.residual (shaders/fnn-residual.glsl:25-34).
  * grl_add, grl_gelu, grl_silu and grl_relu may run in place (out == a, out == b, y == x).
  * Every other entry point of this header needs its outputs distinct from its inputs unless its own
- * comment says otherwise (grl_gemm_nt_res: C may be the residual; grl_bert_layer_fwd: x is updated in place). */
+ * comment says otherwise (grl_gemm_nt_res, grl_gemm_nt_resln: C may be the residual; grl_bert_layer_fwd, grl_bert_layer_fwd_fused: x / r is
+ * updated in place). */
 int grl_add(grl_ctx* ctx, int dtype, int64_t n, const void* a, const void* b, void* out);
 /* Replaces VulkanFNN.activation_gelu (backend/fnn.py:285-342, shaders/activation-gelu.glsl:23-53). */
 int grl_gelu(grl_ctx* ctx, int dtype, int64_t n, const void* x, void* y);
@@ -316,6 +348,31 @@ int64_t grl_bert_layer_workspace(int dtype, int64_t B, int64_t S, int64_t H, int
 int grl_bert_layer_fwd(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
                        int64_t d_ff, const grl_bert_layer* w, const float* mask, float eps,
                        void* x, void* workspace);
+
+/* The same layer with both LayerNorms folded into the GEMMs around them: no LayerNorm pass over HBM.  The residual
+ * stream travels as RAW rows r plus their statistics: on entry r holds the rows whose LayerNorm (in_g, in_b, statistics
+ * in `stats`) is the layer's input x; on return r holds x1 + FFN(x1) (x1 = LN(x + attention block; ln1)) and `stats`
+ * its statistics, so that the layer's output LN(r; ln2) is formed by the next layer (whose in_g / in_b are this
+ * layer's ln2 parameters) or by one grl_layernorm after the last layer.
+ *   qkv = LN(r).Wqkv^T          grl_ln_gemm_nt_stats on r with the weight folded by grl_ln_fold(in_g, in_b)
+ *   r   = attn.Wo^T + LN(r)     grl_gemm_nt_resln (in place), statistics of the new r out
+ *   ff  = gelu(LN(r; ln1).W1^T) grl_ln_gemm_nt_stats, weight folded with ln1
+ *   r   = ff.W2^T + LN(r; ln1)  grl_gemm_nt_resln (in place)
+ * Same recipe as grl_bert_layer_fwd (utils/vulkan_sentence_transformer.py:972-1035); needs d_model and d_ff multiples
+ * of 64 (bf16) / 32 (fp32), else GRL_ERR_SHAPE.  stats: (B*S, 2) floats, 16-byte aligned. */
+typedef struct grl_bert_layer_fused {
+    const void*  ws_qkv; const float* c_qkv;  const float* bf_qkv;   /* grl_ln_fold of (w_qkv, b_qkv) with in_g, in_b */
+    const float* in_g;   const float* in_b;                           /* the LayerNorm that turns r into the layer input */
+    const void*  w_o;    const float* b_o;
+    const float* ln1_g;  const float* ln1_b;
+    const void*  ws_ff1; const float* c_ff1;  const float* bf_ff1;   /* grl_ln_fold of (w_ff1, b_ff1) with ln1_g, ln1_b */
+    const void*  w_ff2;  const float* b_ff2;
+} grl_bert_layer_fused;
+
+int64_t grl_bert_layer_fused_workspace(int dtype, int64_t B, int64_t S, int64_t H, int64_t D, int64_t d_ff);
+int grl_bert_layer_fwd_fused(grl_ctx* ctx, int dtype, int64_t B, int64_t S, int64_t H, int64_t D,
+                             int64_t d_ff, const grl_bert_layer_fused* w, const float* mask, float eps,
+                             void* r, float* stats, void* workspace);
 
 #ifdef __cplusplus
 }

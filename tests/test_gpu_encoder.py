@@ -122,26 +122,36 @@ def test_encoder_batch_independence_full_config(backend):
     np.testing.assert_allclose(np.linalg.norm(full, axis=1), 1.0, atol=1e-4)
 
 
-def test_bench_shape_forward_b128(backend):
+@pytest.mark.parametrize("fused", [True, False])
+def test_bench_shape_forward_b128(backend, fused):
     """The forward the benchmark times (BASELINE configs[2]: 12 layers, d=768, 12x64 heads, FFN 3072, batch 128 x seq 512,
-    bf16, M = 65536 rows per GEMM): sampled sequences equal their own batch-of-one runs through all 12 layers, and the
-    first layer at full batch width is checked against the float64 oracle of the same recipe with bf16 storage emulated."""
+    bf16, M = 65536 rows per GEMM), in both layer forms (LayerNorms folded into the GEMMs, which is what the benchmark
+    runs, and the seven-launch layer): sampled sequences equal their own batch-of-one runs through all 12 layers, and
+    the first layer at full batch width is checked against the float64 oracle of the same recipe with bf16 storage
+    emulated.  The seven-launch layer computes every output element with the same arithmetic whatever the batch, so
+    the two runs differ by almost nothing; the folded form merges its row statistics from per-tile partials whose
+    number depends on the tile size the batch selects, the last float bit of a statistic flips bf16 roundings, and
+    twelve layers spread that: both runs are then equally valid bf16 results, compared at the bf16 tolerance."""
     cfg = EncoderConfig()
     w = random_bert_weights(cfg, seed=20260134)
     rng = rng_for(3)
     B, S = 128, 512
     ids = rng.integers(0, cfg.vocab, (B, S))
-    enc = BertEncoder(backend, cfg, w, dtype="bf16")
+    enc = BertEncoder(backend, cfg, w, dtype="bf16", fused=fused)
     h = enc.forward(ids, None, pool=False)
     assert h.shape == (B, S, cfg.d_model) and np.isfinite(h).all()
     for b in (0, 77, 127):
         one = enc.forward(ids[b:b + 1], None, pool=False)
-        np.testing.assert_allclose(h[b:b + 1], one, atol=3e-2)          # same kernels, other tile walk: bf16 rounding only
-        assert O.max_rel(h[b:b + 1], one) < 5e-3
+        if fused:
+            assert O.max_rel(h[b:b + 1], one) < TOL_BF16
+            assert np.abs(h[b:b + 1] - one).mean() < 1e-2
+        else:
+            np.testing.assert_allclose(h[b:b + 1], one, atol=3e-2)          # same kernels, other tile walk: bf16 rounding only
+            assert O.max_rel(h[b:b + 1], one) < 5e-3
     enc.release_activations()
     cfg1 = EncoderConfig(layers=1)
     w1 = dict(w, layers=w["layers"][:1])
-    enc1 = BertEncoder(backend, cfg1, w1, dtype="bf16")
+    enc1 = BertEncoder(backend, cfg1, w1, dtype="bf16", fused=fused)
     h1 = enc1.forward(ids, None, pool=False)
     for b in (3, 64, 126):
         ref = truth_encoder(w1, cfg1, ids[b:b + 1], None, O.bf16_round)

@@ -1,0 +1,182 @@
+"""The LayerNorm-free form of the post-LN layer (reference recipe utils/vulkan_sentence_transformer.py:972-1035):
+`grl_ln_gemm_nt_stats` (a GEMM that reads LayerNorm(x) without x ever being normalised in memory, statistics given),
+`grl_gemm_nt_resln` (a GEMM that adds LayerNorm(R) re-formed from raw rows and writes the row statistics of its own
+output) and `grl_bert_layer_fwd_fused` built from them, each through the C ABI against the float64 oracle of the
+unfused formulas, plus the fused encoder against the seven-launch one.
+Tolerances: max|y-ref|/max|ref| <= 1e-4 (fp32), <= 2e-2 (bf16)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import TOL_F32, TOL_BF16
+from oracle import oracle_np as O
+from grilly_amd import _lib as L
+from grilly_amd import BertEncoder, EncoderConfig, random_bert_weights
+
+pytestmark = pytest.mark.gpu
+
+
+def _code(dtype):
+    return L.GRL_BF16 if dtype == "bf16" else L.GRL_F32
+
+
+def _q(dtype, a):
+    return O.bf16_round(a) if dtype == "bf16" else a
+
+
+def _stats(x, eps):
+    x = x.astype(np.float64)
+    mu = x.mean(-1)
+    sd = np.sqrt(x.var(-1) + eps)
+    return np.stack([1 / sd, mu / sd], -1)
+
+
+# (M, K, N): 256x256 tiles with ragged edges / 128x128 tiles / a single small tile
+SHAPES = [(4096 + 37, 768, 3072 + 8), (8192, 3072, 768), (300, 128, 200), (64, 64, 8)]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("epi", ["none", "gelu"])
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_ln_gemm_with_given_statistics(backend, dtype, epi, M, K, N):
+    c, code = backend.core, _code(dtype)
+    if dtype == "fp32" and K % 32 or dtype == "bf16" and K % 64:
+        pytest.skip("K is not a whole number of 128-byte slabs for this type")
+    rng = np.random.default_rng(M + K + N)
+    x = _q(dtype, (rng.standard_normal((M, K)) * 1.5 + 0.7 * rng.standard_normal((M, 1))).astype(np.float32))
+    W = _q(dtype, (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32))
+    g = (1 + 0.2 * rng.standard_normal(K)).astype(np.float32)
+    bt = (0.3 * rng.standard_normal(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    eps = 1e-5
+    es = 2 if dtype == "bf16" else 4
+    dx, dw, dg, dbt, db = c.upload(x, code), c.upload(W, code), c.upload(g), c.upload(bt), c.upload(b)
+    ws, cs, bf, st, out = c.alloc(N * K * es), c.alloc(N * 4), c.alloc(N * 4), c.alloc(M * 8), c.alloc(M * N * es)
+    try:
+        L.check(c.lib.grl_ln_fold(c.ctx, code, N, K, dw.ptr, dg.ptr, dbt.ptr, db.ptr, ws.ptr, cs.ptr, bf.ptr), "fold")
+        L.check(c.lib.grl_ln_stats(c.ctx, code, M, K, dx.ptr, eps, st.ptr), "stats")
+        L.check(c.lib.grl_ln_gemm_nt_stats(c.ctx, code, code, M, N, K, dx.ptr, ws.ptr, cs.ptr, bf.ptr, st.ptr, out.ptr,
+                                           L.EPI_GELU if epi == "gelu" else L.EPI_NONE), "ln_gemm_nt_stats")
+        y = c.download(out, (M, N), code)
+        rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 40)]))
+        # the weight the kernel multiplies by is gamma*W rounded to the storage type
+        wsq = _q(dtype, (W.astype(np.float64) * g[None, :]).astype(np.float32)).astype(np.float64)
+        xs = x[rows].astype(np.float64)
+        mu, sd = xs.mean(-1, keepdims=True), np.sqrt(xs.var(-1, keepdims=True) + eps)
+        pre = ((xs - mu) / sd) @ wsq.T + (b + W.astype(np.float64) @ bt)
+        ref = O.truth_gelu(pre) if epi == "gelu" else pre
+        assert np.isfinite(y).all()
+        assert O.max_rel(y[rows], ref) < (TOL_BF16 if dtype == "bf16" else TOL_F32)
+        # and it is the LayerNorm + linear of the unfused chain (weights unrounded) within the bf16 tolerance
+        ref2 = O.truth_linear(O.truth_layernorm(x[rows], g, bt, eps), W, b, epi)
+        assert O.max_rel(y[rows], ref2) < (TOL_BF16 if dtype == "bf16" else TOL_F32)
+    finally:
+        for t in (dx, dw, dg, dbt, db, ws, cs, bf, st, out):
+            t.free()
+    with c.alloc(64) as t:
+        assert c.lib.grl_ln_gemm_nt_stats(c.ctx, code, code, 1, 8, 64, t.ptr, t.ptr, t.ptr, t.ptr, t.ptr, t.ptr, L.EPI_SILU) == L.ERR_ARG
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("inplace", [False, True])
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_gemm_with_layernormed_residual_and_row_statistics(backend, dtype, inplace, M, K, N):
+    c, code = backend.core, _code(dtype)
+    if dtype == "fp32" and K % 32 or dtype == "bf16" and K % 64:
+        pytest.skip("K is not a whole number of 128-byte slabs for this type")
+    rng = np.random.default_rng(7 * M + K + N)
+    A = _q(dtype, rng.standard_normal((M, K)).astype(np.float32))
+    W = _q(dtype, (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32))
+    b = rng.standard_normal(N).astype(np.float32)
+    R = _q(dtype, (2.0 * rng.standard_normal((M, N)) + rng.standard_normal((M, 1))).astype(np.float32))
+    g = (1 + 0.2 * rng.standard_normal(N)).astype(np.float32)
+    bt = (0.3 * rng.standard_normal(N)).astype(np.float32)
+    eps_r, eps = 1e-5, 1e-6
+    rst = _stats(R, eps_r).astype(np.float32)
+    es = 2 if dtype == "bf16" else 4
+    dA, dW, db, dR, dst, dg, dbt = c.upload(A, code), c.upload(W, code), c.upload(b), c.upload(R, code), c.upload(rst), c.upload(g), c.upload(bt)
+    dC = dR if inplace else c.alloc(M * N * es)
+    so = c.alloc(M * 8)
+    wk = c.alloc(c.lib.grl_gemm_nt_resln_workspace(M, N))
+    try:
+        L.check(c.lib.grl_gemm_nt_resln(c.ctx, code, M, N, K, dA.ptr, dW.ptr, db.ptr, dR.ptr, dst.ptr, dg.ptr, dbt.ptr, dC.ptr,
+                                        eps, so.ptr, wk.ptr), "gemm_nt_resln")
+        y = c.download(dC, (M, N), code)
+        stats = c.download(so, (M, 2))
+        rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 40)]))
+        ref = O.truth_linear(A[rows], W, b) + O.truth_layernorm(R[rows], g, bt, eps_r)
+        tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+        assert np.isfinite(y).all() and np.isfinite(stats).all()
+        assert O.max_rel(y[rows], ref) < tol
+        # statistics of the rows as written (every row): they feed the next LayerNorm-folded GEMM
+        want = _stats(y, eps)
+        assert O.max_rel(stats[:, 0], want[:, 0]) < (5e-3 if dtype == "bf16" else 1e-4)
+        assert np.abs(stats[:, 1] - want[:, 1]).max() < (5e-3 if dtype == "bf16" else 1e-4) * max(1.0, np.abs(want[:, 1]).max())
+        # a second run is bit-identical (partials are merged in a fixed order)
+        if not inplace:
+            L.check(c.lib.grl_gemm_nt_resln(c.ctx, code, M, N, K, dA.ptr, dW.ptr, db.ptr, dR.ptr, dst.ptr, dg.ptr, dbt.ptr, dC.ptr,
+                                            eps, so.ptr, wk.ptr), "gemm_nt_resln")
+            np.testing.assert_array_equal(c.download(dC, (M, N), code), y)
+            np.testing.assert_array_equal(c.download(so, (M, 2)), stats)
+    finally:
+        for t in (dA, dW, db, dR, dst, dg, dbt, so, wk):
+            t.free()
+        if not inplace:
+            dC.free()
+
+
+def test_resln_rejects_what_the_staged_kernels_do_not_take(backend):
+    c = backend.core
+    with c.alloc(4096) as t:
+        args = (t.ptr, t.ptr, None, t.ptr, t.ptr, t.ptr, t.ptr, t.ptr, 1e-5, t.ptr, t.ptr)
+        assert c.lib.grl_gemm_nt_resln(c.ctx, L.GRL_F32, 4, 8, 24, *args) == L.ERR_SHAPE            # K not a whole slab
+        assert c.lib.grl_gemm_nt_resln(c.ctx, L.GRL_BF16, 4, 12, 64, *args) == L.ERR_SHAPE          # rows of 24 bytes
+        assert c.lib.grl_gemm_nt_resln(c.ctx, L.GRL_F32, 4, 8, 32, t.ptr, None, None, *args[3:]) == L.ERR_ARG
+        assert c.lib.grl_gemm_nt_resln(c.ctx, L.GRL_F32, 0, 8, 32, *args) == 0
+        f = L.BertLayerFused()
+        assert c.lib.grl_bert_layer_fwd_fused(c.ctx, L.GRL_F32, 1, 4, 2, 8, 64, ctypes.byref(f), None, 1e-5, t.ptr, t.ptr, t.ptr) == L.ERR_ARG
+    assert c.lib.grl_bert_layer_fused_workspace(L.GRL_F32, 2, 16, 2, 32, 128) > 0
+    cfg = EncoderConfig(layers=1, d_model=48, heads=3, d_ff=96, vocab=50, max_pos=16)
+    with pytest.raises(ValueError):
+        BertEncoder(backend, cfg, random_bert_weights(cfg, seed=0), dtype="bf16", fused=True)
+    assert BertEncoder(backend, cfg, random_bert_weights(cfg, seed=0), dtype="bf16").fused is False
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("d,heads,ff,S", [(128, 4, 512, 40), (768, 12, 3072, 512), (384, 12, 1536, 100)])
+def test_fused_encoder_equals_the_unfused_one(backend, dtype, d, heads, ff, S):
+    """Both layer forms against the float64 oracle, with non-trivial biases and LayerNorm parameters (the fused form
+    folds gamma into weights and beta into biases) and a padding mask; and against each other."""
+    cfg = EncoderConfig(layers=2, d_model=d, heads=heads, d_ff=ff, vocab=300, max_pos=512)
+    w = random_bert_weights(cfg, seed=d + S)
+    rng = np.random.default_rng(d + S)
+    w["emb_ln_g"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    w["emb_ln_b"] = (0.1 * rng.standard_normal(d)).astype(np.float32)
+    for lw in w["layers"]:
+        for k in ("b_qkv", "b_o", "b_ff1", "b_ff2", "ln1_b", "ln2_b"):
+            lw[k] = (rng.standard_normal(lw[k].shape) * 0.05).astype(np.float32)
+        for k in ("ln1_g", "ln2_g"):
+            lw[k] = (1 + rng.standard_normal(lw[k].shape) * 0.1).astype(np.float32)
+    B = 3
+    ids = rng.integers(0, cfg.vocab, (B, S))
+    lens = np.array([S, max(1, S // 3), S - 1])
+    mask = (np.arange(S)[None] < lens[:, None]).astype(np.float32)
+    fused = BertEncoder(backend, cfg, w, dtype=dtype, fused=True)
+    plain = BertEncoder(backend, cfg, w, dtype=dtype, fused=False)
+    assert fused.fused and not plain.fused
+    hf, hp = fused.forward(ids, mask, pool=False), plain.forward(ids, mask, pool=False)
+    quant = O.bf16_round if dtype == "bf16" else None
+    qf = (lambda a: a) if quant is None else (lambda a: quant(np.asarray(a, np.float32)).astype(np.float64))
+    x = qf(O.truth_layernorm(qf(O.truth_embed(ids, w["tok_emb"], w["pos_emb"], w["type_emb"])), w["emb_ln_g"], w["emb_ln_b"], cfg.eps))
+    for lw in w["layers"]:
+        lq = {k: (quant(v) if (quant and k.startswith("w_")) else v) for k, v in lw.items()}
+        x = O.truth_bert_layer(x, lq, mask, heads, cfg.eps, quant)
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    assert np.isfinite(hf).all()
+    assert O.max_rel(hp, x) < tol
+    assert O.max_rel(hf, x) < tol
+    assert O.max_rel(hf, hp) < tol
+    pf, pp = fused.forward(ids, mask, pool=True), plain.forward(ids, mask, pool=True)
+    assert O.max_rel(pf, pp) < (1e-4 if dtype == "fp32" else 1e-2)
+    fused.release_activations(); plain.release_activations()
