@@ -108,11 +108,21 @@ template <> struct MfmaSlab<uint16_t> {   // bf16: 16 B = 8 values, k = 8*(lane/
     static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), acc, 0, 0, 0);
     }
+    // acc = w.x + c: the first product of a tile starts from c (zeros or the bias) without a copy
+    static __device__ __forceinline__ void run_from(const u32x4& w, const u32x4& x, const f32x16& c, f32x16& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), c, 0, 0, 0);
+    }
 };
 template <> struct MfmaSlab<float> {      // fp32: 16 B = 4 values, each feeds one 32x32x2 MFMA
     static __device__ __forceinline__ void run(const u32x4& w, const u32x4& x, f32x16& acc) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u2f(w[e]), u2f(x[e]), acc, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void run_from(const u32x4& w, const u32x4& x, const f32x16& c, f32x16& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u2f(w[0]), u2f(x[0]), c, 0, 0, 0);
+#pragma unroll
+        for (int e = 1; e < 4; ++e)
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u2f(w[e]), u2f(x[e]), acc, 0, 0, 0);
     }
 };
@@ -637,6 +647,33 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
 
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's transfers (and earlier stores) are done
         __syncthreads();                         // ... and everybody else's; all staging reads of the last tile too
+        // What every accumulator block starts from: the bias of its columns when the LDS-staged epilogue follows (the first
+        // MFMA of a block takes it as its C operand, so the epilogue has no bias add left), else zeros (the direct
+        // epilogue adds the bias itself; the folded LayerNorm scales the sum before its bias).  Accumulator register
+        // 4q+e of block b holds column 8q + 4*(lane/32) + e of the block.
+        constexpr bool BIASC = !LN;
+        f32x16 c0[TN];
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) c0[b][r] = 0.f;
+        if (BIASC && staged) {
+            const char* bl = lds + 2 * STAGE + bbuf * BIASB;
+#pragma unroll
+            for (int b = 0; b < TN; ++b) {
+                const bool up = DUAL && b >= TNO;
+                const float* bsrc = up ? p.bias2 : p.bias;
+                if (bsrc) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int nl = wn * WNO + (b % TNO) * 32 + 8 * q + 4 * lg;
+                        const f32x4 v = *(const f32x4*)(bl + (up ? BNO * 4 : 0) + nl * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) c0[b][4 * q + e] = v[e];
+                    }
+                }
+            }
+        }
         auto k_slab = [&](int kt, auto ifirst) {
             constexpr bool FIRST = decltype(ifirst)::value;
             if (kt + 1 < KT) {
@@ -647,9 +684,6 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                 }
             }
             const char* s = lds + (kt & 1) * STAGE;
-#ifndef GRL_KLOOP
-#define GRL_KLOOP 2
-#endif
             auto load_frags = [&](int sl, u32x4 (&xf)[TM], u32x4 (&wf)[TN]) {
                 const int ch = 2 * sl + lg;
 #pragma unroll
@@ -661,36 +695,23 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                 static_for<TM>([&](auto ia) {
                     static_for<TN>([&](auto ib) {
                         constexpr int a = decltype(ia)::value, b = decltype(ib)::value;
-                        if (FIRST && sl == 0) {
-#pragma unroll
-                            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;      // folds into the MFMA's C operand
-                        }
-                        MfmaSlab<T>::run(wf[b], xf[a], acc[a][b]);
+                        if (FIRST && sl == 0) MfmaSlab<T>::run_from(wf[b], xf[a], c0[b], acc[a][b]);
+                        else MfmaSlab<T>::run(wf[b], xf[a], acc[a][b]);
                     });
                 });
             };
-            if constexpr (GRL_KLOOP == 2) {
-                // two fragment sets: the reads of the next 16-deep step are issued in front of this step's MFMAs
-                u32x4 xf[2][TM], wf[2][TN];
-                load_frags(0, xf[0], wf[0]);
+            // Two fragment sets: the LDS reads of the next 16-deep step are issued in front of this step's eight MFMAs, and
+            // fences keep the scheduler from regrouping them (left to itself it sinks the reads to save registers, down to
+            // one activation fragment at a time and a wait in front of every second MFMA in the kernels with the larger
+            // epilogues; pinned and double-buffered, every GEMM here gains 3 to 8 %).
+            u32x4 xf[2][TM], wf[2][TN];
+            load_frags(0, xf[0], wf[0]);
 #pragma unroll
-                for (int sl = 0; sl < 4; ++sl) {
-                    if (sl + 1 < 4) load_frags(sl + 1, xf[(sl + 1) & 1], wf[(sl + 1) & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
-                    run_mfmas(sl, xf[sl & 1], wf[sl & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            } else {
-#pragma unroll
-                for (int sl = 0; sl < 4; ++sl) {
-                    u32x4 xf[TM], wf[TN];
-                    load_frags(sl, xf, wf);
-                    // The kernels whose epilogues need more registers make the scheduler shrink this loop's fragment set to
-                    // one activation fragment at a time (a wait in front of every second MFMA); the fence keeps the six
-                    // reads of a 16-deep step together in front of its eight MFMAs, as in the other kernels.
-                    if constexpr (LN || RL || GRL_KLOOP == 1) __builtin_amdgcn_sched_barrier(0);
-                    run_mfmas(sl, xf, wf);
-                }
+            for (int sl = 0; sl < 4; ++sl) {
+                if (sl + 1 < 4) load_frags(sl + 1, xf[(sl + 1) & 1], wf[(sl + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                run_mfmas(sl, xf[sl & 1], wf[sl & 1]);
+                __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();
@@ -745,7 +766,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             // bias of this lane's 4-column groups, once per tile (columns past N hold zero)
             // (the dual-weight kernel with the folded LayerNorm reads them from LDS where they are used instead: two bias
             // sets in registers next to its two accumulator sets and the row factor do not fit)
-            constexpr bool BREG = !(LN && DUAL);
+            constexpr bool BREG = LN && !DUAL;         // (without the folded LayerNorm the bias is in the accumulators already)
             f32x4 bv1[BREG ? TNO : 1][4], bv2[BREG ? TNO : 1][4];
             if constexpr (BREG) {
 #pragma unroll
@@ -781,22 +802,21 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                         constexpr int q = decltype(iq)::value;
                         const int nl = wn * WNO + b * 32 + 8 * q + 4 * lg;
                         float v[4];
-                        f32x4 b1, b2 = {0.f, 0.f, 0.f, 0.f};
+                        f32x4 b1 = {0.f, 0.f, 0.f, 0.f}, b2 = {0.f, 0.f, 0.f, 0.f};
                         if constexpr (BREG) {
                             b1 = bv1[BREG ? b : 0][q];
-                            if (DUAL) b2 = bv2[BREG ? b : 0][q];
-                        } else {
+                        } else if constexpr (LN) {
                             b1 = *(const f32x4*)(bias_lds + nl * 4);            // the folded biases always exist
                             b2 = *(const f32x4*)(bias_lds + BNO * 4 + nl * 4);
                         }
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = LN ? acc[a][b][4 * q + e] * rs + b1[e] : acc[a][b][4 * q + e] + b1[e];
+                        for (int e = 0; e < 4; ++e) v[e] = LN ? acc[a][b][4 * q + e] * rs + b1[e] : acc[a][b][4 * q + e];
                         if (DUAL) {
                             float up[4];
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
                                 up[e] = acc[a][DUAL ? b + TNO : b][4 * q + e];
-                                up[e] = LN ? up[e] * rs + b2[e] : up[e] + b2[e];
+                                if constexpr (LN) up[e] = up[e] * rs + b2[e];
                             }
                             glu_apply4(v, up, p);
                         } else {

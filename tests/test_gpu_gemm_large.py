@@ -100,7 +100,9 @@ def test_big_tile_glu(backend, dtype, act, M, K, N, bias):
         out2, g, u = fn(x, Wg, Wu, bg, bu, return_cache=True, dtype=dtype)     # direct epilogue with the fp32 pre-activations
         assert O.max_rel(out2[rows], t_out) < tol(dtype)
         assert O.max_rel(g[rows], t_g) < tol(dtype) and O.max_rel(u[rows], t_u) < tol(dtype)
-        np.testing.assert_array_equal(out2, out)
+        # the staged epilogue starts its accumulators from the bias, the direct one adds the bias after the sum: the two
+        # agree to the last bits of the float sums
+        assert O.max_rel(out2, out) < (2e-6 if dtype == "fp32" else 8e-3)
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
