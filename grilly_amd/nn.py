@@ -5,8 +5,9 @@ same class names, constructor arguments, parameter names and call conventions.
 Differences, all on purpose:
   * forward only (the reference's backward methods belong to its autograd path);
   * no CPU fallback: a failing backend call raises instead of silently recomputing in numpy;
-  * MultiheadAttention goes through the fused attention kernel, so it cannot hand back the
-    attention weights: it returns (output, None).
+  * MultiheadAttention with need_weights=False goes through the fused attention kernel (which never forms
+    the weights) and returns (output, None); with need_weights=True, or key / value of another length than the
+    query, it takes the score GEMM -> softmax -> output GEMM route and returns (output, weights (B,H,Sq,Sk)).
 """
 import numpy as np
 
