@@ -684,6 +684,16 @@ def main():
                                    "with the power state of the board and differ by up to 20 % between boxes (the same launches inside "
                                    "the forward, between other kernels, are not systematically slower or faster): see "
                                    "profiles/encoder_forward_bert_base_bf16_kernel_stats.md"}
+        if fused:
+            # the plain instantiation (what linear / fused_qkv_projection launch; the dominant kernel of the seven-launch
+            # layer and of earlier measurements of this benchmark), same definition: mean FLOPs over mean duration
+            gp = [kt[k] for k in ("gemm_qkv", "gemm_out", "gemm_ffn2")]
+            fl, ms3 = sum(r["flops"] for r in gp) / 3, sum(r["ms"] for r in gp) / 3
+            out["roofline_plain_gemm"] = {"kernel": f"gemm_nt_dma_kernel<{tname},{tname},256,256,2,4,EPI_NONE>", "launches": ["gemm_qkv", "gemm_out", "gemm_ffn2"],
+                                          "achieved": round(fl / (ms3 * 1e-3) / 1e12, 1), "peak": peak / 1e12, "unit": "TFLOP/s",
+                                          "frac": round(fl / (ms3 * 1e-3) / peak, 4), "avg_launch_ms": round(ms3, 4),
+                                          "shader_clock_ghz": round(sum(r["shader_clock_ghz"] for r in gp) / 3, 3),
+                                          "note": "not launched by the default forward (its GEMMs carry the folded LayerNorms); bench.py --unfused times the forward built from it"}
     extra = {}
     hidden32 = None
     if not a.no_extra and a.dtype == "bf16":

@@ -227,6 +227,11 @@ template <> struct Chunk<float> {
         for (int e = 0; e < 4; ++e) v[e] = u2f(c[e]);
     }
     static __device__ __forceinline__ u32x4 pack(const float (&v)[4]) { return u32x4{f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])}; }
+    // sum and sum of squares of the chunk's values as stored
+    static __device__ __forceinline__ void moments(const u32x4&, const float (&v)[4], float& s, float& q) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { s += v[e]; q = fmaf(v[e], v[e], q); }
+    }
 };
 template <> struct Chunk<uint16_t> {
     static constexpr int N = 8;
@@ -236,6 +241,17 @@ template <> struct Chunk<uint16_t> {
     }
     static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
         return u32x4{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])};
+    }
+    // sum and sum of squares of the chunk's values as stored (the rounded bf16 pairs, two per dot instruction)
+    static __device__ __forceinline__ void moments(const u32x4& c, const float (&)[8], float& s, float& q) {
+        typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2v;
+        const bf16x2v one2 = __builtin_bit_cast(bf16x2v, 0x3f803f80u);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const bf16x2v w = __builtin_bit_cast(bf16x2v, (uint32_t)c[e]);
+            s = __builtin_amdgcn_fdot2_f32_bf16(w, one2, s, false);
+            q = __builtin_amdgcn_fdot2_f32_bf16(w, w, q, false);
+        }
     }
 };
 
@@ -672,6 +688,18 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                         for (int e = 0; e < 4; ++e) c0[b][4 * q + e] = v[e];
                     }
                 }
+                if constexpr (RL) {
+                    // the beta of the LayerNorm that the epilogue re-forms on the residual is a per-column constant too
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int n = n0 + wn * WNO + b * 32 + 8 * q + 4 * lg;      // N is a multiple of 4 here
+                        if (n < p.N) {
+                            const f32x4 v = *(const f32x4*)(p.res_beta + n);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) c0[b][4 * q + e] += v[e];
+                        }
+                    }
+                }
             }
         }
         auto k_slab = [&](int kt, auto ifirst) {
@@ -846,16 +874,15 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             // EPI_RESLN: this thread's columns are the same in every chunk it handles (the chunk index advances by a
             // multiple of the chunks per row), so the norm's gamma / beta for them are loaded once per tile
             static_assert(NT % CPR == 0, "a thread keeps its chunk column");
-            float gq[RL ? EPCO : 1], bq[RL ? EPCO : 1];
+            float gq[RL ? EPCO : 1];
             if constexpr (RL) {
                 const int nq = n0 + (tid % CPR) * EPCO;          // N is a multiple of the chunk here: whole chunks in or out
 #pragma unroll
                 for (int e = 0; e < EPCO; e += 4) {
                     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
                     const f32x4 gv = nq + e < p.N ? *(const f32x4*)(p.res_gamma + nq + e) : zero;
-                    const f32x4 bv = nq + e < p.N ? *(const f32x4*)(p.res_beta + nq + e) : zero;
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) { gq[e + k] = gv[k]; bq[e + k] = bv[k]; }
+                    for (int k = 0; k < 4; ++k) gq[e + k] = gv[k];
                 }
             }
             // last step of a staged chunk: residual (plain, or LayerNorm re-formed from the raw residual rows and
@@ -879,7 +906,15 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                 const int m = m0 + rt;
                 const int n = n0 + cc * EPCO;
                 const bool in = m < p.M && n < p.N;
-                if constexpr (EPI == EPI_RES) out = add_chunk<OutT>(out, rres);
+                if constexpr (EPI == EPI_RES) {
+                    out = add_chunk<OutT>(out, rres);
+                    // keep the sum in front of the range test: sunk into the conditional store, every chunk's first use of
+                    // its residual registers sits behind a branch, and the wait-count pass then puts a full vmcnt(0) (which
+                    // also waits for the stores of the chunks before) in front of each of them
+                    uint32_t o0 = out[0], o1 = out[1], o2 = out[2], o3 = out[3];
+                    asm volatile("" : "+v"(o0), "+v"(o1), "+v"(o2), "+v"(o3));
+                    out = u32x4{o0, o1, o2, o3};
+                }
                 if constexpr (RL) {
                     const float rs = rstat[0], rsm = rstat[1];
                     float xr[EPCO], g[EPCO], o[EPCO];
@@ -887,16 +922,14 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
                     Chunk<OutT>::unpack(out, g);
                     // sum and sum of squares of the row's columns in this tile (columns past N contribute 0: gamma, beta,
                     // bias and the products are 0 there); the two reductions are independent and interleave
+                    // (the norm's beta travels with the bias in the accumulators' starting values)
                     float sum = 0.f, sq = 0.f;
 #pragma unroll
-                    for (int e = 0; e < EPCO; ++e) {
-                        o[e] = fmaf(fmaf(xr[e], rs, -rsm), gq[e], bq[e] + g[e]);
-                        sum += o[e];
-                        sq = fmaf(o[e], o[e], sq);
-                    }
+                    for (int e = 0; e < EPCO; ++e) o[e] = fmaf(fmaf(xr[e], rs, -rsm), gq[e], g[e]);
+                    out = Chunk<OutT>::pack(o);
+                    Chunk<OutT>::moments(out, o, sum, sq);
                     sum = group_sum<CPR>(sum);
                     sq = group_sum<CPR>(sq);
-                    out = Chunk<OutT>::pack(o);
                     if (cc == 0 && m < p.M) {
                         const f32x2_t pr = {sum, sq};
                         *(f32x2_t*)(p.part_out + ((int64_t)(n0 / BNO) * p.M + m) * 2) = pr;
@@ -926,19 +959,28 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p)
             // Barriers here are LDS-only (a fence would also wait for the global stores of earlier bands).
             if constexpr (NREG == 2) {
                 // two regions: band a+1 is converted and written while band a's staged rows are on their
-                // way back from LDS, one barrier per band
+                // way back from LDS, one barrier per band.
+                // Residual chunks: the memory counter retires in issue order, so a load requested behind a band's stores
+                // can only be waited for together with those stores (a round trip to HBM per band).  All of the tile's
+                // residual chunks are therefore requested before its first store: the first RESAHEAD bands up front, the
+                // rest as soon as the accumulators of the bands already staged have freed their registers.
+                constexpr bool HASRES = EPI == EPI_RES || RL;
+                constexpr int RESAHEAD = TM < 2 ? TM : 2;
+                u32x4 res[HASRES ? TM : 1][PER];
                 issue_next();
+                if constexpr (HASRES) static_for<RESAHEAD>([&](auto ia) { fetch_res(ia, res[decltype(ia)::value]); });
                 stage_band(std::integral_constant<int, 0>{});
                 static_for<TM>([&](auto ia) {
                     constexpr int a = decltype(ia)::value;
                     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                    u32x4 val[PER], res[PER];
+                    u32x4 val[PER];
                     f32x2_t rst[PER];
                     fetch_band(ia, val);
                     fetch_rstats(ia, rst);
-                    fetch_res(ia, res);
                     if constexpr (a + 1 < TM) stage_band(std::integral_constant<int, a + 1>{});
-                    store_band(ia, val, res, rst);
+                    if constexpr (HASRES && a == 0 && TM > RESAHEAD)
+                        static_for<TM - RESAHEAD>([&](auto ib) { fetch_res(std::integral_constant<int, decltype(ib)::value + RESAHEAD>{}, res[decltype(ib)::value + RESAHEAD]); });
+                    store_band(ia, val, res[HASRES ? a : 0], rst);
                 });
             } else {
                 issue_next();
