@@ -90,6 +90,39 @@ def median(v):
     return float(np.median(np.asarray(v, np.float64)))
 
 
+def forward_kernel_times(backend, enc, cfg, forwards=8):
+    """Durations of the layer's launches INSIDE whole forwards: the layer entry points record a lap event at entry and after
+    each of their kernels (grl_timer_lap_trace), `forwards` forwards run back to back behind two untimed ones, and every
+    interval is attributed to the launch it follows (a residual-type GEMM's interval includes its 3-5 us moment merge).
+    Returns {launch name: {ms (mean), median_ms, n}} and "layer_ms": what the kernels do under the forward's sustained
+    load, next to the back-to-back table of kernel_table()."""
+    from grilly_amd import _lib as L
+    import ctypes
+    core = backend.core
+    fused = getattr(enc, "fused", False)
+    names = ["gemm_qkv_ln", "fa2_fwd", "gemm_out_resln", "gemm_ffn1_ln_gelu", "gemm_ffn2_resln"] if fused else \
+            ["gemm_qkv", "fa2_fwd", "gemm_out", "layernorm_residual", "gemm_ffn1_gelu", "gemm_ffn2", "layernorm_residual"]
+    per_layer = len(names) + 1                         # the mark at layer entry
+    assert 1 + per_layer * cfg.layers <= 256
+    acc = {}
+    for _ in range(2):
+        enc.launch(pool=True)
+    nxt, ms = ctypes.c_int(), ctypes.c_float()
+    for _ in range(forwards):
+        L.check(core.lib.grl_timer_lap_trace(core.ctx, 0, None))
+        enc.launch(pool=True)
+        L.check(core.lib.grl_timer_lap_trace(core.ctx, -1, ctypes.byref(nxt)))
+        assert nxt.value == 1 + per_layer * cfg.layers, (nxt.value, per_layer, cfg.layers)
+        for layer in range(cfg.layers):
+            base = 1 + layer * per_layer               # index of the layer's entry mark
+            for j, nm in enumerate(names):
+                L.check(core.lib.grl_timer_lap_ms(core.ctx, base + j, base + j + 1, ctypes.byref(ms)))
+                acc.setdefault(nm, []).append(float(ms.value))
+    out = {nm: {"ms": round(float(np.mean(v)), 4), "median_ms": round(median(v), 4), "n": len(v)} for nm, v in acc.items()}
+    out["layer_ms"] = round(sum(sum(v) for v in acc.values()) / (forwards * cfg.layers), 4)
+    return out
+
+
 def download_rows(core, buf, row0, nrows, ncols, code):
     """rows [row0, row0+nrows) of a device matrix with `ncols` columns -> float32 numpy"""
     from grilly_amd import _lib as L
@@ -651,39 +684,57 @@ def main():
     # hidden states of the first sequences after the timed steps (the pooled output is computed from them)
     gpu_hidden = download_rows(backend.core, enc.x, 0, nseq * S, cfg.d_model, enc.code).reshape(nseq, S, cfg.d_model)
     if not a.no_kernels:
+        # the layer's launches timed inside whole forwards first (the GPU is in the forward's power state), then back to back
+        fk = forward_kernel_times(backend, enc, cfg)
         kt = kernel_table(backend, enc, B, S, a.kernel_reps, check=not a.no_cpu_baseline)
         out["kernels"] = kt
+        for nm, r in fk.items():
+            if nm in kt and kt[nm].get("flops"):
+                r["frac_mfma"] = round(kt[nm]["flops"] / (r["ms"] * 1e-3) / peak, 4)
+            elif nm in kt:
+                r["frac_hbm"] = round(kt[nm]["bytes"] / (r["ms"] * 1e-3) / 8e12, 4)
+        out["forward_kernels"] = fk
         # dominant kernel = the GEMM instantiation with the largest share of the forward.  With the LayerNorms folded
         # into the GEMMs that is the one whose epilogue adds the re-formed LayerNorm residual and reduces the row
         # statistics (out-proj and FFN2: two launches per layer); in the seven-launch layer the plain instantiation
-        # (QKV, out-proj, FFN2: three launches per layer).  Average FLOPs per launch over average duration per launch.
+        # (QKV, out-proj, FFN2: three launches per layer).  Average FLOPs per launch over average duration per launch,
+        # the durations being those INSIDE the forward (lap events between the layer's launches); the same launches
+        # timed back to back in a table of their own are reported next to it.
         fused = getattr(enc, "fused", False)
         names = ("gemm_out_resln", "gemm_ffn2_resln") if fused else ("gemm_qkv", "gemm_out", "gemm_ffn2")
         tname = "float" if a.dtype == "fp32" else "bf16"
         kname = f"gemm_nt_dma_kernel<{tname},{tname},256,256,2,4,{'EPI_RESLN' if fused else 'EPI_NONE'}>"
         g = [kt[k] for k in names]
         avg_flops = sum(r["flops"] for r in g) / len(g)
-        avg_ms = sum(r["ms"] for r in g) / len(g)
-        clk = sum(r["shader_clock_ghz"] for r in g) / len(g)
-        ach = avg_flops / (avg_ms * 1e-3) / 1e12
+        fwd_ms = sum(fk[k]["ms"] for k in names) / len(names)
+        fwd_med = sum(fk[k]["median_ms"] for k in names) / len(names)
+        ach = avg_flops / (fwd_ms * 1e-3) / 1e12
+        tab_ms = sum(r["ms"] for r in g) / len(g)
+        tab_clk = sum(r["shader_clock_ghz"] for r in g) / len(g)
+        tab = avg_flops / (tab_ms * 1e-3) / 1e12
         traffic, at_commit = gemm_traffic(a.dtype, B, S, kname)
         out["roofline"] = {"kernel": kname, "launches": list(names),
                            "bound": "mfma", "achieved": round(ach, 1), "peak": peak / 1e12, "unit": "TFLOP/s",
                            "frac": round(ach * 1e12 / peak, 4),
                            "traffic": traffic, "traffic_measured_at_commit": at_commit,
                            "algorithmic_bytes": sum(r["bytes"] for r in g) / len(g),
-                           "avg_launch_ms": round(avg_ms, 4), "median_launch_ms": round(sum(r["median_ms"] for r in g) / len(g), 4),
+                           "avg_launch_ms": round(fwd_ms, 4), "median_launch_ms": round(fwd_med, 4),
+                           "launches_timed": sum(fk[k]["n"] for k in names),
                            "flops_per_launch": avg_flops,
-                           "shader_clock_ghz": round(clk, 3), "nominal_clock_ghz": NOMINAL_GHZ,
-                           "frac_at_measured_clock": round(ach * 1e12 / (peak * clk / NOMINAL_GHZ), 4),
+                           "shader_clock_ghz": round(fwd_clock, 3), "nominal_clock_ghz": NOMINAL_GHZ,
+                           "frac_at_measured_clock": round(ach * 1e12 / (peak * fwd_clock / NOMINAL_GHZ), 4),
                            "launches_per_step": len(names) * cfg.layers,
+                           "back_to_back": {"avg_launch_ms": round(tab_ms, 4), "median_launch_ms": round(sum(r["median_ms"] for r in g) / len(g), 4),
+                                            "achieved": round(tab, 1), "frac": round(tab * 1e12 / peak, 4), "shader_clock_ghz": round(tab_clk, 3),
+                                            "frac_at_measured_clock": round(tab * 1e12 / (peak * tab_clk / NOMINAL_GHZ), 4)},
                            "clock_note": "peak = 256 CUs x 4 SIMDs x 1024 bf16 FLOP per cycle (fp32: 64) x the nominal 2.4 GHz; under the board's "
-                                         "power limit the timed launches run at shader_clock_ghz (probe kernel beside them), and "
-                                         "frac_at_measured_clock is the same achieved rate against the peak at that clock",
-                           "note": "launches timed back to back on the layer's real operands; per-kernel durations move by about +-10 % "
-                                   "with the power state of the board and differ by up to 20 % between boxes (the same launches inside "
-                                   "the forward, between other kernels, are not systematically slower or faster): see "
-                                   "profiles/encoder_forward_bert_base_bf16_kernel_stats.md"}
+                                         "power limit the launches run at shader_clock_ghz (probe kernel beside the forward, or beside the "
+                                         "back-to-back launches), and frac_at_measured_clock is the same achieved rate against the peak at that clock",
+                           "note": "achieved / frac / avg_launch_ms: the kernel's launches inside whole forwards (lap events between the "
+                                   "layer's launches; a launch's interval includes its 3-5 us moment-merge kernel), i.e. under the sustained "
+                                   "load of the timed region; back_to_back: the same launches in a table of their own (`kernels`), where "
+                                   "the board often holds a higher clock because the load comes in bursts of a few milliseconds between "
+                                   "host-side checks.  Both move with the box (up to 20 % between boxes)."}
         if fused:
             # the plain instantiation (what linear / fused_qkv_projection launch; the dominant kernel of the seven-launch
             # layer and of earlier measurements of this benchmark), same definition: mean FLOPs over mean duration

@@ -61,6 +61,7 @@ SIGNATURES = {
     "grl_timer_stop": (c_int, [c_void_p, ctypes.POINTER(c_float)]),
     "grl_timer_lap": (c_int, [c_void_p, c_int]),
     "grl_timer_lap_ms": (c_int, [c_void_p, c_int, c_int, ctypes.POINTER(c_float)]),
+    "grl_timer_lap_trace": (c_int, [c_void_p, c_int, ctypes.POINTER(c_int)]),
     "grl_mfma_probe": (c_int, [c_void_p, c_int, c_void_p, c_int, ctypes.POINTER(c_float), ctypes.POINTER(ctypes.c_double)]),
     "grl_clock_probe_begin": (c_int, [c_void_p, c_float]),
     "grl_clock_probe_end": (c_int, [c_void_p, ctypes.POINTER(c_float)]),

@@ -17,6 +17,7 @@ struct grl_ctx {
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     hipEvent_t laps[GRL_MAX_LAPS] = {};   // lap events (grl_timer_lap), created on first use
+    int lap_next = -1;                    // >= 0: the layer entry points record a lap after each of their launches (grl_timer_lap_trace)
     hipDeviceProp_t prop{};
     std::mutex mu;          // guards the pool
     std::mutex timer_mu;    // guards the event pair
@@ -42,6 +43,10 @@ struct grl_ctx {
 int grl_rope_table_get(grl_ctx* c, int S, int D, float base, float scaling, int style, const float** out);
 
 void grl_set_error(const char* fmt, ...);
+
+// one lap event behind the launches enqueued so far, when a lap trace is on (and has indices left); used by the
+// entry points that launch several kernels, so that a caller can time the launches inside them
+void grl_lap_mark(grl_ctx* c);
 
 #define GRL_CHECK_HIP(expr)                                                              \
     do {                                                                                 \

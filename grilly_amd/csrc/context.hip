@@ -242,6 +242,34 @@ extern "C" int grl_timer_lap_ms(grl_ctx* c, int from, int to, float* ms) {
     return GRL_OK;
 }
 
+// lap trace: the multi-launch entry points (the encoder layers) record lap first, first+1, ... after each of their launches
+extern "C" int grl_timer_lap_trace(grl_ctx* c, int first, int* next) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_timer_lap_trace: null context");
+    GRL_REQUIRE(first >= -1 && first < GRL_MAX_LAPS, GRL_ERR_ARG, "grl_timer_lap_trace: first index %d outside -1..%d", first, GRL_MAX_LAPS - 1);
+    int old;
+    {
+        std::lock_guard<std::mutex> lk(c->timer_mu);
+        old = c->lap_next;
+        c->lap_next = -1;
+    }
+    if (next) *next = old;
+    if (first < 0) return GRL_OK;
+    int rc = grl_timer_lap(c, first);          // the trace starts with a lap of its own: index `first`
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lk(c->timer_mu);
+    c->lap_next = first + 1;
+    return GRL_OK;
+}
+void grl_lap_mark(grl_ctx* c) {
+    int idx;
+    {
+        std::lock_guard<std::mutex> lk(c->timer_mu);
+        if (c->lap_next < 0 || c->lap_next >= GRL_MAX_LAPS) return;
+        idx = c->lap_next++;
+    }
+    grl_timer_lap(c, idx);
+}
+
 // ---- matrix-core ceiling probe ---------------------------------------------------------------------------------
 // Nothing but MFMAs on register-resident operands: eight waves per CU (two per SIMD, as in the GEMM kernels), each
 // with the GEMM wave tile's accumulators (128 registers) and two alternating sets of operand fragments, no memory

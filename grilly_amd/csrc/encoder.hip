@@ -33,14 +33,22 @@ extern "C" int grl_bert_layer_fwd(grl_ctx* c, int dtype, int64_t B, int64_t S, i
     char* proj = attn + pad(M * d * es);
     char* ff = proj + pad(M * d * es);
     int rc;
+    grl_lap_mark(c);
     if ((rc = grl_gemm_nt(c, dtype, dtype, M, 3 * d, d, x, w->w_qkv, w->b_qkv, qkv, GRL_EPI_NONE))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_fa2_fwd_strided(c, dtype, B, S, H, D, qkv, qkv + d * es, qkv + 2 * d * es, mask, attn,
                                   3 * d, 3 * d, 3 * d, d, 1.0f / sqrtf((float)D), 0, GRL_ROPE_NONE, 10000.f, 1.f))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_gemm_nt(c, dtype, dtype, M, d, d, attn, w->w_o, w->b_o, proj, GRL_EPI_NONE))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_layernorm(c, dtype, M, d, x, proj, w->ln1_g, w->ln1_b, eps, x))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_gemm_nt(c, dtype, dtype, M, d_ff, d, x, w->w_ff1, w->b_ff1, ff, GRL_EPI_GELU))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_gemm_nt(c, dtype, dtype, M, d, d_ff, ff, w->w_ff2, w->b_ff2, proj, GRL_EPI_NONE))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_layernorm(c, dtype, M, d, x, proj, w->ln2_g, w->ln2_b, eps, x))) return rc;
+    grl_lap_mark(c);
     return GRL_OK;
 }
 
@@ -75,11 +83,17 @@ extern "C" int grl_bert_layer_fwd_fused(grl_ctx* c, int dtype, int64_t B, int64_
     float* stats1 = (float*)(ff + pad(M * d_ff * es));
     char* part = (char*)stats1 + pad(M * 8);
     int rc;
+    grl_lap_mark(c);
     if ((rc = grl_ln_gemm_nt_stats(c, dtype, dtype, M, 3 * d, d, r, w->ws_qkv, w->c_qkv, w->bf_qkv, stats, qkv, GRL_EPI_NONE))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_fa2_fwd_strided(c, dtype, B, S, H, D, qkv, qkv + d * es, qkv + 2 * d * es, mask, attn,
                                   3 * d, 3 * d, 3 * d, d, 1.0f / sqrtf((float)D), 0, GRL_ROPE_NONE, 10000.f, 1.f))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_gemm_nt_resln(c, dtype, M, d, d, attn, w->w_o, w->b_o, r, stats, w->in_g, w->in_b, r, eps, stats1, part))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_ln_gemm_nt_stats(c, dtype, dtype, M, d_ff, d, r, w->ws_ff1, w->c_ff1, w->bf_ff1, stats1, ff, GRL_EPI_GELU))) return rc;
+    grl_lap_mark(c);
     if ((rc = grl_gemm_nt_resln(c, dtype, M, d, d_ff, ff, w->w_ff2, w->b_ff2, r, stats1, w->ln1_g, w->ln1_b, r, eps, stats, part))) return rc;
+    grl_lap_mark(c);
     return GRL_OK;
 }

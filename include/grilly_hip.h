@@ -110,6 +110,12 @@ int grl_timer_stop(grl_ctx* ctx, float* elapsed_ms);   /* synchronises */
  * per-launch durations (for medians) without host synchronisations between the launches. */
 int grl_timer_lap(grl_ctx* ctx, int index);
 int grl_timer_lap_ms(grl_ctx* ctx, int from, int to, float* elapsed_ms);
+/* Lap trace: between grl_timer_lap_trace(ctx, first, NULL) and grl_timer_lap_trace(ctx, -1, &next) the encoder-layer entry
+ * points (grl_bert_layer_fwd, grl_bert_layer_fwd_fused) record a lap at entry and after each kernel they launch, with
+ * indices first+1, first+2, ... (lap `first` is recorded by the call that turns the trace on; marks beyond index 255 are
+ * dropped).  `next` receives the index the next mark would have used, or -1 when no trace was on.  For timing the
+ * launches inside a forward; one trace per context at a time. */
+int grl_timer_lap_trace(grl_ctx* ctx, int first, int* next);
 /* Matrix-core ceiling probe (measurement aid, no counterpart in the reference): every CU runs eight waves that issue
  * nothing but MFMAs on register-resident operands (kind 0: v_mfma_f32_32x32x16_bf16, kind 1: v_mfma_f32_16x16x32_bf16)
  * for `iters` loop iterations, after one untimed warm-up launch.  `operands` points to 64 KiB of device memory whose

@@ -180,3 +180,46 @@ def test_fused_encoder_equals_the_unfused_one(backend, dtype, d, heads, ff, S):
     pf, pp = fused.forward(ids, mask, pool=True), plain.forward(ids, mask, pool=True)
     assert O.max_rel(pf, pp) < (1e-4 if dtype == "fp32" else 1e-2)
     fused.release_activations(); plain.release_activations()
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_lap_trace_marks_every_launch_of_the_layers(backend, fused):
+    """With a lap trace on, each layer call records a lap at entry and after each of its kernels (five with the folded
+    LayerNorms, seven without); the intervals are non-negative and add up to the time between the first and the last
+    lap; with the trace off the layers record nothing; the hidden states do not depend on the trace."""
+    c = backend.core
+    cfg = EncoderConfig(layers=3, d_model=128, heads=2, d_ff=256, vocab=100, max_pos=64)
+    w = random_bert_weights(cfg, seed=5)
+    enc = BertEncoder(backend, cfg, w, dtype="bf16", fused=fused)
+    rng = np.random.default_rng(5)
+    ids = rng.integers(0, cfg.vocab, (4, 40))
+    want = enc.forward(ids, None, pool=False)
+    per_layer = (5 if fused else 7) + 1
+    nxt, ms = ctypes.c_int(123), ctypes.c_float()
+    L.check(c.lib.grl_timer_lap_trace(c.ctx, -1, ctypes.byref(nxt)))
+    assert nxt.value == -1                                  # no trace was on
+    L.check(c.lib.grl_timer_lap_trace(c.ctx, 10, None))
+    got = enc.forward(ids, None, pool=False)
+    L.check(c.lib.grl_timer_lap_trace(c.ctx, -1, ctypes.byref(nxt)))
+    assert nxt.value == 11 + per_layer * cfg.layers
+    np.testing.assert_array_equal(got, want)
+    parts = []
+    for i in range(10, nxt.value - 1):
+        L.check(c.lib.grl_timer_lap_ms(c.ctx, i, i + 1, ctypes.byref(ms)))
+        assert ms.value >= 0.0
+        parts.append(ms.value)
+    L.check(c.lib.grl_timer_lap_ms(c.ctx, 10, nxt.value - 1, ctypes.byref(ms)))
+    assert abs(sum(parts) - ms.value) < 0.05 + 0.05 * ms.value
+    # off again: a forward leaves the next index alone
+    enc.forward(ids, None, pool=False)
+    L.check(c.lib.grl_timer_lap_trace(c.ctx, -1, ctypes.byref(nxt)))
+    assert nxt.value == -1
+    # marks past the last event index are dropped, the forward still runs
+    L.check(c.lib.grl_timer_lap_trace(c.ctx, 250, None))
+    np.testing.assert_array_equal(enc.forward(ids, None, pool=False), want)
+    L.check(c.lib.grl_timer_lap_trace(c.ctx, -1, ctypes.byref(nxt)))
+    assert nxt.value == 256
+    assert c.lib.grl_timer_lap_trace(c.ctx, 256, None) == L.ERR_ARG
+    assert c.lib.grl_timer_lap_trace(c.ctx, -2, None) == L.ERR_ARG
+    assert c.lib.grl_timer_lap_trace(None, 0, None) == L.ERR_ARG
+    enc.release_activations()
