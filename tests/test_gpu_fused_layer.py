@@ -9,7 +9,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from conftest import TOL_F32, TOL_BF16
+from conftest import TOL_F32, TOL_BF16, sweep_rounds
 from oracle import oracle_np as O
 from grilly_amd import _lib as L
 from grilly_amd import BertEncoder, EncoderConfig, random_bert_weights
@@ -223,3 +223,86 @@ def test_lap_trace_marks_every_launch_of_the_layers(backend, fused):
     assert c.lib.grl_timer_lap_trace(c.ctx, -2, None) == L.ERR_ARG
     assert c.lib.grl_timer_lap_trace(None, 0, None) == L.ERR_ARG
     enc.release_activations()
+
+
+def test_resln_and_given_statistics_gemms_randomized(backend):
+    """Seeded sweep over the two GEMM entry points of the LayerNorm-free layer through the C ABI: both storage types,
+    ragged M, widths in 16-byte steps, one to six K slabs, big-tile and small-tile launches, with and without a bias,
+    in place and out of place; outputs against float64 on every row, row statistics against the moments of the stored
+    rows.  GRILLY_SWEEP_ROUNDS continues the stream."""
+    c = backend.core
+    rng = np.random.default_rng(4242)
+    worst = {"fp32": 0.0, "bf16": 0.0}
+    for case in range(36 * sweep_rounds()):
+        if case and case % 50 == 0:
+            print("sweep case", case, flush=True)
+        dtype = "bf16" if case % 2 else "fp32"
+        code, es = _code(dtype), (2 if dtype == "bf16" else 4)
+        slab, chunk = (64, 8) if dtype == "bf16" else (32, 4)
+        K = slab * int(rng.integers(1, 7))
+        if case % 6 == 0:                                   # enough 256 x 256 tiles for the persistent big-tile kernels
+            M, N = int(rng.integers(3100, 4300)), chunk * int(rng.integers(3100 // chunk, 4300 // chunk))
+            while ((M + 255) // 256) * ((N + 255) // 256) < 192:
+                N += 256
+        else:
+            M, N = int(rng.integers(1, 700)), chunk * int(rng.integers(1, 700 // chunk))
+        tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+        eps_r, eps = 1e-5, 1e-6
+        has_bias, inplace = rng.random() < 0.7, rng.random() < 0.5
+        A = _q(dtype, rng.standard_normal((M, K)).astype(np.float32))
+        W = _q(dtype, (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32))
+        b = rng.standard_normal(N).astype(np.float32) if has_bias else None
+        R = _q(dtype, (rng.uniform(0.3, 3.0) * rng.standard_normal((M, N)) + rng.standard_normal((M, 1))).astype(np.float32))
+        g = (1 + 0.2 * rng.standard_normal(N)).astype(np.float32)
+        bt = (0.3 * rng.standard_normal(N)).astype(np.float32)
+        rst = _stats(R, eps_r).astype(np.float32)
+        tag = (case, dtype, M, K, N, has_bias, inplace)
+        dA, dW, dR, dst, dg, dbt = c.upload(A, code), c.upload(W, code), c.upload(R, code), c.upload(rst), c.upload(g), c.upload(bt)
+        db = c.upload(b) if has_bias else None
+        dC = dR if inplace else c.alloc(M * N * es)
+        so, wk = c.alloc(M * 8), c.alloc(c.lib.grl_gemm_nt_resln_workspace(M, N))
+        # second entry point: y2 = LN(y; g2, bt2) . W2^T + b2 from the statistics the first one wrote
+        N2 = chunk * int(rng.integers(1, 40))
+        K2ok = N % slab == 0                                # its K is the first one's N: whole slabs only
+        try:
+            L.check(c.lib.grl_gemm_nt_resln(c.ctx, code, M, N, K, dA.ptr, dW.ptr, db.ptr if db else None, dR.ptr, dst.ptr, dg.ptr, dbt.ptr,
+                                            dC.ptr, eps, so.ptr, wk.ptr), f"gemm_nt_resln {tag}")
+            y = c.download(dC, (M, N), code)
+            stats = c.download(so, (M, 2))
+            ref = O.truth_linear(A, W, b) + O.truth_layernorm(R, g, bt, eps_r)
+            assert np.isfinite(y).all() and np.isfinite(stats).all(), tag
+            err = O.max_rel(y, ref)
+            worst[dtype] = max(worst[dtype], err)
+            assert err < tol, (tag, err)
+            want = _stats(y, eps)
+            stol = 5e-3 if dtype == "bf16" else 2e-4
+            assert O.max_rel(stats[:, 0], want[:, 0]) < stol, tag
+            assert np.abs(stats[:, 1] - want[:, 1]).max() < stol * max(1.0, np.abs(want[:, 1]).max()), tag
+            if K2ok:
+                W2 = _q(dtype, (rng.standard_normal((N2, N)) / np.sqrt(N)).astype(np.float32))
+                g2 = (1 + 0.2 * rng.standard_normal(N)).astype(np.float32)
+                bt2 = (0.3 * rng.standard_normal(N)).astype(np.float32)
+                b2 = rng.standard_normal(N2).astype(np.float32)
+                epi = "gelu" if rng.random() < 0.5 else "none"
+                dW2, dg2, dbt2, db2 = c.upload(W2, code), c.upload(g2), c.upload(bt2), c.upload(b2)
+                ws, cs, bf, out = c.alloc(N2 * N * es), c.alloc(N2 * 4), c.alloc(N2 * 4), c.alloc(M * N2 * es)
+                try:
+                    L.check(c.lib.grl_ln_fold(c.ctx, code, N2, N, dW2.ptr, dg2.ptr, dbt2.ptr, db2.ptr, ws.ptr, cs.ptr, bf.ptr), "fold")
+                    L.check(c.lib.grl_ln_gemm_nt_stats(c.ctx, code, code, M, N2, N, dC.ptr, ws.ptr, cs.ptr, bf.ptr, so.ptr, out.ptr,
+                                                       L.EPI_GELU if epi == "gelu" else L.EPI_NONE), f"ln_gemm_nt_stats {tag}")
+                    y2 = c.download(out, (M, N2), code)
+                    ref2 = O.truth_linear(O.truth_layernorm(y, g2, bt2, eps), W2, b2, epi)
+                    assert np.isfinite(y2).all(), tag
+                    err2 = O.max_rel(y2, ref2)
+                    assert err2 < tol * (1.5 if dtype == "bf16" else 2.0), (tag, N2, epi, err2)
+                finally:
+                    for t in (dW2, dg2, dbt2, db2, ws, cs, bf, out):
+                        t.free()
+        finally:
+            for t in (dA, dW, dR, dst, dg, dbt, so, wk):
+                t.free()
+            if db:
+                db.free()
+            if not inplace:
+                dC.free()
+    print("worst", worst)
