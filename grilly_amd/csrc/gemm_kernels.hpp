@@ -1060,6 +1060,23 @@ __global__ __launch_bounds__(256) void gemm_nt_scalar_kernel(GemmArgs p) {
 }
 
 // ------------------------------------------------------------------ host dispatch
+// 256 x 256 tiles (one persistent workgroup per CU) or 128 x 128 tiles (two per CU)?  Big tiles move half the operand
+// bytes per FLOP, but a launch is as long as its fullest CU: n_big tiles take ceil(n_big / CUs) tile times, and e.g. 320
+// tiles on 256 CUs leave the second pass three quarters empty.  Modelled in units of one 128 x 128 tile's work at full
+// speed: a pass of big tiles costs 4; a full pass of small tiles (two share a CU) 2 x p, a last pass that leaves every
+// CU at most one of them 1 x p, with p the small tile's handicap (measured: none in fp32, whose matrix rate is the
+// bound; 1.17 in bf16, where the global -> LDS path is).  Small tiles are taken when the model gives them 7 % or more
+// (measured at 2048 ... 32768 rows against 384 ... 4096 columns: 13 - 30 % faster where the model says so, within 4 %
+// of the better choice everywhere); below 192 big tiles they are taken anyway.
+static inline bool prefer_big_tiles(int64_t n_big, int64_t n_small, int64_t cus, size_t elem_size) {
+    if (n_big < 192) return false;
+    const double p = elem_size == 4 ? 1.0 : 1.17;
+    const double t_big = 4.0 * (double)((n_big + cus - 1) / cus);
+    const int64_t full = n_small / (2 * cus), rest = n_small % (2 * cus);
+    const double t_small = p * (2.0 * (double)full + (rest == 0 ? 0.0 : (rest <= cus ? 1.0 : 2.0)));
+    return !(t_small < 0.93 * t_big);
+}
+
 template <typename T, typename OutT, int EPI, bool DUAL, bool LN = false>
 static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     const int64_t epc = 16 / (int64_t)sizeof(T);
@@ -1075,7 +1092,7 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     }
     // Tile choice.  The direct-to-LDS kernel needs whole 128-byte K slabs; the 256x256 tile is
     // used once it yields enough workgroups to occupy most of the 256 CUs, else 128x128 tiles.
-    // GRL_GEMM_VARIANT (1..4) forces one variant, for tuning runs.
+    // GRL_GEMM_VARIANT (1..5) forces one variant, for tuning runs.
     static const int forced = [] { const char* e = getenv("GRL_GEMM_VARIANT"); return e ? atoi(e) : 0; }();
     // band height of the tile walk: rows of 8 KiB and more do better with narrow bands (measured)
     static const int group = [] { const char* e = getenv("GRL_GEMM_GROUP"); return e ? atoi(e) : 0; }();
@@ -1086,11 +1103,19 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     GRL_REQUIRE(sm * sn < (1LL << 31), GRL_ERR_SHAPE, "gemm: too many tiles");
     GRL_REQUIRE(a.K * (int64_t)sizeof(T) * 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: K too large (256 rows must span < 2 GiB)");
     const bool slabs = a.K % bke == 0;
-    const bool big = big_m * big_n >= 192;
     const int64_t cus = c->prop.multiProcessorCount;     // one 128 KiB-LDS workgroup per CU, two of the 64 KiB ones
-    int variant = slabs ? (big ? 3 : 4) : (big ? 1 : 2);
-    if (forced >= 1 && forced <= 4 && (slabs || forced <= 2)) variant = forced;
+    const bool big = prefer_big_tiles(big_m * big_n, sm * sn, cus, sizeof(T));
+    // problems of a few 128 x 128 tiles (single sentences, the README-sized operators) leave most CUs idle and pad M up
+    // to 128 rows: 64 x 64 tiles give them four times the workgroups, each with a quarter of the serial K loop
+    const bool tiny = sm * sn <= 16;
+    const int64_t tm = (a.M + 63) / 64, tn = (a.N + 63) / 64;      // 64 output columns per tile (with two weights: 128 LDS rows)
+    int variant = tiny ? 5 : (slabs ? (big ? 3 : 4) : (big ? 1 : 2));
+    if (forced >= 1 && forced <= 5 && (slabs || forced <= 2 || forced == 5)) variant = forced;
     switch (variant) {
+        case 5:
+            a.tiles_m = (int)tm; a.tiles_n = (int)tn;
+            hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 64, (DUAL ? 128 : 64), 2, 2, EPI, DUAL, LN>), dim3((unsigned)(tm * tn)), dim3(256), 0, c->stream, a);
+            break;
         case 1:
             a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
             hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 256, 256, 2, 2, EPI, DUAL, LN>), dim3((unsigned)(big_m * big_n)), dim3(256), 0, c->stream, a);
@@ -1130,7 +1155,7 @@ int launch_gemm_resln(grl_ctx* c, GemmArgs& a, int* tile_cols) {
     const int64_t sm = (a.M + 127) / 128, sn = (a.N + 127) / 128;
     GRL_REQUIRE(sm * sn < (1LL << 31), GRL_ERR_SHAPE, "gemm: too many tiles");
     const int64_t cus = c->prop.multiProcessorCount;
-    if (big_m * big_n >= 192) {
+    if (prefer_big_tiles(big_m * big_n, sm * sn, cus, sizeof(T))) {
         a.tiles_m = (int)big_m; a.tiles_n = (int)big_n; *tile_cols = 256;
         hipLaunchKernelGGL((gemm_nt_dma_kernel<T, OutT, 256, 256, 2, 4, EPI_RESLN, false, false>), dim3((unsigned)std::min<int64_t>(big_m * big_n, cus)), dim3(512), 0, c->stream, a);
     } else {

@@ -202,3 +202,34 @@ def test_randomized_shapes_over_every_kernel_variant(backend):
         worst[dtype] = max(worst[dtype], err)
         assert err < tol(dtype), (case, dtype, M, K, N, epi, b is not None, err)
     assert worst["fp32"] < TOL_F32 and worst["bf16"] < TOL_BF16
+
+
+# (M, K, N) either side of the tile choice: at most sixteen 128 x 128 tiles (64 x 64 tiles, also with a K tail and with
+# ragged edges), 320 and 192 big tiles whose last pass would stay mostly empty (128 x 128 tiles instead), 256 and 512 big
+# tiles that fill their passes (256 x 256 tiles)
+TILE_CHOICE = [(32, 384, 128), (100, 72, 200), (500, 256, 460), (16384, 384, 1152), (4096, 768, 3072), (8192, 768, 2048), (8192, 512, 4096)]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("M,K,N", TILE_CHOICE)
+def test_linear_across_the_tile_choice(backend, dtype, M, K, N):
+    """Every tile size the launcher picks by problem shape gives the same product: fused GELU, the gated dual GEMM and
+    the LayerNorm-folded GEMM against float64 on band-edge and random rows."""
+    rng = np.random.default_rng(M + 5 * N + K)
+    x, W, b = gen(rng, M, K, N, 1.0 / np.sqrt(K))
+    x, W = prep(dtype, x, W)
+    rows = band_rows(M, rng, band=64, per=1) if M <= 1024 else band_rows(M, rng)
+    f = backend.fnn
+    y = f.fused_linear_gelu(x, W, b, dtype=dtype)
+    assert y.shape == (M, N) and np.isfinite(y).all()
+    assert O.max_rel(y[rows], O.truth_linear(x[rows], W, b, "gelu")) < tol(dtype)
+    Nh = N // 2
+    g = f.fused_swiglu(x, W[:Nh], W[Nh:2 * Nh], b[:Nh], b[Nh:2 * Nh], dtype=dtype)
+    up = O.truth_linear(x[rows], W[Nh:2 * Nh], b[Nh:2 * Nh])
+    gate = O.truth_linear(x[rows], W[:Nh], b[:Nh])
+    assert O.max_rel(g[rows], gate * (up / (1 + np.exp(-up)))) < tol(dtype)
+    gamma = (1 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(K)).astype(np.float32)
+    z = f.fused_layernorm_linear(x, gamma, beta, W, b, dtype=dtype)
+    ref = O.truth_linear(O.truth_layernorm(x[rows], gamma, beta), W, b)
+    assert O.max_rel(z[rows], ref) < tol(dtype) * (1.5 if dtype == "bf16" else 1.0)
