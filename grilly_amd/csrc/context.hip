@@ -275,7 +275,7 @@ void grl_lap_mark(grl_ctx* c) {
 // with the GEMM wave tile's accumulators (128 registers) and two alternating sets of operand fragments, no memory
 // access inside the loop.  What this reaches is what the matrix cores deliver under the board's power limit for the
 // given operand bits (zeros, or the caller's data), i.e. the ceiling the GEMM and attention kernels work under.
-template <int KIND>
+template <int KIND, int ORDER = 0>
 __global__ __launch_bounds__(512) void mfma_probe_kernel(const u32x4* __restrict__ operands, float* __restrict__ sink, int iters) {
     const int lane = threadIdx.x & 63;
     constexpr int NA = KIND == 0 ? 4 : 8, NB = KIND == 0 ? 2 : 4;       // fragments of a 128 x 64 wave tile
@@ -295,14 +295,30 @@ __global__ __launch_bounds__(512) void mfma_probe_kernel(const u32x4* __restrict
             for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+        // ORDER 0: the four activation-side fragments outermost (an operand pair shares one fragment with the pair before it
+        // every second instruction); 1: the two weight-side fragments outermost (one operand unchanged for four instructions
+        // in a row); 2: the same with the inner walk reversed on every second pass (the turn shares both); 3: one operand pair
+        // for every instruction (what operand reuse could save at most)
+        auto one = [&](int s, int a, int b) __attribute__((always_inline)) {
+            const int so = ORDER == 3 ? 0 : s, ao = ORDER == 3 ? 0 : a, bo = ORDER == 3 ? 0 : b;
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb[so][bo]), __builtin_bit_cast(bf16x8, fa[so][ao]), acc[a][b], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
+            for (int s = 0; s < 2; ++s) {
+                if constexpr (ORDER == 0 || ORDER == 3) {
 #pragma unroll
-                for (int a = 0; a < NA; ++a)
+                    for (int a = 0; a < NA; ++a)
+#pragma unroll
+                        for (int b = 0; b < NB; ++b) one(s, a, b);
+                } else {
 #pragma unroll
                     for (int b = 0; b < NB; ++b)
-                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb[s][b]), __builtin_bit_cast(bf16x8, fa[s][a]), acc[a][b], 0, 0, 0);
+#pragma unroll
+                        for (int a = 0; a < NA; ++a) one(s, (ORDER == 2 && ((b + s * NB) & 1)) ? NA - 1 - a : a, b);
+                }
+            }
         }
         float t = 0.f;
 #pragma unroll
@@ -340,7 +356,7 @@ __global__ __launch_bounds__(512) void mfma_probe_kernel(const u32x4* __restrict
 
 extern "C" int grl_mfma_probe(grl_ctx* c, int kind, const void* operands, int iters, float* ms, double* flops) {
     GRL_REQUIRE(c && ms && flops, GRL_ERR_ARG, "grl_mfma_probe: null argument");
-    GRL_REQUIRE(kind == 0 || kind == 1, GRL_ERR_ARG, "grl_mfma_probe: kind must be 0 (32x32x16 bf16) or 1 (16x16x32 bf16)");
+    GRL_REQUIRE(kind >= 0 && kind <= 4, GRL_ERR_ARG, "grl_mfma_probe: kind must be 0 (32x32x16 bf16), 1 (16x16x32 bf16) or 2..4 (32x32x16 in another operand order)");
     GRL_REQUIRE(iters > 0 && iters <= (1 << 20), GRL_ERR_ARG, "grl_mfma_probe: iters must be in 1..2^20");
     GRL_REQUIRE((((uintptr_t)operands) & 15u) == 0, GRL_ERR_ARG, "grl_mfma_probe: operands must be 16-byte aligned (64 KiB of them, or NULL for zeros)");
     float* sink = (float*)grl_malloc(c, 256);
@@ -348,6 +364,9 @@ extern "C" int grl_mfma_probe(grl_ctx* c, int kind, const void* operands, int it
     const int cus = c->prop.multiProcessorCount;
     auto launch = [&](int n) {
         if (kind == 0) hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(cus), dim3(512), 0, c->stream, (const u32x4*)operands, sink, n);
+        else if (kind == 2) hipLaunchKernelGGL((mfma_probe_kernel<0, 1>), dim3(cus), dim3(512), 0, c->stream, (const u32x4*)operands, sink, n);
+        else if (kind == 3) hipLaunchKernelGGL((mfma_probe_kernel<0, 2>), dim3(cus), dim3(512), 0, c->stream, (const u32x4*)operands, sink, n);
+        else if (kind == 4) hipLaunchKernelGGL((mfma_probe_kernel<0, 3>), dim3(cus), dim3(512), 0, c->stream, (const u32x4*)operands, sink, n);
         else hipLaunchKernelGGL(mfma_probe_kernel<1>, dim3(cus), dim3(512), 0, c->stream, (const u32x4*)operands, sink, n);
     };
     launch(iters);                                   // warm-up: clocks and power settle
@@ -359,7 +378,7 @@ extern "C" int grl_mfma_probe(grl_ctx* c, int kind, const void* operands, int it
     grl_free(c, sink);
     if (rc == GRL_ERR_HIP) grl_set_error("grl_mfma_probe: launch failed");
     // per iteration and wave: 2 fragment sets x a 128 x 64 wave tile x 16 (32) deep = 2 x 128*64*2*16 flops (kind 0), x 32 (kind 1)
-    *flops = (double)iters * 2.0 * 128.0 * 64.0 * 2.0 * (kind == 0 ? 16.0 : 32.0) * 8.0 * cus;
+    *flops = (double)iters * 2.0 * 128.0 * 64.0 * 2.0 * (kind == 1 ? 32.0 : 16.0) * 8.0 * cus;
     return rc;
 }
 

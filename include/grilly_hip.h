@@ -117,7 +117,9 @@ int grl_timer_lap_ms(grl_ctx* ctx, int from, int to, float* elapsed_ms);
  * launches inside a forward; one trace per context at a time. */
 int grl_timer_lap_trace(grl_ctx* ctx, int first, int* next);
 /* Matrix-core ceiling probe (measurement aid, no counterpart in the reference): every CU runs eight waves that issue
- * nothing but MFMAs on register-resident operands (kind 0: v_mfma_f32_32x32x16_bf16, kind 1: v_mfma_f32_16x16x32_bf16)
+ * nothing but MFMAs on register-resident operands (kind 0: v_mfma_f32_32x32x16_bf16 in the GEMM kernels' operand order,
+ * kind 1: v_mfma_f32_16x16x32_bf16; kinds 2, 3, 4: the 32x32x16 loop with one operand held for four instructions in a
+ * row, with a serpentine walk, and with the same operand pair for every instruction)
  * for `iters` loop iterations, after one untimed warm-up launch.  `operands` points to 64 KiB of device memory whose
  * bits become the operand fragments (NULL: all-zero operands).  Returns the launch duration and the FLOPs it
  * executed: the rate the matrix cores sustain under the board's power limit for those operand bits. */

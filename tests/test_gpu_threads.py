@@ -124,3 +124,49 @@ def test_concurrent_rope_attention_with_growing_lengths(backend):
     assert not any(t.is_alive() for t in threads), "a worker did not finish"
     assert not errors, errors
 
+
+
+def test_lap_events_and_matrix_core_probe(backend):
+    """The two other measurement aids: lap events give the time between any two recorded points of the stream (in order,
+    additive), and the register-resident MFMA loop reports its FLOP count and a plausible rate for every operand order
+    and both instruction shapes, on zero and on caller-supplied operand bits."""
+    import ctypes
+    from grilly_amd import _lib as L
+    c = backend.core
+    x = c.upload(np.ones((512, 512), np.float32))
+    y = c.alloc(512 * 512 * 4)
+    ms = ctypes.c_float()
+    try:
+        for i in range(4):
+            L.check(c.lib.grl_timer_lap(c.ctx, i))
+            L.check(c.lib.grl_gemm_nt(c.ctx, L.GRL_F32, L.GRL_F32, 512, 512, 512, x.ptr, x.ptr, None, y.ptr, L.EPI_NONE))
+        L.check(c.lib.grl_timer_lap(c.ctx, 4))
+        parts = []
+        for i in range(4):
+            L.check(c.lib.grl_timer_lap_ms(c.ctx, i, i + 1, ctypes.byref(ms)))
+            assert 0.0 < ms.value < 50.0
+            parts.append(ms.value)
+        L.check(c.lib.grl_timer_lap_ms(c.ctx, 0, 4, ctypes.byref(ms)))
+        assert abs(sum(parts) - ms.value) < 0.02 + 0.05 * ms.value
+        assert c.lib.grl_timer_lap(c.ctx, 256) == L.ERR_ARG and c.lib.grl_timer_lap(c.ctx, -1) == L.ERR_ARG
+        assert c.lib.grl_timer_lap_ms(c.ctx, 0, 255, ctypes.byref(ms)) == L.ERR_ARG       # lap 255 was never recorded
+        np.testing.assert_allclose(c.download(y, (512, 512)), 512.0)
+    finally:
+        x.free(); y.free()
+    rng = np.random.default_rng(0)
+    ops = c.upload(rng.standard_normal(32768).astype(np.float32), L.GRL_BF16)       # 64 KiB of bf16
+    fl = ctypes.c_double()
+    try:
+        for kind in range(5):
+            for ptr in (None, ops.ptr):
+                L.check(c.lib.grl_mfma_probe(c.ctx, kind, ptr, 200, ctypes.byref(ms), ctypes.byref(fl)), "mfma_probe")
+                cus = c.device_info()["compute_units"]
+                assert fl.value == 200 * 2 * 128 * 64 * 2 * (32 if kind == 1 else 16) * 8 * cus
+                rate = fl.value / (ms.value * 1e-3)
+                assert 0.05e15 < rate < 2.7e15, (kind, ptr is None, rate)          # below the 2.5 PFLOP/s peak (+ timer slack)
+        assert c.lib.grl_mfma_probe(c.ctx, 5, None, 10, ctypes.byref(ms), ctypes.byref(fl)) == L.ERR_ARG
+        assert c.lib.grl_mfma_probe(c.ctx, 0, None, 0, ctypes.byref(ms), ctypes.byref(fl)) == L.ERR_ARG
+        assert c.lib.grl_mfma_probe(c.ctx, 0, ops.ptr + 4, 10, ctypes.byref(ms), ctypes.byref(fl)) == L.ERR_ARG
+        assert c.lib.grl_mfma_probe(c.ctx, 0, None, 10, None, ctypes.byref(fl)) == L.ERR_ARG
+    finally:
+        ops.free()
