@@ -33,6 +33,12 @@ struct grl_ctx {
     std::mutex tab_mu;
     std::vector<rope_table> rope_tables;
     std::vector<void*> retired_tables;
+    // pinned staging ring for small host -> device copies (grl_h2d): the caller's buffer is copied here and the transfer
+    // runs asynchronously on the stream; a wrap-around waits for the stream, i.e. for every transfer still reading the ring
+    std::mutex stage_mu;
+    char* stage = nullptr;
+    size_t stage_cap = 0, stage_off = 0;
+    bool stage_failed = false;          // pinned allocation refused once: stay on the blocking path
     // shader-clock probe (grl_clock_probe_begin / _end): its own stream, so that it runs beside the work it observes
     hipStream_t probe_stream = nullptr;
     uint64_t* probe_out = nullptr;      // device: {shader cycles, 100 MHz ticks}

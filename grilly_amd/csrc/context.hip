@@ -63,6 +63,7 @@ extern "C" void grl_destroy(grl_ctx* c) {
     for (auto& e : c->laps) if (e) hipEventDestroy(e);
     if (c->probe_stream) { hipStreamSynchronize(c->probe_stream); hipStreamDestroy(c->probe_stream); }
     if (c->probe_out) hipFree(c->probe_out);
+    if (c->stage) hipHostFree(c->stage);
     hipStreamDestroy(c->stream);
     delete c;
 }
@@ -168,9 +169,34 @@ extern "C" int grl_pool_trim(grl_ctx* c) {
 }
 
 // ---------------------------------------------------------------- copies
+// Host -> device.  Returns when the caller's buffer has been consumed; the transfer is ordered on the context stream like
+// a kernel launch (work enqueued later on this context sees the data, grl_sync / grl_d2h wait for it).  Copies of up to
+// 4 MiB go through a pinned staging ring (one memcpy, then a truly asynchronous transfer: no wait per upload, which is
+// most of the cost of a small numpy -> numpy operator call); larger ones are handed to the runtime and waited for.
+static constexpr size_t GRL_STAGE_MAX = 4u << 20, GRL_STAGE_RING = 32u << 20;
 extern "C" int grl_h2d(grl_ctx* c, void* dst, const void* src, size_t bytes) {
     GRL_REQUIRE(c && (bytes == 0 || (dst && src)), GRL_ERR_ARG, "grl_h2d: null argument");
     if (!bytes) return GRL_OK;
+    if (bytes <= GRL_STAGE_MAX) {
+        std::lock_guard<std::mutex> lk(c->stage_mu);
+        if (!c->stage && !c->stage_failed) {
+            GRL_CHECK_HIP(hipSetDevice(c->device));
+            void* p = nullptr;
+            if (hipHostMalloc(&p, GRL_STAGE_RING, hipHostMallocDefault) == hipSuccess) { c->stage = (char*)p; c->stage_cap = GRL_STAGE_RING; }
+            else { (void)hipGetLastError(); c->stage_failed = true; }
+        }
+        if (c->stage) {
+            if (c->stage_off + bytes > c->stage_cap) {
+                GRL_CHECK_HIP(hipStreamSynchronize(c->stream));      // every earlier transfer has left the ring
+                c->stage_off = 0;
+            }
+            char* slot = c->stage + c->stage_off;
+            memcpy(slot, src, bytes);
+            GRL_CHECK_HIP(hipMemcpyAsync(dst, slot, bytes, hipMemcpyHostToDevice, c->stream));
+            c->stage_off += (bytes + 255) & ~(size_t)255;
+            return GRL_OK;
+        }
+    }
     GRL_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, c->stream));
     GRL_CHECK_HIP(hipStreamSynchronize(c->stream));
     return GRL_OK;

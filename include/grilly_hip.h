@@ -90,8 +90,11 @@ int   grl_free(grl_ctx* ctx, void* ptr);
 int   grl_pool_get_stats(grl_ctx* ctx, grl_pool_stats* out);
 int   grl_pool_trim(grl_ctx* ctx);     /* return cached blocks to the driver */
 
-/* Host <-> device copies (blocking), replacing _upload_buffer / _download_buffer
- * (backend/core.py:345-360).  grl_sync replaces vkQueueWaitIdle (backend/core.py:418). */
+/* Host <-> device copies, replacing _upload_buffer / _download_buffer (backend/core.py:345-360).  grl_h2d returns when
+ * the host buffer has been consumed (the caller may reuse it at once); the transfer itself is ordered on the context
+ * stream like a kernel launch, so later calls on this context see the data and grl_sync / grl_d2h wait for it.  A
+ * consumer on another stream or context must grl_sync first.  grl_d2h blocks until the data is in the host buffer.
+ * grl_sync replaces vkQueueWaitIdle (backend/core.py:418). */
 int grl_h2d(grl_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
 int grl_d2h(grl_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
 int grl_d2d(grl_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes);
