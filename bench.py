@@ -512,6 +512,11 @@ def mfma_ceiling(backend, iters=20000):
             ghz = c.clock_probe_end()
             out.setdefault(name, {})[label] = {"ms": round(ms.value, 3), "tflops": round(fl.value / ms.value / 1e9, 1),
                                                "frac_of_peak": round(fl.value / (ms.value * 1e-3) / PEAK_BF16, 4), "shader_clock_ghz": round(ghz, 3)}
+    # the 32x32x16 loop again with its fragments paired in other orders (random operands): does the order matter?
+    for kind, label in ((2, "one_operand_held_for_four"), (3, "serpentine_walk"), (4, "same_operand_pair_always")):
+        ms, fl = ctypes.c_float(), ctypes.c_double()
+        L.check(c.lib.grl_mfma_probe(c.ctx, kind, rnd.ptr, iters, ctypes.byref(ms), ctypes.byref(fl)), "mfma_probe")
+        out.setdefault("v_mfma_f32_32x32x16_bf16_operand_order", {})[label] = {"ms": round(ms.value, 3), "frac_of_peak": round(fl.value / (ms.value * 1e-3) / PEAK_BF16, 4)}
     rnd.free()
     return out
 
