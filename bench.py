@@ -594,7 +594,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the fp32 forward and the two single-operator configurations")
-    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "kernels", "copy", "fa2_long", "swiglu_mlp", "prenorm_forward", "small", "mfma_ceiling"],
+    ap.add_argument("--mode", default="forward", choices=["forward", "gemm", "kernels", "copy", "fa2_long", "swiglu_mlp", "prenorm_forward", "small", "mfma_ceiling", "gemm_shapes"],
                     help="forward: the benchmark; gemm / copy: only launch the dominant GEMM kernel at its three "
                          "layer shapes, or a plain 1 GiB copy kernel (for rocprofv3 counter runs); kernels: every kernel of "
                          "the layer at its layer shape, nothing else (counter runs); fa2_long: "
@@ -602,7 +602,8 @@ def main():
                          "X[16384,4096] through gate/up [11008,4096] + silu*up + down [4096,11008], bf16; prenorm_forward: the "
                          "pre-norm / rotary / GeGLU encoder at the ModernBERT-base shape, batch 128 x seq 512, bf16; small: the README "
                          "operators (configs[0]) in microseconds and the MiniLM-shaped fp32 encoder (configs[1]); mfma_ceiling: "
-                         "register-resident MFMA loops, zero and random operands (what the power limit leaves of the matrix peak)")
+                         "register-resident MFMA loops, zero and random operands (what the power limit leaves of the matrix peak); gemm_shapes: "
+                         "fused GELU linear at mid-size shapes either side of the tile choice (GRL_GEMM_VARIANT=3 / 4 forces a tile size)")
     ap.add_argument("--cpu-sequences", type=int, default=12)
     ap.add_argument("--unfused", action="store_true", help="run the seven-launch layer (two LayerNorm passes per layer) instead of the "
                     "layer with both LayerNorms folded into its GEMMs")
@@ -631,6 +632,29 @@ def main():
     if a.mode == "small":
         r0, r1 = small_configs(backend, a.kernel_reps, check=not a.no_cpu_baseline)
         print(json.dumps({"mode": "small", "readme_ops": r0, "minilm_forward": r1}))
+        backend.cleanup()
+        return
+    if a.mode == "gemm_shapes":
+        # fused GELU linear at mid-size shapes either side of the launcher's tile choice, both storage types: median launch in
+        # microseconds.  GRL_GEMM_VARIANT=3 / 4 in the environment forces 256 x 256 / 128 x 128 tiles for comparison.
+        from grilly_amd import _lib as L
+        c = backend.core
+        rng = np.random.default_rng(0)
+        shapes = [(16384, 1152, 384), (16384, 384, 384), (16384, 1536, 384), (16384, 384, 1536), (8192, 2304, 768), (8192, 768, 768),
+                  (8192, 3072, 768), (8192, 768, 3072), (4096, 2304, 768), (4096, 3072, 768), (4096, 768, 3072), (2048, 3072, 768),
+                  (2048, 768, 3072), (32768, 768, 768), (32768, 3072, 768), (20000, 1024, 1024), (12000, 4096, 1024)]
+        res = {}
+        for dt, code, es in (("fp32", L.GRL_F32, 4), ("bf16", L.GRL_BF16, 2)):
+            for (M, N, K) in shapes:
+                x = c.upload(rng.standard_normal((M, K)).astype(np.float32), code)
+                w = c.upload((rng.standard_normal((N, K)) * 0.02).astype(np.float32), code)
+                bias = c.upload(rng.standard_normal(N).astype(np.float32))
+                y = c.alloc(M * N * es)
+                fn = lambda: L.check(c.lib.grl_gemm_nt(c.ctx, code, code, M, N, K, x.ptr, w.ptr, bias.ptr, y.ptr, L.EPI_GELU))
+                res[f"{dt} {M}x{N}x{K}"] = round(median(lap_times(c, fn, 30)) * 1e3, 1)
+                for t in (x, w, bias, y):
+                    t.free()
+        print(json.dumps({"mode": "gemm_shapes", "forced_variant": os.environ.get("GRL_GEMM_VARIANT"), "median_us": res}))
         backend.cleanup()
         return
     if a.mode == "mfma_ceiling":
