@@ -66,6 +66,7 @@ SIGNATURES = {
     "grl_clock_probe_begin": (c_int, [c_void_p, c_float]),
     "grl_clock_probe_end": (c_int, [c_void_p, ctypes.POINTER(c_float)]),
     "grl_cast": (c_int, [c_void_p, c_int, c_int, c_i64, c_void_p, c_void_p]),
+    "grl_gemm_plan": (c_int, [c_int, c_i64, c_i64, c_i64, c_int, c_int]),
     "grl_gemm_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_int]),
     "grl_gemm_nn": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "grl_gemm_nn_noalloc": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_void_p]),

@@ -171,6 +171,12 @@ extern "C" int grl_ln_gemm_nt_stats(grl_ctx* c, int in_dtype, int out_dtype, int
     return dispatch_types_ln(c, a, in_dtype, out_dtype, epilogue == GRL_EPI_GELU ? EPI_GELU : EPI_NONE);
 }
 
+// which kernel / tile size grl_gemm_nt and its siblings pick for a 16-byte aligned problem (pure host arithmetic)
+extern "C" int grl_gemm_plan(int dtype, int64_t M, int64_t N, int64_t K, int dual, int compute_units) {
+    if (!grl_valid_dtype(dtype) || M <= 0 || N <= 0 || K <= 0 || compute_units <= 0) return GRL_ERR_ARG;
+    return gemm_variant(M, N, K, dtype == GRL_F32 ? 4 : 2, dual != 0, compute_units);
+}
+
 // ---- C = A.W^T + bias + LayerNorm(R), and the row statistics of C ------------------------------------------------
 extern template int launch_gemm_resln<float, float>(grl_ctx*, GemmArgs&, int*);
 extern template int launch_gemm_resln<uint16_t, uint16_t>(grl_ctx*, GemmArgs&, int*);

@@ -1077,6 +1077,21 @@ static inline bool prefer_big_tiles(int64_t n_big, int64_t n_small, int64_t cus,
     return !(t_small < 0.93 * t_big);
 }
 
+// Which kernel a 16-byte aligned problem gets: 1 register-staged 256 x 256 tiles, 2 register-staged 128 x 128, 3 direct-to-LDS
+// 256 x 256 (persistent), 4 direct-to-LDS 128 x 128, 5 register-staged 64 x 64.  The direct-to-LDS kernels need K to be a
+// whole number of 128-byte slabs.  Problems of at most sixteen 128 x 128 tiles (single sentences, the README-sized
+// operators) leave most CUs idle and pad M up to 128 rows: 64 x 64 tiles give them four times the workgroups, each with a
+// quarter of the serial K loop.  `dual`: the gated kernels, whose tiles hold half as many output columns.
+static inline int gemm_variant(int64_t M, int64_t N, int64_t K, size_t elem_size, bool dual, int64_t cus) {
+    const int64_t bke = 128 / (int64_t)elem_size;
+    const int64_t big_m = (M + 255) / 256, big_n = (N + (dual ? 127 : 255)) / (dual ? 128 : 256);
+    const int64_t sm = (M + 127) / 128, sn = (N + (dual ? 63 : 127)) / (dual ? 64 : 128);
+    if (sm * sn <= 16) return 5;
+    const bool slabs = K % bke == 0;
+    const bool big = prefer_big_tiles(big_m * big_n, sm * sn, cus, elem_size);
+    return slabs ? (big ? 3 : 4) : (big ? 1 : 2);
+}
+
 template <typename T, typename OutT, int EPI, bool DUAL, bool LN = false>
 static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     const int64_t epc = 16 / (int64_t)sizeof(T);
@@ -1090,9 +1105,7 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
         GRL_CHECK_LAUNCH();
         return GRL_OK;
     }
-    // Tile choice.  The direct-to-LDS kernel needs whole 128-byte K slabs; the 256x256 tile is
-    // used once it yields enough workgroups to occupy most of the 256 CUs, else 128x128 tiles.
-    // GRL_GEMM_VARIANT (1..5) forces one variant, for tuning runs.
+    // Tile choice: gemm_variant().  GRL_GEMM_VARIANT (1..5) forces one variant, for tuning runs.
     static const int forced = [] { const char* e = getenv("GRL_GEMM_VARIANT"); return e ? atoi(e) : 0; }();
     // band height of the tile walk: rows of 8 KiB and more do better with narrow bands (measured)
     static const int group = [] { const char* e = getenv("GRL_GEMM_GROUP"); return e ? atoi(e) : 0; }();
@@ -1104,12 +1117,8 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     GRL_REQUIRE(a.K * (int64_t)sizeof(T) * 256 < (1LL << 31), GRL_ERR_SHAPE, "gemm: K too large (256 rows must span < 2 GiB)");
     const bool slabs = a.K % bke == 0;
     const int64_t cus = c->prop.multiProcessorCount;     // one 128 KiB-LDS workgroup per CU, two of the 64 KiB ones
-    const bool big = prefer_big_tiles(big_m * big_n, sm * sn, cus, sizeof(T));
-    // problems of a few 128 x 128 tiles (single sentences, the README-sized operators) leave most CUs idle and pad M up
-    // to 128 rows: 64 x 64 tiles give them four times the workgroups, each with a quarter of the serial K loop
-    const bool tiny = sm * sn <= 16;
     const int64_t tm = (a.M + 63) / 64, tn = (a.N + 63) / 64;      // 64 output columns per tile (with two weights: 128 LDS rows)
-    int variant = tiny ? 5 : (slabs ? (big ? 3 : 4) : (big ? 1 : 2));
+    int variant = gemm_variant(a.M, a.N, a.K, sizeof(T), DUAL, cus);
     if (forced >= 1 && forced <= 5 && (slabs || forced <= 2 || forced == 5)) variant = forced;
     switch (variant) {
         case 5:

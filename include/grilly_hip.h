@@ -148,6 +148,11 @@ int grl_cast(grl_ctx* ctx, int src_dtype, int dst_dtype, int64_t n, const void* 
  * in_dtype is the type of A and W, out_dtype the type of C; bias may be NULL. */
 int grl_gemm_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
                 const void* A, const void* W, const float* bias, void* C, int epilogue);
+/* Which kernel grl_gemm_nt and its siblings launch for a problem whose operands are 16-byte aligned, as pure host
+ * arithmetic (no device needed; no counterpart in the reference): 1 / 2 register-staged 256 x 256 / 128 x 128 tiles,
+ * 3 / 4 direct-to-LDS 256 x 256 (persistent) / 128 x 128 tiles, 5 register-staged 64 x 64 tiles.  `dual` selects the
+ * gated two-weight kernels, `compute_units` the CU count of the device (256 on MI355X).  Negative on bad arguments. */
+int grl_gemm_plan(int dtype, int64_t M, int64_t N, int64_t K, int dual, int compute_units);
 
 /* C = A.B with B (K,N) row-major.  Replaces VulkanFNN.gemm (backend/fnn.py:104-166,
  * shaders/gemm_mnk.glsl:35-88).  workspace must hold K*N elements of in_dtype (the

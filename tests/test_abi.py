@@ -93,3 +93,24 @@ def test_dtype_codes_and_encoder_config():
     assert len(w["layers"]) == 2 and w["layers"][0]["w_qkv"].shape == (192, 64) and w["layers"][0]["w_ff2"].shape == (64, 128)
     assert abs(float(w["tok_emb"].std()) - 0.02) < 2e-3
     assert MINILM_L6.head_dim == 32
+
+
+def test_gemm_tile_choice_for_the_benchmark_shapes():
+    """grl_gemm_plan is the launcher's tile choice as host arithmetic: the benchmark's shapes (65536 rows: whole passes
+    of 256 x 256 tiles over 256 CUs) and the SwiGLU MLP stay on the persistent big-tile kernel, the MiniLM-shaped
+    GEMMs whose big tiles would leave the last pass mostly empty get 128 x 128 tiles, README-sized problems 64 x 64
+    tiles, and a K that is not a whole number of 128-byte slabs the register-staged kernels."""
+    lib = L.load()
+    plan = lambda dt, M, N, K, dual=0, cus=256: lib.grl_gemm_plan(dt, M, N, K, dual, cus)
+    for dt in (L.GRL_BF16, L.GRL_F32):
+        for (N, K) in [(2304, 768), (768, 768), (3072, 768), (768, 3072)]:
+            assert plan(dt, 65536, N, K) == 3, (dt, N, K)
+    assert plan(L.GRL_BF16, 16384, 11008, 4096, dual=1) == 3 and plan(L.GRL_BF16, 16384, 4096, 11008) == 3
+    assert plan(L.GRL_BF16, 65536, 1152, 768, dual=1) == 3                  # the pre-norm encoder's gated GEMM
+    # 16384 x 1152: 320 big tiles = two passes, the second a quarter full; 1152 small tiles = two full passes and a bit
+    assert plan(L.GRL_F32, 16384, 1152, 384) == 4 and plan(L.GRL_F32, 16384, 1536, 384) == 4
+    assert plan(L.GRL_F32, 16384, 384, 384) == 4                             # below 192 big tiles: always small
+    assert plan(L.GRL_BF16, 8192, 2304, 768) == 4 and plan(L.GRL_BF16, 32768, 3072, 768) == 3
+    assert plan(L.GRL_F32, 32, 128, 384) == 5 and plan(L.GRL_BF16, 128, 2304, 768) == 4 and plan(L.GRL_BF16, 128, 768, 768) == 5
+    assert plan(L.GRL_F32, 4096, 4096, 1000) == 1 and plan(L.GRL_F32, 1024, 1024, 1000) == 2      # K tail: register-staged
+    assert plan(L.GRL_F32, 0, 8, 8) == L.ERR_ARG and plan(7, 8, 8, 8) == L.ERR_ARG and plan(L.GRL_F32, 8, 8, 8, cus=0) == L.ERR_ARG
