@@ -82,6 +82,7 @@ SIGNATURES = {
     "grl_ln_stats": (c_int, [c_void_p, c_int, c_i64, c_i64, c_void_p, c_float, c_void_p]),
     "grl_ln_gemm_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 4 + [c_float, c_void_p, c_void_p]),
     "grl_ln_glu_nt": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 7 + [c_float, c_void_p, c_void_p, c_int]),
+    "grl_ln_glu_nt_stats": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 7 + [c_void_p, c_void_p, c_int]),
     "grl_ln_gemm_nt_stats": (c_int, [c_void_p, c_int, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 6 + [c_int]),
     "grl_gemm_nt_resln_workspace": (c_i64, [c_i64, c_i64]),
     "grl_gemm_nt_resln": (c_int, [c_void_p, c_int, c_i64, c_i64, c_i64] + [c_void_p] * 8 + [c_float, c_void_p, c_void_p]),

@@ -229,21 +229,24 @@ extern "C" int grl_gemm_nt_resln(grl_ctx* c, int dtype, int64_t M, int64_t N, in
     return GRL_OK;
 }
 
-extern "C" int grl_ln_glu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
-                             const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
-                             const float* bias_gate_folded, const float* bias_up_folded, float eps, float* stats,
-                             void* out, int activation) {
-    GRL_REQUIRE(c, GRL_ERR_ARG, "grl_ln_glu_nt: null context");
-    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_ln_glu_nt: bad dtype");
+// stats == given: {1/sd, mean/sd} per row of x are the caller's (from grl_ln_stats or a GEMM epilogue); else they are computed here
+static int ln_glu_nt_impl(grl_ctx* c, const char* who, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                          const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
+                          const float* bias_gate_folded, const float* bias_up_folded, bool given, float eps, float* stats,
+                          void* out, int activation) {
+    GRL_REQUIRE(c, GRL_ERR_ARG, "%s: null context", who);
+    GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "%s: bad dtype", who);
     GRL_REQUIRE(activation == GRL_EPI_SILU || activation == GRL_EPI_RELU || activation == GRL_EPI_GELU, GRL_ERR_ARG,
-                "grl_ln_glu_nt: activation must be GRL_EPI_SILU, GRL_EPI_RELU or GRL_EPI_GELU (got %d)", activation);
-    int rc = check_dims("grl_ln_glu_nt", M, N, K);
+                "%s: activation must be GRL_EPI_SILU, GRL_EPI_RELU or GRL_EPI_GELU (got %d)", who, activation);
+    int rc = check_dims(who, M, N, K);
     if (rc) return rc;
     if (M == 0 || N == 0) return GRL_OK;
     GRL_REQUIRE(out && K > 0 && x && Wg_scaled && Wu_scaled && colsum_gate && colsum_up && bias_gate_folded && bias_up_folded && stats,
-                GRL_ERR_ARG, "grl_ln_glu_nt: null argument or K == 0");
-    rc = grl_ln_stats(c, in_dtype, M, K, x, eps, stats);
-    if (rc) return rc;
+                GRL_ERR_ARG, "%s: null argument or K == 0", who);
+    if (!given) {
+        rc = grl_ln_stats(c, in_dtype, M, K, x, eps, stats);
+        if (rc) return rc;
+    }
     GemmArgs a{};
     a.A = x; a.W = Wg_scaled; a.W2 = Wu_scaled; a.C = out;
     a.bias = bias_gate_folded; a.bias2 = bias_up_folded;
@@ -251,6 +254,21 @@ extern "C" int grl_ln_glu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M,
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     a.act = activation;
     return dispatch_types_ln(c, a, in_dtype, out_dtype, EPI_GLU);
+}
+
+extern "C" int grl_ln_glu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                             const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
+                             const float* bias_gate_folded, const float* bias_up_folded, float eps, float* stats,
+                             void* out, int activation) {
+    return ln_glu_nt_impl(c, "grl_ln_glu_nt", in_dtype, out_dtype, M, N, K, x, Wg_scaled, Wu_scaled, colsum_gate, colsum_up,
+                          bias_gate_folded, bias_up_folded, false, eps, stats, out, activation);
+}
+extern "C" int grl_ln_glu_nt_stats(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                                   const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
+                                   const float* bias_gate_folded, const float* bias_up_folded, const float* stats,
+                                   void* out, int activation) {
+    return ln_glu_nt_impl(c, "grl_ln_glu_nt_stats", in_dtype, out_dtype, M, N, K, x, Wg_scaled, Wu_scaled, colsum_gate, colsum_up,
+                          bias_gate_folded, bias_up_folded, true, 0.f, const_cast<float*>(stats), out, activation);
 }
 
 extern "C" int grl_swiglu_nt(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,

@@ -263,10 +263,11 @@ class PreNormEncoder:
     The packed Wqkv is one GEMM; attention reads its three column blocks in place.  The +-50 / +-1e6 clips the
     reference puts around the gate (:924-930) are not applied: they only act beyond those magnitudes."""
 
-    def __init__(self, core, cfg, weights, dtype="fp32"):
+    def __init__(self, core, cfg, weights, dtype="fp32", stats_from_gemm=None):
         self.core = core.core if hasattr(core, "core") else core
         if not isinstance(self.core, HipCore):
             raise TypeError("PreNormEncoder needs a Compute() backend or its HipCore")
+        self._stats_from_gemm = stats_from_gemm        # None: wherever the kernel takes the width
         if cfg.head_dim * cfg.heads != cfg.d_model or cfg.head_dim % 2 or cfg.head_dim > 128:
             raise ValueError("d_model must be heads*head_dim with an even head_dim up to 128 (rotary positions)")
         self.cfg, self.dtype, self.code = cfg, dtype, dtype_code(dtype)
@@ -310,6 +311,19 @@ class PreNormEncoder:
         act = B * S * cfg.d_model * es
         self.x, self.att = (c.alloc(act) for _ in range(2))
         self.stats = c.alloc(B * S * 8)                # {1/sd, mean/sd} per row, for the GEMM that carries the MLP's LayerNorm
+        # The row statistics come out of the epilogue of the output projection that writes the rows (the GEMM entry point
+        # that adds LayerNorm(residual) and reduces the moments of what it stores, here with the identity in place of the
+        # LayerNorm: statistics {1, 0}, scale 1, shift 0) where that kernel takes the shape; else from a pass over the rows.
+        slab = 64 if self.code == L.GRL_BF16 else 32
+        self.stats_from_gemm = cfg.d_model % slab == 0 if self._stats_from_gemm is None else bool(self._stats_from_gemm)
+        if self.stats_from_gemm and cfg.d_model % slab:
+            raise ValueError(f"row statistics out of the GEMM epilogue need d_model to be a multiple of {slab}")
+        if self.stats_from_gemm:
+            ident = np.zeros((B * S, 2), np.float32)
+            ident[:, 0] = 1.0
+            self.ident_stats = c.upload_raw(ident)
+            self.ones, self.zeros = c.upload_raw(np.ones(cfg.d_model, np.float32)), c.upload_raw(np.zeros(cfg.d_model, np.float32))
+            self.part = c.alloc(int(c.lib.grl_gemm_nt_resln_workspace(B * S, cfg.d_model)))
         self.qkv = c.alloc(3 * act)                    # packed (M, 3d): Q, K, V are its three column blocks
         self.h = c.alloc(B * S * cfg.d_ff * es)
         self.ids = c.alloc(B * S * 4)
@@ -324,6 +338,9 @@ class PreNormEncoder:
         if self._shape is not None:
             for b in (self.x, self.qkv, self.att, self.stats, self.h, self.ids, self.mask, self.first, self.pooled):
                 b.free()
+            if self.stats_from_gemm:
+                for b in (self.ident_stats, self.ones, self.zeros, self.part):
+                    b.free()
             self._shape = None
 
     def set_inputs(self, input_ids, attention_mask=None):
@@ -361,12 +378,20 @@ class PreNormEncoder:
                                             self.qkv.ptr + 2 * d * es, mask, self.att.ptr, 3 * d, 3 * d, 3 * d, d,
                                             1.0 / float(np.sqrt(D)), 0, L.ROPE_HALF, cfg.rope_base, cfg.rope_scaling),
                     "attention")
-            L.check(lib.grl_gemm_nt_res(c.ctx, code, code, M, d, d, self.att.ptr, w["w_o"].ptr, w["b_o"].ptr, self.x.ptr,
-                                        self.x.ptr), "output projection + residual")
             # LayerNorm + dual GEMM; the dual GEMM activates its second ("up") operand: that is the first half of Wi here
-            L.check(lib.grl_ln_glu_nt(c.ctx, code, code, M, ff, d, self.x.ptr, w["ws_gate"].ptr, w["ws_in"].ptr,
-                                      w["cs_gate"].ptr, w["cs_in"].ptr, w["bf_gate"].ptr, w["bf_in"].ptr, cfg.eps,
-                                      self.stats.ptr, self.h.ptr, L.EPI_GELU), "mlp layernorm + geglu")
+            if self.stats_from_gemm:
+                L.check(lib.grl_gemm_nt_resln(c.ctx, code, M, d, d, self.att.ptr, w["w_o"].ptr, w["b_o"].ptr, self.x.ptr,
+                                              self.ident_stats.ptr, self.ones.ptr, self.zeros.ptr, self.x.ptr, cfg.eps,
+                                              self.stats.ptr, self.part.ptr), "output projection + residual + row statistics")
+                L.check(lib.grl_ln_glu_nt_stats(c.ctx, code, code, M, ff, d, self.x.ptr, w["ws_gate"].ptr, w["ws_in"].ptr,
+                                                w["cs_gate"].ptr, w["cs_in"].ptr, w["bf_gate"].ptr, w["bf_in"].ptr,
+                                                self.stats.ptr, self.h.ptr, L.EPI_GELU), "mlp layernorm + geglu")
+            else:
+                L.check(lib.grl_gemm_nt_res(c.ctx, code, code, M, d, d, self.att.ptr, w["w_o"].ptr, w["b_o"].ptr, self.x.ptr,
+                                            self.x.ptr), "output projection + residual")
+                L.check(lib.grl_ln_glu_nt(c.ctx, code, code, M, ff, d, self.x.ptr, w["ws_gate"].ptr, w["ws_in"].ptr,
+                                          w["cs_gate"].ptr, w["cs_in"].ptr, w["bf_gate"].ptr, w["bf_in"].ptr, cfg.eps,
+                                          self.stats.ptr, self.h.ptr, L.EPI_GELU), "mlp layernorm + geglu")
             L.check(lib.grl_gemm_nt_res(c.ctx, code, code, M, d, ff, self.h.ptr, w["w_ff2"].ptr, w["b_ff2"].ptr, self.x.ptr,
                                         self.x.ptr), "mlp output + residual")
         if self.final is not None:

@@ -278,6 +278,12 @@ int grl_ln_glu_nt(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t 
                   const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
                   const float* bias_gate_folded, const float* bias_up_folded, float eps, float* stats,
                   void* out, int activation);
+/* grl_ln_glu_nt with the row statistics given ({1/sd, mean/sd} per row of x, e.g. written by grl_gemm_nt_resln when it
+ * produced x): no pass over x in front of the GEMM. */
+int grl_ln_glu_nt_stats(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K, const void* x,
+                        const void* Wg_scaled, const void* Wu_scaled, const float* colsum_gate, const float* colsum_up,
+                        const float* bias_gate_folded, const float* bias_up_folded, const float* stats,
+                        void* out, int activation);
 /* grl_ln_gemm_nt with the row statistics given ({1/sd, mean/sd} per row of x, as grl_ln_stats or grl_gemm_nt_resln
  * write them) and a choice of epilogue: GRL_EPI_NONE or GRL_EPI_GELU (out = gelu(LN(x).W^T + b), the first half of the
  * feed-forward block behind a LayerNorm, utils/vulkan_sentence_transformer.py:1004-1012). */

@@ -277,3 +277,68 @@ def test_gated_and_ln_folded_gemms_c_abi_randomized(backend):
                     b.free()
         if case and case % 50 == 0:
             print("sweep case", case, flush=True)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_residual_gemm_statistics_feed_the_gated_gemm(backend, dtype):
+    """The pre-norm layer's chain without a pass over the rows: grl_gemm_nt_resln with the identity in place of the
+    LayerNorm on its residual (statistics {1, 0}, scale 1, shift 0) is the plain residual GEMM x + att.Wo^T + b,
+    and the row statistics it writes drive grl_ln_glu_nt_stats to what grl_ln_glu_nt computes from its own pass."""
+    import ctypes
+    from grilly_amd import _lib as L
+    c = backend.core
+    code, es = (L.GRL_BF16, 2) if dtype == "bf16" else (L.GRL_F32, 4)
+    rng = np.random.default_rng(31)
+    M, d, ff, eps = 1000, 256, 320, 1e-5
+    qd = (lambda a: O.bf16_round(a)) if dtype == "bf16" else (lambda a: a)
+    att = qd(rng.standard_normal((M, d)).astype(np.float32))
+    Wo = qd((rng.standard_normal((d, d)) / np.sqrt(d)).astype(np.float32))
+    bo = rng.standard_normal(d).astype(np.float32)
+    x = qd((1.5 * rng.standard_normal((M, d)) + rng.standard_normal((M, 1))).astype(np.float32))
+    Wg, Wu = (qd((rng.standard_normal((ff, d)) / np.sqrt(d)).astype(np.float32)) for _ in range(2))
+    bg, bu = (rng.standard_normal(ff).astype(np.float32) for _ in range(2))
+    g, bt = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32), (0.1 * rng.standard_normal(d)).astype(np.float32)
+    ident = np.zeros((M, 2), np.float32); ident[:, 0] = 1.0
+    up = lambda a, cd=L.GRL_F32: c.upload(a, cd)
+    datt, dWo, dbo, dx1, dx2 = up(att, code), up(Wo, code), up(bo), up(x, code), up(x, code)
+    did, dones, dzeros = up(ident), up(np.ones(d, np.float32)), up(np.zeros(d, np.float32))
+    dWg, dWu, dbg, dbu, dg, dbt = up(Wg, code), up(Wu, code), up(bg), up(bu), up(g), up(bt)
+    st1, st2 = c.alloc(M * 8), c.alloc(M * 8)
+    part = c.alloc(int(c.lib.grl_gemm_nt_resln_workspace(M, d)))
+    wsg, wsu = c.alloc(ff * d * es), c.alloc(ff * d * es)
+    csg, csu, bfg, bfu = (c.alloc(ff * 4) for _ in range(4))
+    h1, h2 = c.alloc(M * ff * es), c.alloc(M * ff * es)
+    bufs = [datt, dWo, dbo, dx1, dx2, did, dones, dzeros, dWg, dWu, dbg, dbu, dg, dbt, st1, st2, part, wsg, wsu, csg, csu, bfg, bfu, h1, h2]
+    try:
+        L.check(c.lib.grl_ln_fold(c.ctx, code, ff, d, dWg.ptr, dg.ptr, dbt.ptr, dbg.ptr, wsg.ptr, csg.ptr, bfg.ptr))
+        L.check(c.lib.grl_ln_fold(c.ctx, code, ff, d, dWu.ptr, dg.ptr, dbt.ptr, dbu.ptr, wsu.ptr, csu.ptr, bfu.ptr))
+        # route 1: residual GEMM, then the gated GEMM with its own statistics pass
+        L.check(c.lib.grl_gemm_nt_res(c.ctx, code, code, M, d, d, datt.ptr, dWo.ptr, dbo.ptr, dx1.ptr, dx1.ptr))
+        L.check(c.lib.grl_ln_glu_nt(c.ctx, code, code, M, ff, d, dx1.ptr, wsg.ptr, wsu.ptr, csg.ptr, csu.ptr, bfg.ptr, bfu.ptr, eps,
+                                    st1.ptr, h1.ptr, L.EPI_GELU))
+        # route 2: the statistics out of the residual GEMM's epilogue
+        L.check(c.lib.grl_gemm_nt_resln(c.ctx, code, M, d, d, datt.ptr, dWo.ptr, dbo.ptr, dx2.ptr, did.ptr, dones.ptr, dzeros.ptr,
+                                        dx2.ptr, eps, st2.ptr, part.ptr))
+        L.check(c.lib.grl_ln_glu_nt_stats(c.ctx, code, code, M, ff, d, dx2.ptr, wsg.ptr, wsu.ptr, csg.ptr, csu.ptr, bfg.ptr, bfu.ptr,
+                                          st2.ptr, h2.ptr, L.EPI_GELU))
+        x1, x2 = c.download(dx1, (M, d), code), c.download(dx2, (M, d), code)
+        # (the two entry points may pick different tile sizes, and the staged epilogue starts its sums from the bias where the
+        # direct one adds it last: equal up to the last bit, not bit for bit)
+        assert O.max_rel(x1, x2) < (2e-6 if dtype == "fp32" else 8e-3)
+        # the statistics describe the rows as each route stored them (in bf16 the two differ by single roundings)
+        for xs, st in ((x1, st1), (x2, st2)):
+            got = c.download(st, (M, 2))
+            mu, sd = xs.astype(np.float64).mean(-1), np.sqrt(xs.astype(np.float64).var(-1) + eps)
+            assert O.max_rel(got[:, 0], 1 / sd) < 1e-4 and np.abs(got[:, 1] - mu / sd).max() < 1e-4 * max(1.0, np.abs(mu / sd).max())
+        y1, y2 = c.download(h1, (M, ff), code), c.download(h2, (M, ff), code)
+        tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+        assert O.max_rel(y2, y1) < tol * 0.5
+        ref_x = O.truth_linear(att, Wo, bo) + x.astype(np.float64)
+        xn = O.truth_layernorm(x2, g, bt, eps)
+        ref = O.truth_linear(xn, Wg, bg) * O.truth_gelu(O.truth_linear(xn, Wu, bu))
+        assert O.max_rel(x2, ref_x) < tol and O.max_rel(y2, ref) < tol * (1.5 if dtype == "bf16" else 1.0)
+        assert c.lib.grl_ln_glu_nt_stats(c.ctx, code, code, M, ff, d, dx2.ptr, wsg.ptr, wsu.ptr, csg.ptr, csu.ptr, bfg.ptr, bfu.ptr,
+                                         None, h2.ptr, L.EPI_GELU) == L.ERR_ARG
+    finally:
+        for b in bufs:
+            b.free()
