@@ -99,7 +99,7 @@ def forward_kernel_times(backend, enc, cfg, forwards=8):
     from grilly_amd import _lib as L
     import ctypes
     core = backend.core
-    fused = getattr(enc, "fused", False)
+    fused = getattr(enc, "fused_now", False)
     names = ["gemm_qkv_ln", "fa2_fwd", "gemm_out_resln", "gemm_ffn1_ln_gelu", "gemm_ffn2_resln"] if fused else \
             ["gemm_qkv", "fa2_fwd", "gemm_out", "layernorm_residual", "gemm_ffn1_gelu", "gemm_ffn2", "layernorm_residual"]
     per_layer = len(names) + 1                         # the mark at layer entry
@@ -188,7 +188,7 @@ def kernel_table(backend, enc, B, S, reps, only=None, check=True):
         L.check(f())
     c.sync()
     fused_runs = []
-    if getattr(enc, "fused", False):
+    if getattr(enc, "fused_now", False):
         # the four GEMMs of the layer in the form the forward launches them (LayerNorms folded in): the raw residual
         # stream r0 = x (its "LayerNorm" statistics are those of x itself), r1 = out-proj + LN(r0), ff, r2 = FFN2 + LN(r1)
         fs = enc.fused_structs[0]
@@ -675,7 +675,7 @@ def main():
     if a.mode in ("gemm", "kernels"):
         only = None
         if a.mode == "gemm":        # the launches of the dominant GEMM instantiation only (counter runs)
-            only = ("gemm_out_resln", "gemm_ffn2_resln") if enc.fused else ("gemm_qkv", "gemm_out", "gemm_ffn2")
+            only = ("gemm_out_resln", "gemm_ffn2_resln") if enc.fused_now else ("gemm_qkv", "gemm_out", "gemm_ffn2")
         kt = kernel_table(backend, enc, B, S, a.kernel_reps, only=only, check=False)
         print(json.dumps({"mode": a.mode, "kernels": kt, "launches_each": a.kernel_reps + WARM}))
         backend.cleanup()
@@ -729,7 +729,7 @@ def main():
         # (QKV, out-proj, FFN2: three launches per layer).  Average FLOPs per launch over average duration per launch,
         # the durations being those INSIDE the forward (lap events between the layer's launches); the same launches
         # timed back to back in a table of their own are reported next to it.
-        fused = getattr(enc, "fused", False)
+        fused = getattr(enc, "fused_now", False)
         names = ("gemm_out_resln", "gemm_ffn2_resln") if fused else ("gemm_qkv", "gemm_out", "gemm_ffn2")
         tname = "float" if a.dtype == "fp32" else "bf16"
         kname = f"gemm_nt_dma_kernel<{tname},{tname},256,256,2,4,{'EPI_RESLN' if fused else 'EPI_NONE'}>"

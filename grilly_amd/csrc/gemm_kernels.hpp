@@ -490,8 +490,11 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
 //   swizzled by row) -> 16-byte row-contiguous global stores, 32 output rows per wave-row
 //   per pass, two staging regions used alternately so a pass costs one barrier.
 // =====================================================================================
+// (launch bounds: the four-wave workgroups of the 128 x 128 tiles run two to a CU, i.e. two waves per SIMD, like the one
+// eight-wave workgroup of the 256 x 256 tiles: the register budget is 256 per lane either way, and an instantiation that
+// would take more must spill rather than halve the occupancy)
 template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL, bool LN = false>
-__global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_dma_kernel(GemmArgs p) {
+__global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN <= 4 ? 2 : 1)) void gemm_nt_dma_kernel(GemmArgs p) {
     constexpr int NW = WGM * WGN, NT = NW * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 32, TN = WN / 32;

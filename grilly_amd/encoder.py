@@ -65,10 +65,16 @@ def random_bert_weights(cfg, seed=0, std=0.02):
 
 class BertEncoder:
     """fused=None (default): both LayerNorms of every layer are folded into the GEMMs around them whenever the
-    direct-to-LDS GEMM kernels take the layer's shapes (d_model and d_ff multiples of 64 in bf16, 32 in fp32): the
-    residual stream then travels as raw rows plus row statistics and no LayerNorm pass runs over HBM between the
-    embedding and the final LayerNorm (grl_bert_layer_fwd_fused).  fused=False keeps the seven-launch layer with its
-    two LayerNorm passes (grl_bert_layer_fwd); fused=True insists and raises for shapes the fused layer does not take."""
+    direct-to-LDS GEMM kernels take the layer's shapes (d_model and d_ff multiples of 64 in bf16, 32 in fp32) and the
+    batch has at least FUSED_MIN_ROWS token rows: the residual stream then travels as raw rows plus row statistics and
+    no LayerNorm pass runs over HBM between the embedding and the final LayerNorm (grl_bert_layer_fwd_fused).  Smaller
+    batches run the seven-launch layer with its two LayerNorm passes (grl_bert_layer_fwd): a handful of token rows
+    make a handful of tiles, the plain GEMMs then take 64 x 64 tiles while the fused layer's residual GEMM has none
+    below 128 x 128, and the LayerNorm passes it saves cost next to nothing there (one sentence of 32 tokens in fp32:
+    2.7 against 4.5 ms; level at 4096 rows; the fused layer 4 - 7 % ahead at 8192 - 16384 rows in bf16).  Both weight
+    sets stay resident.  fused=False always takes the seven-launch layer;
+    fused=True always the fused one, and raises for shapes it does not take."""
+    FUSED_MIN_ROWS = 8192
 
     def __init__(self, core, cfg, weights, dtype="fp32", fused=None):
         self.core = core.core if hasattr(core, "core") else core
@@ -95,6 +101,7 @@ class BertEncoder:
         if fused and not eligible:
             raise ValueError(f"the fused layer needs d_model and d_ff to be multiples of {slab} in {dtype}")
         self.fused = eligible if fused is None else bool(fused)
+        self._fused_min_rows = self.FUSED_MIN_ROWS if fused is None else 0
         self.fused_structs = []
         if self.fused:
             # every GEMM that reads a LayerNorm's output gets that norm folded into its weight (once, here):
@@ -131,7 +138,8 @@ class BertEncoder:
         if S > cfg.max_pos:
             raise ValueError(f"sequence length {S} exceeds max_pos {cfg.max_pos}")
         es = 2 if self.code == L.GRL_BF16 else 4
-        wsfn = c.lib.grl_bert_layer_fused_workspace if self.fused else c.lib.grl_bert_layer_workspace
+        self.fused_now = self.fused and B * S >= self._fused_min_rows        # which layer form this batch runs
+        wsfn = c.lib.grl_bert_layer_fused_workspace if self.fused_now else c.lib.grl_bert_layer_workspace
         ws = wsfn(self.code, B, S, cfg.heads, cfg.head_dim, cfg.d_ff)
         self.x = c.alloc(B * S * cfg.d_model * es)
         self.stats = c.alloc(max(B * S, 1) * 8)        # {1/sd, mean/sd} per row of the raw residual stream (fused layers)
@@ -169,7 +177,7 @@ class BertEncoder:
         B, S = self._shape
         cfg, c, lib = self.cfg, self.core, self.core.lib
         mask = self.mask.ptr if self.has_mask else None
-        if self.fused and B * S > 0:
+        if self.fused_now and B * S > 0:
             # raw embedding rows + their statistics; every layer consumes and produces (raw rows, statistics); the last
             # layer's second LayerNorm is the one pass that writes normalised rows
             L.check(lib.grl_embed(c.ctx, self.code, B, S, cfg.d_model, cfg.vocab, self.ids.ptr, self.tok.ptr, self.pos.ptr,
