@@ -1082,14 +1082,19 @@ static inline bool prefer_big_tiles(int64_t n_big, int64_t n_small, int64_t cus,
 
 // Which kernel a 16-byte aligned problem gets: 1 register-staged 256 x 256 tiles, 2 register-staged 128 x 128, 3 direct-to-LDS
 // 256 x 256 (persistent), 4 direct-to-LDS 128 x 128, 5 register-staged 64 x 64.  The direct-to-LDS kernels need K to be a
-// whole number of 128-byte slabs.  Problems of at most sixteen 128 x 128 tiles (single sentences, the README-sized
-// operators) leave most CUs idle and pad M up to 128 rows: 64 x 64 tiles give them four times the workgroups, each with a
-// quarter of the serial K loop.  `dual`: the gated kernels, whose tiles hold half as many output columns.
+// whole number of 128-byte slabs.  Problems that 128 x 128 tiles would spread over a fraction of the CUs (single
+// sentences, small batches, the README-sized operators) take 64 x 64 tiles: four times the workgroups, each with a quarter
+// of the serial K loop, and no rows padded up to 128.  Measured at 32 ... 2048 rows against the BERT-base widths: in fp32,
+// whose matrix rate is the bound, they win up to about four 64 x 64 tiles per CU (32 x 2304 x 768: 56 -> 24 us,
+// 1024 x 768 x 3072: 203 -> 83 us), in bf16 up to one per CU (128 x 768 x 768: 12.8 -> 10.4 us, 1024 x 768 x 3072:
+// 37.9 -> 31.9 us; beyond that the direct-to-LDS kernel is ahead).  `dual`: the gated kernels, whose 128-row tiles hold
+// half as many output columns.
 static inline int gemm_variant(int64_t M, int64_t N, int64_t K, size_t elem_size, bool dual, int64_t cus) {
     const int64_t bke = 128 / (int64_t)elem_size;
     const int64_t big_m = (M + 255) / 256, big_n = (N + (dual ? 127 : 255)) / (dual ? 128 : 256);
     const int64_t sm = (M + 127) / 128, sn = (N + (dual ? 63 : 127)) / (dual ? 64 : 128);
-    if (sm * sn <= 16) return 5;
+    const int64_t t64 = ((M + 63) / 64) * ((N + 63) / 64);
+    if (t64 <= cus * (elem_size == 4 ? 4 : 1)) return 5;
     const bool slabs = K % bke == 0;
     const bool big = prefer_big_tiles(big_m * big_n, sm * sn, cus, elem_size);
     return slabs ? (big ? 3 : 4) : (big ? 1 : 2);

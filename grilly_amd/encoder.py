@@ -71,7 +71,7 @@ class BertEncoder:
     batches run the seven-launch layer with its two LayerNorm passes (grl_bert_layer_fwd): a handful of token rows
     make a handful of tiles, the plain GEMMs then take 64 x 64 tiles while the fused layer's residual GEMM has none
     below 128 x 128, and the LayerNorm passes it saves cost next to nothing there (one sentence of 32 tokens in fp32:
-    2.7 against 4.5 ms; level at 4096 rows; the fused layer 4 - 7 % ahead at 8192 - 16384 rows in bf16).  Both weight
+    1.9 against 4.5 ms; level at 4096 rows; the fused layer 4 - 7 % ahead at 8192 - 16384 rows in bf16).  Both weight
     sets stay resident.  fused=False always takes the seven-launch layer;
     fused=True always the fused one, and raises for shapes it does not take."""
     FUSED_MIN_ROWS = 8192

@@ -111,6 +111,9 @@ def test_gemm_tile_choice_for_the_benchmark_shapes():
     assert plan(L.GRL_F32, 16384, 1152, 384) == 4 and plan(L.GRL_F32, 16384, 1536, 384) == 4
     assert plan(L.GRL_F32, 16384, 384, 384) == 4                             # below 192 big tiles: always small
     assert plan(L.GRL_BF16, 8192, 2304, 768) == 4 and plan(L.GRL_BF16, 32768, 3072, 768) == 3
-    assert plan(L.GRL_F32, 32, 128, 384) == 5 and plan(L.GRL_BF16, 128, 2304, 768) == 4 and plan(L.GRL_BF16, 128, 768, 768) == 5
-    assert plan(L.GRL_F32, 4096, 4096, 1000) == 1 and plan(L.GRL_F32, 1024, 1024, 1000) == 2      # K tail: register-staged
+    # small batches: 64 x 64 tiles up to one per CU in bf16, four per CU in fp32
+    assert plan(L.GRL_F32, 32, 128, 384) == 5 and plan(L.GRL_BF16, 128, 2304, 768) == 5 and plan(L.GRL_BF16, 128, 768, 768) == 5
+    assert plan(L.GRL_BF16, 1024, 768, 3072) == 5 and plan(L.GRL_BF16, 1024, 2304, 768) == 4
+    assert plan(L.GRL_F32, 1024, 3072, 768) == 5 and plan(L.GRL_F32, 2048, 3072, 768) == 4
+    assert plan(L.GRL_F32, 4096, 4096, 1000) == 1 and plan(L.GRL_F32, 4096, 2048, 1000) == 2      # K tail: register-staged
     assert plan(L.GRL_F32, 0, 8, 8) == L.ERR_ARG and plan(7, 8, 8, 8) == L.ERR_ARG and plan(L.GRL_F32, 8, 8, 8, cus=0) == L.ERR_ARG

@@ -180,6 +180,8 @@ def test_randomized_shapes_over_every_kernel_variant(backend):
                 N += 256
             if kkind == 2:
                 M //= 8                        # the one-thread-per-output kernel is slow: keep it small
+        elif case % 7 in (1, 4) and kkind != 2:   # too many 64 x 64 tiles for one pass, too few 256 x 256 ones: the 128 x 128 kernels
+            M = int(rng.integers(1100, 2600)); N = int(rng.integers(1100, 2600))
         else:
             M = int(rng.integers(1, 900)); N = int(rng.integers(1, 900))
         epi = epis[int(rng.integers(0, len(epis)))]
@@ -204,7 +206,7 @@ def test_randomized_shapes_over_every_kernel_variant(backend):
     assert worst["fp32"] < TOL_F32 and worst["bf16"] < TOL_BF16
 
 
-# (M, K, N) either side of the tile choice: at most sixteen 128 x 128 tiles (64 x 64 tiles, also with a K tail and with
+# (M, K, N) either side of the tile choice: few enough 64 x 64 tiles for one pass over the CUs (also with a K tail and with
 # ragged edges), 320 and 192 big tiles whose last pass would stay mostly empty (128 x 128 tiles instead), 256 and 512 big
 # tiles that fill their passes (256 x 256 tiles)
 TILE_CHOICE = [(32, 384, 128), (100, 72, 200), (500, 256, 460), (16384, 384, 1152), (4096, 768, 3072), (8192, 768, 2048), (8192, 512, 4096)]
