@@ -490,6 +490,25 @@ def small_configs(backend, reps, check=True):
     return r0, r1
 
 
+def small_batch_latency(backend, weights, cfg, reps):
+    """The benchmark's encoder at the other end of the batch range: one sentence and eight sentences of 128 tokens, both
+    storage types, median milliseconds per forward (device-resident, no host synchronisation between forwards).  The
+    launcher's small-tile choice and the encoder's choice of layer form by batch size are what these figures show."""
+    from grilly_amd import BertEncoder
+    rng = np.random.default_rng(11)
+    out = {"workload": "BERT-base-shaped encoder forward at batch 1 and batch 8, seq 128, no padding, embeddings + layers + mean pooling"}
+    for dtype in ("bf16", "fp32"):
+        enc = BertEncoder(backend, cfg, weights, dtype=dtype)
+        for B in (1, 8):
+            ids = rng.integers(0, cfg.vocab, (B, 128))
+            enc.set_inputs(ids, None)
+            t = lap_times(backend.core, lambda: enc.launch(pool=True), reps, warm=5)
+            out[f"{dtype}_batch{B}_median_ms"] = round(median(t), 4)
+        enc.release_activations()
+        del enc
+    return out
+
+
 def mfma_ceiling(backend, iters=20000):
     """What the matrix cores deliver under the board's power limit with nothing else going on: a register-resident loop
     of MFMAs (grl_mfma_probe: eight waves per CU, the GEMM's 128 x 64 wave tile, no memory access in the loop) for both
@@ -631,7 +650,8 @@ def main():
         return
     if a.mode == "small":
         r0, r1 = small_configs(backend, a.kernel_reps, check=not a.no_cpu_baseline)
-        print(json.dumps({"mode": "small", "readme_ops": r0, "minilm_forward": r1}))
+        lat = small_batch_latency(backend, random_bert_weights(cfg, seed=seed), cfg, a.kernel_reps)
+        print(json.dumps({"mode": "small", "readme_ops": r0, "minilm_forward": r1, "small_batch_latency": lat}))
         backend.cleanup()
         return
     if a.mode == "gemm_shapes":
@@ -797,6 +817,7 @@ def main():
             backend.core.lib.grl_pool_trim(backend.core.ctx)
         r0, r1 = small_configs(backend, 20, check=not a.no_cpu_baseline)
         extra["readme_ops"], extra["minilm_forward"] = r0, r1
+        extra["small_batch_latency"] = small_batch_latency(backend, weights, cfg, 20)
         extra["mfma_ceiling"] = mfma_ceiling(backend)
         out["extra"] = extra
     if not a.no_cpu_baseline:
