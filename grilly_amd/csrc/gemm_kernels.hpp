@@ -53,6 +53,10 @@ struct GemmArgs {
     const float* res_gamma;  // (N)
     const float* res_beta;   // (N)
     float* part_out;         // (tiles_n, M, 2): {sum, sum of squares} of each output row's columns in that tile
+    // split K (register-staged 64 x 64 kernel, template flag SPLITK): workgroup (x, y) multiplies the y-th share of the K
+    // slabs of tile x and writes its raw fp32 sums to kpart[y]; gemm_splitk_finish_kernel adds the shares and runs the epilogue
+    int ksplit;              // number of shares (grid.y)
+    float* kpart;            // (ksplit, M, N) fp32
 };
 
 // Epilogue template codes.  NONE / GELU / SILU are compiled in (the encoder's hot shapes); EPI_RT picks
@@ -335,8 +339,9 @@ __device__ __forceinline__ void epilogue_direct(f32x16 (&acc)[TM][TN], const Gem
 
 // BN counts LDS rows of the weight tile; with DUAL it is 2x the output-column count of the
 // tile (first half gate rows, second half up rows).
-template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL, bool LN = false>
+template <typename T, typename OutT, int BM, int BN, int WGM, int WGN, int EPI, bool DUAL, bool LN = false, bool SPLITK = false>
 __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
+    static_assert(!SPLITK || (!DUAL && !LN), "split K: plain single-weight products only (the epilogue runs in the finishing kernel)");
     constexpr int NT = WGM * WGN * 64;
     constexpr int EPC = 16 / (int)sizeof(T);     // elements per 16-byte chunk
     constexpr int BK = 8 * EPC;                  // elements per 128-byte slab row
@@ -440,11 +445,17 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
     }
 
     const int KT = (p.K + BK - 1) / BK;
-    load_slab(0);
-    stash_slab(0);
+    int kt0 = 0, kt1 = KT;
+    if constexpr (SPLITK) {                       // this workgroup's share of the slabs (the host leaves no share empty)
+        const int per = (KT + p.ksplit - 1) / p.ksplit;
+        kt0 = (int)blockIdx.y * per;
+        kt1 = kt0 + per < KT ? kt0 + per : KT;
+    }
+    load_slab(kt0);
+    stash_slab(kt0);
     __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const bool more = kt + 1 < KT;
+    for (int kt = kt0; kt < kt1; ++kt) {
+        const bool more = kt + 1 < kt1;
         if (more) load_slab(kt + 1);
         const char* s = lds + (kt & 1) * STAGE;
 #pragma unroll
@@ -465,7 +476,43 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_nt_kernel(GemmArgs p) {
         __syncthreads();
     }
 
-    epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL, LN>(acc, p, m0, n0, wm, wn, li, lg);
+    if constexpr (SPLITK) {
+        GemmArgs q = p;                            // raw sums of this share, fp32, no bias / activation / residual
+        q.C = p.kpart + (int64_t)blockIdx.y * p.M * p.N;
+        q.bias = nullptr;
+        epilogue_direct<float, TM, TN, TNO, WM, WNO, EPI_NONE, false, false>(acc, q, m0, n0, wm, wn, li, lg);
+    } else {
+        epilogue_direct<OutT, TM, TN, TNO, WM, WNO, EPI, DUAL, LN>(acc, p, m0, n0, wm, wn, li, lg);
+    }
+}
+
+// Second half of a split-K product: C = epilogue(sum of the shares + bias) (+ residual), four adjacent outputs per thread
+// (N is a multiple of 4 here).  The shares are added in ascending order, so the result does not depend on scheduling.
+template <typename OutT, int EPI>
+__global__ __launch_bounds__(256) void gemm_splitk_finish_kernel(GemmArgs p) {
+    const int64_t quads = (int64_t)p.M * p.N / 4;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= quads) return;
+    const int64_t o = i * 4;
+    const int n = (int)(o % p.N);
+    f32x4 acc = *(const f32x4*)(p.kpart + o);
+    for (int sidx = 1; sidx < p.ksplit; ++sidx) {
+        const f32x4 t = *(const f32x4*)(p.kpart + (int64_t)sidx * p.M * p.N + o);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += t[e];
+    }
+    float v[4] = {acc[0], acc[1], acc[2], acc[3]};
+    if (p.bias) {
+        const f32x4 bv = *(const f32x4*)(p.bias + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += bv[e];
+    }
+    if constexpr (EPI == EPI_GELU) gelu_fast4(v);
+    else
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = epi_apply<EPI>(v[e], p);
+    if constexpr (EPI == EPI_RES) add4<OutT>((const OutT*)p.residual + o, v);
+    store4<OutT>((OutT*)p.C + o, v[0], v[1], v[2], v[3]);
 }
 
 // =====================================================================================
@@ -1129,10 +1176,35 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
     int variant = gemm_variant(a.M, a.N, a.K, sizeof(T), DUAL, cus);
     if (forced >= 1 && forced <= 5 && (slabs || forced <= 2 || forced == 5)) variant = forced;
     switch (variant) {
-        case 5:
+        case 5: {
             a.tiles_m = (int)tm; a.tiles_n = (int)tn;
+            // Few tiles and a long K (one sentence through a feed-forward block: 24 tiles, 96 slabs in fp32) leave most CUs
+            // idle behind a serial K loop whose every slab costs a memory round trip: the slabs are shared out over up to
+            // 8 workgroups per tile (16 slabs or more, at least 4 per share, at most about one workgroup per CU in all), which write raw
+            // fp32 sums to a pool buffer, and a small second kernel adds them and runs the epilogue.  GRL_GEMM_SPLITK=0
+            // switches it off, for tuning runs.
+            static const int splitk_env = [] { const char* e = getenv("GRL_GEMM_SPLITK"); return e ? atoi(e) : -1; }();
+            int ks = 1;
+            if constexpr (!DUAL && !LN && (EPI == EPI_NONE || EPI == EPI_GELU || EPI == EPI_SILU || EPI == EPI_RT || EPI == EPI_RES)) {
+                const int64_t KT = (a.K + bke - 1) / bke, t64 = tm * tn;
+                if (splitk_env != 0 && a.N % 4 == 0 && KT >= 16 && 2 * t64 <= cus) {
+                    ks = (int)std::min<int64_t>(std::min<int64_t>(8, cus / t64), KT / 4);
+                    while (ks > 1 && ((KT + ks - 1) / ks) * (ks - 1) >= KT) --ks;      // no empty share
+                }
+                if (ks > 1) {
+                    a.ksplit = ks;
+                    a.kpart = (float*)grl_malloc(c, (size_t)ks * a.M * a.N * sizeof(float));
+                    if (!a.kpart) return GRL_ERR_OOM;
+                    hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 64, 64, 2, 2, EPI, false, false, true>), dim3((unsigned)(tm * tn), (unsigned)ks), dim3(256), 0, c->stream, a);
+                    const int64_t quads = (int64_t)a.M * a.N / 4;
+                    hipLaunchKernelGGL((gemm_splitk_finish_kernel<OutT, EPI>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, c->stream, a);
+                    grl_free(c, a.kpart);          // back to the pool: later users are ordered behind these launches on the stream
+                    break;
+                }
+            }
             hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 64, (DUAL ? 128 : 64), 2, 2, EPI, DUAL, LN>), dim3((unsigned)(tm * tn)), dim3(256), 0, c->stream, a);
             break;
+        }
         case 1:
             a.tiles_m = (int)big_m; a.tiles_n = (int)big_n;
             hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, 256, 256, 2, 2, EPI, DUAL, LN>), dim3((unsigned)(big_m * big_n)), dim3(256), 0, c->stream, a);

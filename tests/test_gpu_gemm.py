@@ -360,3 +360,42 @@ def test_gemm_nt_c_abi_randomized(backend):
         assert (got[:lead] == 7.0).all() and (got[lead + M * N:] == 7.0).all(), info
         if case and case % 50 == 0:
             print("sweep case", case, flush=True)
+
+
+# (M, K, N): few 64 x 64 tiles and at least sixteen K slabs: the launcher shares the slabs of a tile out over several
+# workgroups and a second kernel adds the shares and runs the epilogue.  One sentence through the feed-forward block's
+# second GEMM; a single row; ragged M and N (N a multiple of 4); a K tail in the last share; fp32 K = 512 is exactly 16 slabs
+# (bf16: 8, not split).
+SPLIT_K = [(32, 3072, 768), (128, 3072, 768), (1, 4096, 64), (100, 1024, 200), (70, 1000, 36), (50, 512, 40)]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("epi", ["none", "gelu", "silu", "relu", "roswish", "res"])
+@pytest.mark.parametrize("M,K,N", SPLIT_K)
+def test_split_k_products(backend, dtype, epi, M, K, N):
+    rng = np.random.default_rng(M + 3 * K + 7 * N + len(epi))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    W = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    if dtype == "bf16":
+        x, W = O.bf16_round(x), O.bf16_round(W)
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    f = backend.fnn
+    for bias in (b, None):
+        if epi == "res":
+            r = (2.0 * rng.standard_normal((M, N))).astype(np.float32)
+            r = O.bf16_round(r) if dtype == "bf16" else r
+            y = f.fused_linear_residual(x, W, bias, r, dtype=dtype)
+            ref = O.truth_linear(x, W, bias) + r.astype(np.float64)
+        else:
+            y = {"none": lambda: f.linear(x, W, bias, dtype=dtype),
+                 "gelu": lambda: f.fused_linear_gelu(x, W, bias, dtype=dtype),
+                 "silu": lambda: f.fused_linear_silu(x, W, bias, dtype=dtype),
+                 "relu": lambda: f.fused_linear_relu(x, W, bias, dtype=dtype),
+                 "roswish": lambda: f.fused_linear_roswish(x, W, bias, alpha=0.7, beta=1.3, dtype=dtype)}[epi]()
+            ref = O.truth_linear(x, W, bias, epi, 0.7, 1.3)
+        assert y.shape == (M, N) and np.isfinite(y).all()
+        assert O.max_rel(y, ref) < tol, (epi, bias is None)
+    # the same call twice gives the same bits (the shares are added in a fixed order)
+    y1, y2 = f.linear(x, W, b, dtype=dtype), f.linear(x, W, b, dtype=dtype)
+    np.testing.assert_array_equal(y1, y2)
