@@ -54,9 +54,11 @@ __global__ __launch_bounds__(256) void bias_residual_kernel(OutT* C, const OutT*
     elem<OutT>::st(C + i, elem<OutT>::ld(R + i) + (bias ? bias[i % N] : 0.f));
 }
 
-extern "C" int grl_gemm_nt_act(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
-                               const void* A, const void* W, const float* bias, void* C, int epilogue,
-                               float alpha, float beta) {
+// may_allocate == false: for the entry point that promises to allocate nothing (the launcher then leaves the K loop whole
+// instead of sharing it out through a pool buffer)
+static int gemm_nt_act_impl(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                            const void* A, const void* W, const float* bias, void* C, int epilogue,
+                            float alpha, float beta, bool may_allocate) {
     GRL_REQUIRE(c, GRL_ERR_ARG, "grl_gemm_nt: null context");
     GRL_REQUIRE(grl_valid_dtype(in_dtype) && grl_valid_dtype(out_dtype), GRL_ERR_ARG, "grl_gemm_nt: bad dtype");
     GRL_REQUIRE(epilogue >= GRL_EPI_NONE && epilogue <= GRL_EPI_ROSWISH, GRL_ERR_ARG, "grl_gemm_nt: bad epilogue %d", epilogue);
@@ -68,6 +70,7 @@ extern "C" int grl_gemm_nt_act(grl_ctx* c, int in_dtype, int out_dtype, int64_t 
     a.A = A; a.W = W; a.bias = bias; a.C = C;
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     a.act = epilogue; a.alpha = alpha; a.beta = beta;
+    a.no_alloc = !may_allocate;
     const int epi = epilogue <= GRL_EPI_SILU ? epilogue : EPI_RT;
     if (K == 0) {
         int64_t total = M * N;
@@ -78,6 +81,12 @@ extern "C" int grl_gemm_nt_act(grl_ctx* c, int in_dtype, int out_dtype, int64_t 
         return GRL_OK;
     }
     return dispatch_types(c, a, in_dtype, out_dtype, epi);
+}
+
+extern "C" int grl_gemm_nt_act(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
+                               const void* A, const void* W, const float* bias, void* C, int epilogue,
+                               float alpha, float beta) {
+    return gemm_nt_act_impl(c, in_dtype, out_dtype, M, N, K, A, W, bias, C, epilogue, alpha, beta, true);
 }
 
 extern "C" int grl_gemm_nt_res(grl_ctx* c, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
@@ -342,7 +351,7 @@ extern "C" int grl_gemm_nn_noalloc(grl_ctx* c, int in_dtype, int out_dtype, int6
     int rc = check_dims("grl_gemm_nn_noalloc", M, N, K);
     if (rc) return rc;
     if (M == 0 || N == 0) return GRL_OK;
-    if (K == 0) return grl_gemm_nt(c, in_dtype, out_dtype, M, N, 0, A, B, nullptr, C, GRL_EPI_NONE);
+    if (K == 0) return gemm_nt_act_impl(c, in_dtype, out_dtype, M, N, 0, A, B, nullptr, C, GRL_EPI_NONE, 1.0f, 1.0f, false);
     GRL_REQUIRE(A && B && C, GRL_ERR_ARG, "grl_gemm_nn_noalloc: null argument");
     const int64_t need = K * N * (int64_t)grl_dtype_size(in_dtype);
     GRL_REQUIRE(need <= (int64_t)GRL_NN_SCRATCH_BYTES, GRL_ERR_SHAPE,
@@ -357,6 +366,6 @@ extern "C" int grl_gemm_nn_noalloc(grl_ctx* c, int in_dtype, int out_dtype, int6
     // thread A's transpose and A's GEMM (A would then multiply by B's matrix).
     std::lock_guard<std::mutex> pair(g_scratch_pair_mu);
     rc = grl_transpose2d(c, in_dtype, K, N, B, ws);   // (K,N) -> (N,K)
-    if (!rc) rc = grl_gemm_nt(c, in_dtype, out_dtype, M, N, K, A, ws, nullptr, C, GRL_EPI_NONE);
+    if (!rc) rc = gemm_nt_act_impl(c, in_dtype, out_dtype, M, N, K, A, ws, nullptr, C, GRL_EPI_NONE, 1.0f, 1.0f, false);
     return rc;
 }

@@ -57,6 +57,7 @@ struct GemmArgs {
     // slabs of tile x and writes its raw fp32 sums to kpart[y]; gemm_splitk_finish_kernel adds the shares and runs the epilogue
     int ksplit;              // number of shares (grid.y)
     float* kpart;            // (ksplit, M, N) fp32
+    bool no_alloc;           // host side: the caller must not touch the buffer pool (split K takes its buffer there): no split
 };
 
 // Epilogue template codes.  NONE / GELU / SILU are compiled in (the encoder's hot shapes); EPI_RT picks
@@ -1180,16 +1181,17 @@ static int launch_gemm(grl_ctx* c, GemmArgs& a) {
             a.tiles_m = (int)tm; a.tiles_n = (int)tn;
             // Few tiles and a long K (one sentence through a feed-forward block: 24 tiles, 96 slabs in fp32) leave most CUs
             // idle behind a serial K loop whose every slab costs a memory round trip: the slabs are shared out over up to
-            // 8 workgroups per tile (16 slabs or more, at least 4 per share, at most about one workgroup per CU in all), which write raw
+            // 8 workgroups per tile (16 slabs or more, at least 4 per share, at most about two workgroups per CU in all), which write raw
             // fp32 sums to a pool buffer, and a small second kernel adds them and runs the epilogue.  GRL_GEMM_SPLITK=0
             // switches it off, for tuning runs.
             static const int splitk_env = [] { const char* e = getenv("GRL_GEMM_SPLITK"); return e ? atoi(e) : -1; }();
             int ks = 1;
             if constexpr (!DUAL && !LN && (EPI == EPI_NONE || EPI == EPI_GELU || EPI == EPI_SILU || EPI == EPI_RT || EPI == EPI_RES)) {
                 const int64_t KT = (a.K + bke - 1) / bke, t64 = tm * tn;
-                if (splitk_env != 0 && a.N % 4 == 0 && KT >= 16 && 2 * t64 <= cus) {
-                    ks = (int)std::min<int64_t>(std::min<int64_t>(8, cus / t64), KT / 4);
+                if (splitk_env != 0 && !a.no_alloc && a.N % 4 == 0 && KT >= 16 && t64 <= cus) {
+                    ks = (int)std::min<int64_t>(std::min<int64_t>(8, 2 * cus / t64), KT / 4);
                     while (ks > 1 && ((KT + ks - 1) / ks) * (ks - 1) >= KT) --ks;      // no empty share
+                    if (ks == 2 && KT < 48) ks = 1;                                      // two short halves: the second launch costs more
                 }
                 if (ks > 1) {
                     a.ksplit = ks;

@@ -168,7 +168,9 @@ int grl_gemm_nn(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N,
  * GRL_ERR_SHAPE.  All calls on one GPU share the array.  Host threads that call it on ONE context are safe: a lock
  * keeps each call's two launches (transpose into the array, GEMM out of it) adjacent on the context's stream,
  * which then orders the calls.  Calls on two contexts of the same GPU run on two streams and race on the
- * array: the caller must not overlap them. */
+ * array: the caller must not overlap them.  Small products with a long K, whose K loop grl_gemm_nn shares out over
+ * several workgroups through a pool buffer, keep their K loop whole here: results agree with grl_gemm_nn to the
+ * last bits of the sums, not bit for bit. */
 int grl_gemm_nn_noalloc(grl_ctx* ctx, int in_dtype, int out_dtype, int64_t M, int64_t N, int64_t K,
                         const void* A, const void* B, void* C);
 int64_t grl_gemm_nn_noalloc_max_bytes(void);

@@ -1,6 +1,8 @@
 """The allocation-free variant of gemm(A,B): grl_gemm_nn_noalloc keeps the transposed copy of B in a static
-device array instead of a pool buffer.  Called through the C ABI and checked against grl_gemm_nn (same
-kernels, so bit-exact) and the float64 oracle, on two calls in a row, the second with a smaller input (the
+device array instead of a pool buffer.  Called through the C ABI and checked against grl_gemm_nn (equal to the last
+bits, not bit for bit: for small products grl_gemm_nn shares the K loop out over several workgroups through a pool
+buffer, which the allocation-free call must not touch, so the two add their partial sums in another grouping) and the
+float64 oracle, on two calls in a row, the second with a smaller input (the
 array still holds the first call's image), for both storage types; the size limit is an error, and the
 caching pool sees no request during the calls."""
 import numpy as np
@@ -47,7 +49,7 @@ def test_gemm_nn_noalloc_matches_gemm_nn(backend, dtype):
             A, B = O.bf16_round(A), O.bf16_round(B)
         got = _run(c, "noalloc", code, A, B)
         want = _run(c, "pool", code, A, B)
-        np.testing.assert_array_equal(got, want)
+        assert O.max_rel(got, want) < (1e-5 if dtype == "fp32" else 8e-3)
         assert O.max_rel(got, O.truth_gemm(A, B)) < tol
 
 
