@@ -168,7 +168,8 @@ def test_randomized_shapes_over_every_kernel_variant(backend):
         chunk = 8 if dtype == "bf16" else 4
         kkind = case % 3                       # 0: whole slabs, 1: 16-byte rows with a K tail, 2: unaligned rows
         if kkind == 0:
-            K = slab * int(rng.integers(1, 9))
+            # every fifth of these with a long K: small products then share their K loop out over several workgroups
+            K = slab * (int(rng.integers(16, 70)) if case % 5 == 0 else int(rng.integers(1, 9)))
         elif kkind == 1:
             K = chunk * int(rng.integers(1, 60))
             K += chunk if K % slab == 0 else 0
